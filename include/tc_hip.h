@@ -1,0 +1,134 @@
+/* tc_hip — C ABI of the Tensor Comprehensions HIP backend (library libtc_hip.so).
+ *
+ * The reference exposes this path as C++ templates over at::Tensor / DLTensor
+ * (tc::aten::compile / prepareOutputs / run / profile / uncheckedRun in tc/aten/aten_compiler.h,
+ * tc::compile / tc::inferOutputTensorInfo in tc/core/compiler.h, TcExecutor in
+ * tc/core/tc_executor.h, ATenAutotuner in tc/aten/aten_autotuner.h).  Each entry point below
+ * is the plain-C form of one of those; a binding in any language needs nothing else.
+ *
+ * Tensors cross the boundary as DLPack-layout structs (DLTensor / DLConstTensor, the types the
+ * reference's core API takes, tc/core/tensor.h:36-50).  Data pointers are device pointers and
+ * are only borrowed for the duration of a call.  Mapping options cross as text
+ * ("preset;key=value;...", keys named like the reference's fluent setters) or as a serialized
+ * options message.  Every function returns 0 on success; on failure tc_last_error() returns the
+ * message of the C++ exception that was caught on the calling thread (a lang::ErrorReport text
+ * with the highlighted source for TC errors).
+ */
+#ifndef TC_HIP_H
+#define TC_HIP_H
+#include <stddef.h>
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#ifndef TC_DLPACK_TYPES_DEFINED
+#define TC_DLPACK_TYPES_DEFINED
+typedef struct { int32_t device_type; int32_t device_id; } tc_dl_context;
+typedef struct { uint8_t code; uint8_t bits; uint16_t lanes; } tc_dl_datatype; /* code: 0 int, 1 uint, 2 float */
+typedef struct {
+  void* data;
+  tc_dl_context ctx;
+  int32_t ndim;
+  tc_dl_datatype dtype;
+  int64_t* shape;
+  int64_t* strides; /* NULL = contiguous */
+  uint64_t byte_offset;
+} tc_dl_tensor;
+#endif
+
+#define TC_MAX_RANK 8
+typedef struct {
+  tc_dl_datatype dtype;
+  int32_t ndim;
+  int64_t shape[TC_MAX_RANK];
+  int64_t strides[TC_MAX_RANK];
+} tc_tensor_info;
+
+typedef struct tc_executor tc_executor_t;
+
+const char* tc_last_error(void);
+void tc_free(void* p); /* frees strings returned through char** parameters */
+
+/* tc::inferOutputTensorInfo (tc/core/compiler.h:88-92; tc::aten::inferOutputTensorInfo,
+ * tc/aten/aten_compiler.h:35-38).  Writes up to `capacity` entries, *count = number of outputs. */
+int tc_infer_output_info(
+    const char* tc, const char* entry_point,
+    const tc_dl_tensor* const* inputs, int num_inputs,
+    tc_tensor_info* outputs, int capacity, int* count);
+
+/* tc::compile<HipBackend> (tc/core/compiler.h:71-78; tc::aten::compile, aten_compiler.h:56-62).
+ * `options` is option text; see tc_options_* below. */
+int tc_compile(
+    const char* tc, const char* entry_point,
+    const tc_dl_tensor* const* inputs, int num_inputs,
+    const char* options, tc_executor_t** executor);
+/* same with a serialized options message (HipMappingOptions::toProtobufSerializedString) */
+int tc_compile_serialized_options(
+    const char* tc, const char* entry_point,
+    const tc_dl_tensor* const* inputs, int num_inputs,
+    const void* options, size_t options_size, tc_executor_t** executor);
+
+/* TcExecutor::run (tc/core/tc_executor.h:89-92; tc::aten::run, aten_compiler.h:69-73):
+ * checks count, rank, dtype and shape, launches on `stream` (a hipStream_t or NULL), does not
+ * synchronise. */
+int tc_executor_run(
+    const tc_executor_t* executor,
+    const tc_dl_tensor* const* inputs, int num_inputs,
+    const tc_dl_tensor* const* outputs, int num_outputs, void* stream);
+/* TcExecutor::uncheckedRun (tc_executor.h:109-112; tc::aten::uncheckedRun, aten_compiler.h:88-92):
+ * raw device pointers, no checks. */
+int tc_executor_unchecked_run(
+    const tc_executor_t* executor,
+    const void* const* inputs, int num_inputs, void* const* outputs, int num_outputs, void* stream);
+/* TcExecutor::profile (tc_executor.h:94-98; tc::aten::profile, aten_compiler.h:79-83):
+ * like run, bracketed by device events; synchronises.  Times in microseconds (fractional). */
+int tc_executor_profile(
+    const tc_executor_t* executor,
+    const tc_dl_tensor* const* inputs, int num_inputs,
+    const tc_dl_tensor* const* outputs, int num_outputs, void* stream,
+    double* kernel_us, double* cpu_overhead_us);
+
+/* TcExecutor::compiledSource, CudaTcExecutor::grid()/block() (cuda_tc_executor.h:52-60) */
+const char* tc_executor_source(const tc_executor_t* executor);
+int tc_executor_num_kernels(const tc_executor_t* executor);
+int tc_executor_launch_bounds(const tc_executor_t* executor, int kernel, unsigned grid[3], unsigned block[3]);
+const char* tc_executor_kernel_name(const tc_executor_t* executor, int kernel);
+int64_t tc_executor_lds_bytes(const tc_executor_t* executor, int kernel);
+/* CudaTcExecutor::clearRuntimeCompiledFunction (cuda_tc_executor.h:47-50) */
+int tc_executor_clear(tc_executor_t* executor);
+void tc_executor_destroy(tc_executor_t* executor);
+
+/* Mapping options (CudaMappingOptions presets, tc/core/cuda/cuda_mapping_options.cc:327-384).
+ * Presets: naive, single_thread, pointwise, mlp, conv, group_conv, unmapped. */
+int tc_options_normalize(const char* options, char** text);          /* full "key=value;..." form */
+int tc_options_to_serialized(const char* options, void** bytes, size_t* size);
+int tc_options_from_serialized(const void* bytes, size_t size, char** text);
+int tc_options_to_cpp(const char* options, char** cpp);              /* chainable C++ source */
+
+/* The mapper alone: HIP source and launch bounds for the given shapes, nothing compiled or
+ * loaded (what CudaBackend::compileWithTcMapper returns, cuda_tc_executor.cc:71-109). */
+int tc_map(
+    const char* tc, const char* entry_point,
+    const tc_dl_tensor* const* inputs, int num_inputs, const char* options,
+    char** source, int* num_kernels, unsigned* grids /* [8][3] */, unsigned* blocks /* [8][3] */);
+
+/* Front-end dumps in the format of the reference's golden files (tc/lang/test_expected/).
+ * what: "lexer", "exp", "stmt", "function", "sema", "sema_env", "canonical" */
+int tc_lang_dump(const char* text, const char* what, char** out);
+
+/* ATenAutotuner<HipBackend, GeneticSearch>::tune (tc/aten/aten_autotuner.h:79-84,
+ * tc/autotuner/autotuner.h:153-161).  Tensors must live on the current device; outputs are
+ * scratch the candidates write into.  `settings` is "key=value;..." over generations, pop_size,
+ * crossover_rate, mutation_rate, number_elites, threads, seed, cache_file, top_k, fix_* ; NULL = flag
+ * defaults.  Returns the best option text in *best (top_k best, newline separated). */
+int tc_autotune(
+    const char* tc, const char* entry_point,
+    const tc_dl_tensor* const* inputs, int num_inputs,
+    const tc_dl_tensor* const* outputs, int num_outputs,
+    const char* base_options, const char* settings, char** best);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TC_HIP_H */

@@ -1,0 +1,132 @@
+// Device-side helper library prepended to every generated kernel, as source text for hipRTC.
+//
+// Role of tc/core/cuda/cuda_libraries.h:33-285 in the reference, rewritten for 64-lane
+// wavefronts: floor-division helpers for index arithmetic, reduction operators with their
+// identities, and a block reduction "along x" that replaces the CUB-based CubReduceAlongX
+// (:214-285).  The reduction is hand-written: DPP butterflies inside 16-lane rows, lane reads
+// across rows, LDS across wavefronts.
+#pragma once
+#include <string>
+
+namespace tc {
+namespace hip {
+
+constexpr const char* kDeviceTypes = R"HIP(
+typedef long long int64;
+typedef unsigned long long uint64;
+)HIP";
+
+// Halide-style integer semantics for / and % in subscripts (round toward -infinity),
+// cf. floord in tc/core/cuda/cuda_libraries.h:61-66.
+constexpr const char* kDeviceIndexHelpers = R"HIP(
+namespace __tc {
+template <typename T> __device__ __forceinline__ T floordiv(T n, T d) {
+  T q = n / d;
+  return ((n % d != 0) && ((n < 0) != (d < 0))) ? q - 1 : q;
+}
+template <typename T> __device__ __forceinline__ T floormod(T n, T d) { return n - floordiv(n, d) * d; }
+template <typename T> __device__ __forceinline__ T tmin(T a, T b) { return a < b ? a : b; }
+template <typename T> __device__ __forceinline__ T tmax(T a, T b) { return a > b ? a : b; }
+__device__ __forceinline__ float tmin(float a, float b) { return fminf(a, b); }
+__device__ __forceinline__ float tmax(float a, float b) { return fmaxf(a, b); }
+__device__ __forceinline__ double tmin(double a, double b) { return fmin(a, b); }
+__device__ __forceinline__ double tmax(double a, double b) { return fmax(a, b); }
+} // namespace __tc
+)HIP";
+
+// Wave64 reduction library.
+//   __tc::OpSum/OpProd/OpMin/OpMax<T>      operator + identity
+//   __tc::waveAllReduce<Op, WIDTH>(v)      all-reduce over aligned groups of WIDTH lanes
+//                                          (WIDTH a power of two, 2..64)
+//   __tc::blockAllReduceX<Op, BX, BY, BZ>(v, scratch)
+//        reduces v over threadIdx.x separately for every (threadIdx.y, threadIdx.z) and
+//        returns the result to every thread of the row.  `scratch` is LDS of
+//        __tc::reduceScratchElems(BX, BY, BZ) elements; the call contains block barriers, so
+//        every thread of the block must reach it.
+constexpr const char* kDeviceReductions = R"HIP(
+namespace __tc {
+template <typename T> struct OpSum  { static __device__ __forceinline__ T apply(T a, T b) { return a + b; } };
+template <typename T> struct OpProd { static __device__ __forceinline__ T apply(T a, T b) { return a * b; } };
+template <typename T> struct OpMin  { static __device__ __forceinline__ T apply(T a, T b) { return tmin(a, b); } };
+template <typename T> struct OpMax  { static __device__ __forceinline__ T apply(T a, T b) { return tmax(a, b); } };
+
+// lane exchange through the DPP network (no LDS traffic); CTRL is a GFX9 dpp_ctrl code
+template <int CTRL> __device__ __forceinline__ int dppMov(int v) {
+  return __builtin_amdgcn_update_dpp(v, v, CTRL, 0xf, 0xf, false);
+}
+template <int CTRL> __device__ __forceinline__ float dppMov(float v) {
+  return __int_as_float(dppMov<CTRL>(__float_as_int(v)));
+}
+template <int CTRL> __device__ __forceinline__ unsigned dppMov(unsigned v) { return (unsigned)dppMov<CTRL>((int)v); }
+template <int CTRL> __device__ __forceinline__ double dppMov(double v) {
+  long long b = __double_as_longlong(v);
+  int lo = dppMov<CTRL>((int)(b & 0xffffffffLL)), hi = dppMov<CTRL>((int)(b >> 32));
+  return __longlong_as_double(((long long)hi << 32) | (unsigned)lo);
+}
+template <int CTRL> __device__ __forceinline__ long long dppMov(long long b) {
+  int lo = dppMov<CTRL>((int)(b & 0xffffffffLL)), hi = dppMov<CTRL>((int)(b >> 32));
+  return ((long long)hi << 32) | (unsigned)lo;
+}
+template <typename T> __device__ __forceinline__ T laneRead(T v, int lane) { return __shfl(v, lane, 64); }
+
+// 0xB1 = quad_perm[1,0,3,2] (lane^1), 0x4E = quad_perm[2,3,0,1] (lane^2),
+// 0x141 = row_half_mirror (i <-> 7-i), 0x140 = row_mirror (i <-> 15-i).
+template <typename Op, int WIDTH, typename T> __device__ __forceinline__ T waveAllReduce(T v) {
+  static_assert(WIDTH >= 1 && WIDTH <= 64 && (WIDTH & (WIDTH - 1)) == 0, "power of two up to 64");
+  if (WIDTH >= 2) v = Op::apply(v, dppMov<0xB1>(v));
+  if (WIDTH >= 4) v = Op::apply(v, dppMov<0x4E>(v));
+  if (WIDTH >= 8) v = Op::apply(v, dppMov<0x141>(v));
+  if (WIDTH >= 16) v = Op::apply(v, dppMov<0x140>(v));
+  if (WIDTH >= 32) v = Op::apply(v, __shfl_xor(v, 16, 64));
+  if (WIDTH >= 64) v = Op::apply(v, __shfl_xor(v, 32, 64));
+  return v;
+}
+
+__host__ __device__ constexpr int reduceScratchElems(int bx, int by, int bz) {
+  return ((bx & (bx - 1)) == 0 && bx <= 64) ? 1 : (bx % 64 == 0 ? (bx / 64) * by * bz : bx * by * bz);
+}
+
+template <typename Op, int BX, int BY, int BZ, typename T>
+__device__ __forceinline__ T blockAllReduceX(T v, T* scratch) {
+  if (BX == 1) {
+    return v;
+  }
+  if ((BX & (BX - 1)) == 0 && BX <= 64) {
+    // a row of BX threads is an aligned lane group of one wavefront
+    // (linear thread id = x + BX * (y + BY * z), BX divides 64)
+    return waveAllReduce<Op, (((BX & (BX - 1)) == 0 && BX <= 64) ? BX : 1)>(v);
+  }
+  const int row = threadIdx.y + BY * threadIdx.z;
+  if (BX % 64 == 0) {
+    // every wavefront lies inside one row: wave reduce, then combine BX/64 partials through LDS
+    constexpr int W = BX / 64;
+    v = waveAllReduce<Op, 64>(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) scratch[row * W + (threadIdx.x >> 6)] = v;
+    __syncthreads();
+    T r = scratch[row * W];
+#pragma unroll
+    for (int w = 1; w < W; ++w) r = Op::apply(r, scratch[row * W + w]);
+    return r;
+  }
+  // any other row width: rows straddle wavefronts, go through LDS
+  __syncthreads();
+  scratch[row * BX + threadIdx.x] = v;
+  __syncthreads();
+  T r = scratch[row * BX];
+  for (int x = 1; x < BX; ++x) r = Op::apply(r, scratch[row * BX + x]);
+  return r;
+}
+} // namespace __tc
+)HIP";
+
+inline std::string deviceLibrary(bool withReductions) {
+  std::string s = std::string(kDeviceTypes) + kDeviceIndexHelpers;
+  if (withReductions) {
+    s += kDeviceReductions;
+  }
+  return s;
+}
+
+} // namespace hip
+} // namespace tc

@@ -1,0 +1,106 @@
+#include "tc/core/hip/hip_rtc.h"
+
+#include <array>
+#include <iostream>
+
+#include "tc/core/check.h"
+#include "tc/core/flags.h"
+
+namespace tc {
+
+HipRTCFunction::~HipRTCFunction() {
+  if (!cleared_) {
+    try {
+      clear();
+    } catch (...) {
+    }
+  }
+}
+
+void HipRTCFunction::clear() {
+  if (cleared_) return;
+  for (auto& m : modules_) {
+    int old = 0;
+    if (tchip_get_device(&old) == 0) {
+      tchip_set_device(m.first);
+      tchip_module_unload(m.second);
+      tchip_set_device(old);
+    }
+  }
+  modules_.clear();
+  functions_.clear();
+  cleared_ = true;
+}
+
+std::unique_ptr<HipRTCFunction> HipRTCFunction::Compile(const std::string& name, const std::string& source) {
+  std::unique_ptr<HipRTCFunction> res(new HipRTCFunction());
+  res->name_ = name;
+  std::string arch = HipGPUInfo::GPUInfo().GetArch();
+  // Packed-FP32 instruction selection is switched off for all device code of this library.
+  std::vector<const char*> opts = {"-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+  if (tc::flags().fast_math) opts.push_back("-ffast-math");
+  char* code = nullptr;
+  char* log = nullptr;
+  size_t size = 0;
+  int status = tchip_rtc_compile(
+      source.c_str(), (name + ".hip").c_str(), arch.c_str(), opts.data(), static_cast<int>(opts.size()), &code, &size, &log);
+  std::string logText = log ? log : "";
+  tchip_free(log);
+  if (status != 0) {
+    tchip_free(code);
+    throw std::runtime_error("hipRTC compilation of " + name + " failed:\n" + logText + "\n--- source ---\n" + source);
+  }
+  res->code_.assign(code, size);
+  tchip_free(code);
+  return res;
+}
+
+Duration HipRTCFunction::Launch(
+    const std::vector<HipKernelLaunch>& kernels,
+    tchip_stream_t stream,
+    std::vector<int> params,
+    std::vector<void*> outputs,
+    std::vector<const void*> inputs,
+    bool profile) const {
+  TC_CHECK(!cleared_) << "launch of a cleared RTC function";
+  int dev = 0;
+  TC_HIP_CHECK(tchip_get_device(&dev));
+  if (!modules_.count(dev)) {
+    tchip_module_t m = nullptr;
+    TC_HIP_CHECK(tchip_module_load(code_.data(), &m));
+    modules_[dev] = m;
+  }
+  std::vector<void*> args;
+  for (auto& p : params) args.push_back(&p);
+  for (auto& p : outputs) args.push_back(&p);
+  for (auto& p : inputs) args.push_back((void*)&p);
+  TC_CHECK_LE(args.size(), 100u) << "too many kernel arguments";
+  tchip_event_t start = nullptr, stop = nullptr;
+  if (profile) {
+    TC_HIP_CHECK(tchip_event_create(&start));
+    TC_HIP_CHECK(tchip_event_create(&stop));
+    TC_HIP_CHECK(tchip_event_record(start, stream));
+  }
+  for (const auto& k : kernels) {
+    auto key = std::make_pair(dev, k.name);
+    auto it = functions_.find(key);
+    if (it == functions_.end()) {
+      tchip_function_t fn = nullptr;
+      TC_HIP_CHECK(tchip_module_get_function(modules_[dev], k.name.c_str(), &fn));
+      it = functions_.emplace(key, fn).first;
+    }
+    TC_HIP_CHECK(tchip_launch(it->second, k.grid.data(), k.block.data(), 0, stream, args.data()));
+  }
+  if (profile) {
+    float ms = 0;
+    TC_HIP_CHECK(tchip_event_record(stop, stream));
+    TC_HIP_CHECK(tchip_event_sync(stop));
+    TC_HIP_CHECK(tchip_event_elapsed_ms(start, stop, &ms));
+    TC_HIP_CHECK(tchip_event_destroy(start));
+    TC_HIP_CHECK(tchip_event_destroy(stop));
+    return Duration::fromNanoSeconds(static_cast<int64_t>(static_cast<double>(ms) * 1e6 + 0.5));
+  }
+  return Duration::max();
+}
+
+} // namespace tc

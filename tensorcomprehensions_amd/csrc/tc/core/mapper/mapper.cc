@@ -1,0 +1,1381 @@
+#include "tc/core/mapper/mapper.h"
+
+#include <algorithm>
+#include <cstdio>
+#include <functional>
+#include <set>
+#include <sstream>
+
+#include "tc/core/check.h"
+#include "tc/core/hip/hip_libraries.h"
+
+namespace tc {
+namespace mapper {
+namespace {
+
+using ir::Affine;
+using ir::Expr;
+using ir::ExprRef;
+using ir::ReduceOp;
+using ir::ScalarType;
+
+// ------------------------------------------------------------------------------------------
+// expression helpers
+// ------------------------------------------------------------------------------------------
+ExprRef mkExpr(Expr::Kind k, ScalarType t, std::string name, std::vector<ExprRef> args) {
+  auto e = std::make_shared<Expr>();
+  e->kind = k;
+  e->type = t;
+  e->name = std::move(name);
+  e->args = std::move(args);
+  return e;
+}
+ExprRef mkInt(int64_t v) {
+  auto e = std::make_shared<Expr>();
+  e->kind = Expr::IntImm;
+  e->type = ScalarType{ScalarType::Int, 32};
+  e->ival = v;
+  return e;
+}
+ExprRef mkVar(const std::string& n) {
+  return mkExpr(Expr::Var, ScalarType{ScalarType::Int, 32}, n, {});
+}
+ExprRef mkBin(const std::string& op, ExprRef a, ExprRef b) {
+  return mkExpr(Expr::Binary, ScalarType{ScalarType::Int, 32}, op, {std::move(a), std::move(b)});
+}
+
+// Rebuilds `e` bottom-up; `fn` may return a replacement for a node (after its children were
+// rewritten) or nullptr to keep it.
+ExprRef rewrite(const ExprRef& e, const std::function<ExprRef(const ExprRef&)>& fn) {
+  std::vector<ExprRef> args;
+  bool changed = false;
+  for (const auto& a : e->args) {
+    ExprRef n = rewrite(a, fn);
+    changed |= n != a;
+    args.push_back(n);
+  }
+  ExprRef cur = e;
+  if (changed) {
+    auto c = std::make_shared<Expr>(*e);
+    c->args = std::move(args);
+    cur = c;
+  }
+  ExprRef r = fn(cur);
+  return r ? r : cur;
+}
+
+void visit(const ExprRef& e, const std::function<void(const ExprRef&)>& fn) {
+  fn(e);
+  for (const auto& a : e->args) {
+    visit(a, fn);
+  }
+}
+
+bool sameExpr(const ExprRef& a, const ExprRef& b) {
+  if (a->kind != b->kind || a->name != b->name || a->ival != b->ival || a->fval != b->fval ||
+      a->args.size() != b->args.size() || a->type != b->type) {
+    return false;
+  }
+  for (size_t i = 0; i < a->args.size(); ++i) {
+    if (!sameExpr(a->args[i], b->args[i])) {
+      return false;
+    }
+  }
+  return true;
+}
+
+bool affineEqual(const Affine& a, const Affine& b) {
+  return a.valid && b.valid && a.coef == b.coef && a.constant == b.constant;
+}
+
+ScalarType matchType(const ScalarType& a, const ScalarType& b) {
+  if (a == b) return a;
+  if (!a.isFloat() && b.isFloat()) return b;
+  if (a.isFloat() && !b.isFloat()) return a;
+  if (a.isFloat() && b.isFloat()) return a.bits > b.bits ? a : b;
+  if (a.code == ScalarType::UInt && b.code == ScalarType::UInt) return a.bits > b.bits ? a : b;
+  return ScalarType{ScalarType::Int, std::max(a.bits, b.bits)};
+}
+
+std::string floatLiteral(double v, const ScalarType& t) {
+  char buf[64];
+  std::snprintf(buf, sizeof(buf), t.bits == 64 ? "%.17g" : "%.9g", v);
+  std::string s = buf;
+  if (s.find_first_of(".en") == std::string::npos) {
+    s += ".0";
+  }
+  if (s.find("inf") != std::string::npos || s.find("nan") != std::string::npos) {
+    return v > 0 ? "(1.0f/0.0f)" : "(-1.0f/0.0f)";
+  }
+  return t.bits == 64 ? s : s + "f";
+}
+
+int64_t ceilDiv(int64_t a, int64_t b) {
+  return (a + b - 1) / b;
+}
+
+const char* axisName(int a) {
+  return a == 0 ? "x" : a == 1 ? "y" : "z";
+}
+
+// ------------------------------------------------------------------------------------------
+// stage formation and kernel grouping
+// ------------------------------------------------------------------------------------------
+struct RawStage {
+  std::vector<const ir::Statement*> stmts;
+  const ir::Statement& first() const { return *stmts.front(); }
+};
+
+// subscripts of every access to `tensor` in the statement's right-hand side
+std::vector<std::vector<ExprRef>> accessesTo(const ir::Statement& s, const std::string& tensor) {
+  std::vector<std::vector<ExprRef>> out;
+  visit(s.rhs, [&](const ExprRef& e) {
+    if (e->kind == Expr::Load && e->name == tensor) {
+      out.push_back(e->args);
+    }
+  });
+  return out;
+}
+
+bool isIdentityAccess(const std::vector<ExprRef>& subs, const std::vector<std::string>& lhsVars) {
+  if (subs.size() != lhsVars.size()) {
+    return false;
+  }
+  for (size_t i = 0; i < subs.size(); ++i) {
+    if (subs[i]->kind != Expr::Var || subs[i]->name != lhsVars[i]) {
+      return false;
+    }
+  }
+  return true;
+}
+
+bool sameBox(const ir::Statement& a, const ir::Statement& b) {
+  if (a.tensor != b.tensor || a.lhsVars != b.lhsVars) {
+    return false;
+  }
+  for (const auto& v : a.lhsVars) {
+    const ir::Range &ra = a.ranges.at(v), &rb = b.ranges.at(v);
+    if (ra.min != rb.min || ra.max != rb.max) {
+      return false;
+    }
+  }
+  return true;
+}
+
+std::set<std::string> tensorsRead(const ir::Statement& s) {
+  std::set<std::string> r;
+  visit(s.rhs, [&](const ExprRef& e) {
+    if (e->kind == Expr::Load) {
+      r.insert(e->name);
+    }
+  });
+  if (s.op != ReduceOp::None && !s.init) {
+    r.insert(s.tensor);
+  }
+  return r;
+}
+
+// Largest d such that the dependence between stages A (earlier) and B is point-wise in the
+// first d left-hand-side positions of both, or -1 when they cannot share a kernel.
+int sharedPrefix(const RawStage& A, const RawStage& B) {
+  const ir::Statement &a0 = A.first(), &b0 = B.first();
+  size_t d = std::min(a0.lhsVars.size(), b0.lhsVars.size());
+  for (size_t p = 0; p < d; ++p) {
+    const ir::Range &ra = a0.ranges.at(a0.lhsVars[p]), &rb = b0.ranges.at(b0.lhsVars[p]);
+    if (ra.min != rb.min || ra.max != rb.max) {
+      d = p;
+      break;
+    }
+  }
+  auto limitBy = [&](const RawStage& reader, const std::string& tensor, size_t tensorRank) {
+    // every access of `reader` to `tensor` must use its own p-th index at position p
+    for (const auto* s : reader.stmts) {
+      for (const auto& subs : accessesTo(*s, tensor)) {
+        size_t ok = 0;
+        while (ok < d && ok < tensorRank && ok < subs.size() && subs[ok]->kind == Expr::Var &&
+               subs[ok]->name == s->lhsVars[ok]) {
+          ++ok;
+        }
+        d = std::min(d, ok);
+      }
+    }
+  };
+  // RAW / WAW: B touches what A wrote
+  limitBy(B, a0.tensor, a0.lhsVars.size());
+  if (a0.tensor == b0.tensor) {
+    return -1; // same tensor, different box: keep apart
+  }
+  // WAR: A read what B writes
+  limitBy(A, b0.tensor, b0.lhsVars.size());
+  return static_cast<int>(d);
+}
+
+// ------------------------------------------------------------------------------------------
+// stage canonicalisation: collapse + vector lanes
+// ------------------------------------------------------------------------------------------
+struct StageBuilder {
+  const ir::Function& f;
+  StagePlan st;
+
+  explicit StageBuilder(const ir::Function& fn) : f(fn) {}
+
+  LoopVar* var(const std::string& n) {
+    for (auto& v : st.vars) {
+      if (v.name == n) return &v;
+    }
+    return nullptr;
+  }
+
+  void init(const RawStage& raw) {
+    const ir::Statement& s0 = raw.first();
+    st.tensor = s0.tensor;
+    for (const auto& v : s0.lhsVars) {
+      st.lhsSubs.push_back(mkVar(v));
+      LoopVar lv;
+      lv.name = v;
+      lv.min = s0.ranges.at(v).min;
+      lv.extent = s0.ranges.at(v).extent();
+      st.vars.push_back(lv);
+    }
+    st.numParallel = static_cast<int>(st.vars.size());
+    int redId = 0;
+    for (const auto* s : raw.stmts) {
+      StageStmt ss;
+      ss.op = s->op;
+      ss.init = s->init;
+      ss.type = s->type;
+      ExprRef rhs = s->rhs;
+      // reduction variables get stage-unique names (two statements may both use "k")
+      for (const auto& r : s->redVars) {
+        std::string nn = r;
+        if (var(nn)) {
+          nn = r + "_" + std::to_string(redId);
+        }
+        ++redId;
+        if (nn != r) {
+          rhs = rewrite(rhs, [&](const ExprRef& e) -> ExprRef {
+            return (e->kind == Expr::Var && e->name == r) ? mkVar(nn) : nullptr;
+          });
+        }
+        LoopVar lv;
+        lv.name = nn;
+        lv.min = s->ranges.at(r).min;
+        lv.extent = s->ranges.at(r).extent();
+        lv.reduction = true;
+        st.vars.push_back(lv);
+        ss.redVars.push_back(nn);
+      }
+      ss.rhs = rhs;
+      st.stmts.push_back(ss);
+    }
+    auto addView = [&](const ir::Tensor& t, bool out) {
+      TensorView v;
+      v.name = t.name;
+      v.type = t.type;
+      v.extents = t.extents;
+      v.isOutput = out;
+      st.views[t.name] = v;
+    };
+    for (const auto& t : f.inputs) addView(t, false);
+    for (const auto& t : f.outputs) addView(t, true);
+  }
+
+  // variables used as values or inside non-affine subscripts cannot be merged or split
+  std::set<std::string> looseVars() {
+    std::set<std::string> loose;
+    std::function<void(const ExprRef&, bool)> walk = [&](const ExprRef& e, bool inAffineSub) {
+      if (e->kind == Expr::Var && !inAffineSub) {
+        loose.insert(e->name);
+      }
+      if (e->kind == Expr::Load) {
+        for (const auto& a : e->args) {
+          walk(a, ir::toAffine(a).valid);
+        }
+        return;
+      }
+      for (const auto& a : e->args) {
+        walk(a, inAffineSub);
+      }
+    };
+    for (const auto& s : st.stmts) {
+      walk(s.rhs, false);
+    }
+    return loose;
+  }
+
+  // all accesses (tensor, subscripts) of the stage including the store
+  void forEachAccess(const std::function<void(const std::string&, const std::vector<ExprRef>&)>& fn) {
+    fn(st.tensor, st.lhsSubs);
+    for (const auto& s : st.stmts) {
+      visit(s.rhs, [&](const ExprRef& e) {
+        if (e->kind == Expr::Load) fn(e->name, e->args);
+      });
+    }
+  }
+
+  static bool mentions(const ExprRef& e, const std::string& v) {
+    bool m = false;
+    visit(e, [&](const ExprRef& x) { m |= x->kind == Expr::Var && x->name == v; });
+    return m;
+  }
+  static bool isExactly(const ExprRef& e, const std::string& v) {
+    Affine a = ir::toAffine(e);
+    return a.valid && a.constant == 0 && a.coef.size() == 1 && a.coefOf(v) == 1;
+  }
+
+  // Merge adjacent parallel variables a,b when every access that mentions them has `a` alone in
+  // some dimension j and `b` alone in dimension j+1 spanning that whole dimension: the pair then
+  // walks memory exactly like one variable of extent |a|*|b| over the merged dimension.
+  bool tryCollapse(size_t k) {
+    LoopVar &a = st.vars[k], &b = st.vars[k + 1];
+    if (a.min != 0 || b.min != 0) return false;
+    auto loose = looseVars();
+    if (loose.count(a.name) || loose.count(b.name)) return false;
+    std::map<std::string, std::set<size_t>> mergeAt; // tensor -> dims j to merge with j+1
+    bool ok = true;
+    forEachAccess([&](const std::string& t, const std::vector<ExprRef>& subs) {
+      bool any = false;
+      for (const auto& s : subs) any |= mentions(s, a.name) || mentions(s, b.name);
+      if (!any) return;
+      size_t found = subs.size();
+      for (size_t j = 0; j + 1 < subs.size(); ++j) {
+        if (isExactly(subs[j], a.name) && isExactly(subs[j + 1], b.name)) found = j;
+      }
+      if (found == subs.size() || st.views.at(t).extents[found + 1] != b.extent) {
+        ok = false;
+        return;
+      }
+      for (size_t j = 0; j < subs.size(); ++j) {
+        if (j != found && j != found + 1 && (mentions(subs[j], a.name) || mentions(subs[j], b.name))) {
+          ok = false;
+        }
+      }
+      mergeAt[t].insert(found);
+    });
+    if (!ok) return false;
+    for (const auto& m : mergeAt) {
+      if (m.second.size() != 1) return false; // one merge position per tensor
+    }
+    std::string merged = a.name + "_" + b.name;
+    int64_t eb = b.extent;
+    auto rewriteSubs = [&](const std::string& t, const std::vector<ExprRef>& subs) {
+      auto it = mergeAt.find(t);
+      if (it == mergeAt.end()) return subs;
+      size_t j = *it->second.begin();
+      std::vector<ExprRef> out(subs.begin(), subs.begin() + j);
+      if (isExactly(subs[j], a.name) && isExactly(subs[j + 1], b.name)) {
+        out.push_back(mkVar(merged));
+      } else {
+        out.push_back(mkBin("+", mkBin("*", subs[j], mkInt(st.views.at(t).extents[j + 1])), subs[j + 1]));
+      }
+      out.insert(out.end(), subs.begin() + j + 2, subs.end());
+      return out;
+    };
+    st.lhsSubs = rewriteSubs(st.tensor, st.lhsSubs);
+    for (auto& s : st.stmts) {
+      s.rhs = rewrite(s.rhs, [&](const ExprRef& e) -> ExprRef {
+        if (e->kind != Expr::Load || !mergeAt.count(e->name)) return nullptr;
+        auto c = std::make_shared<Expr>(*e);
+        c->args = rewriteSubs(e->name, e->args);
+        return c;
+      });
+    }
+    for (const auto& m : mergeAt) {
+      auto& ext = st.views.at(m.first).extents;
+      size_t j = *m.second.begin();
+      ext[j] *= ext[j + 1];
+      ext.erase(ext.begin() + j + 1);
+    }
+    a.name = merged;
+    a.extent *= eb;
+    st.vars.erase(st.vars.begin() + k + 1);
+    st.numParallel -= 1;
+    return true;
+  }
+
+  void collapse() {
+    for (size_t k = 0; k + 1 < static_cast<size_t>(st.numParallel);) {
+      if (!tryCollapse(k)) ++k;
+    }
+  }
+
+  // x = xo * V + xv with xv the innermost, always unrolled lane variable
+  bool splitLanes(const std::string& name, int64_t V) {
+    LoopVar* v = var(name);
+    if (!v || V <= 1 || v->min != 0 || v->extent % V != 0 || v->extent == V) return false;
+    if (looseVars().count(name)) return false;
+    std::string xo = name + "_o", xv = name + "_v";
+    ExprRef repl = mkBin("+", mkBin("*", mkVar(xo), mkInt(V)), mkVar(xv));
+    auto sub = [&](const ExprRef& e) -> ExprRef {
+      return (e->kind == Expr::Var && e->name == name) ? repl : nullptr;
+    };
+    for (auto& s : st.lhsSubs) s = rewrite(s, sub);
+    for (auto& s : st.stmts) {
+      s.rhs = rewrite(s.rhs, sub);
+      for (size_t i = 0; i < s.redVars.size(); ++i) {
+        if (s.redVars[i] == name) {
+          s.redVars[i] = xo;
+          s.redVars.insert(s.redVars.begin() + i + 1, xv);
+          break;
+        }
+      }
+    }
+    size_t idx = v - &st.vars[0];
+    LoopVar lane = *v;
+    lane.name = xv;
+    lane.extent = V;
+    lane.vectorLane = true;
+    st.vars[idx].name = xo;
+    st.vars[idx].extent /= V;
+    st.vars.insert(st.vars.begin() + idx + 1, lane);
+    if (!lane.reduction) st.numParallel += 1;
+    return true;
+  }
+};
+
+// ------------------------------------------------------------------------------------------
+// code emission
+// ------------------------------------------------------------------------------------------
+class Emitter {
+ public:
+  std::ostringstream out;
+  int indent = 0;
+  void line(const std::string& s) { out << std::string(indent * 2, ' ') << s << "\n"; }
+  void open(const std::string& s) {
+    line(s.empty() ? "{" : s + " {");
+    ++indent;
+  }
+  void close() {
+    --indent;
+    line("}");
+  }
+};
+
+struct KernelCtx {
+  const ir::Function& f;
+  const HipMappingOptions& opts;
+  KernelPlan& k;
+  std::string idx = "int"; // index arithmetic type
+  int64_t NT() const { return k.block[0] * k.block[1] * k.block[2]; }
+};
+
+class StageCodegen {
+ public:
+  StageCodegen(KernelCtx& kc, StagePlan& st, int stageIdx, Emitter& em)
+      : kc_(kc), st_(st), stageIdx_(stageIdx), em_(em) {}
+
+  // --- naming -------------------------------------------------------------------------------
+  std::string iv(const LoopVar& v) const { return "i_" + v.name; }
+  std::string tv(const LoopVar& v) const { return v.numTiles > 1 ? "t_" + v.name : "0"; }
+
+  const LoopVar& var(const std::string& n) const {
+    for (const auto& v : st_.vars) {
+      if (v.name == n) return v;
+    }
+    TC_CHECK(false) << "unknown loop variable " << n;
+    return st_.vars[0];
+  }
+
+  // affine over i_<var> values -> C
+  std::string affineStr(const Affine& a) const {
+    std::ostringstream ss;
+    bool first = true;
+    for (const auto& c : a.coef) {
+      if (c.second == 0) continue;
+      int64_t k = c.second;
+      if (!first) ss << (k < 0 ? " - " : " + ");
+      else if (k < 0) ss << "-";
+      int64_t m = k < 0 ? -k : k;
+      if (m != 1) ss << m << " * ";
+      ss << "i_" << c.first;
+      first = false;
+    }
+    if (first) {
+      ss << a.constant;
+    } else if (a.constant != 0) {
+      ss << (a.constant < 0 ? " - " : " + ") << (a.constant < 0 ? -a.constant : a.constant);
+    }
+    return ss.str();
+  }
+
+  // --- expressions --------------------------------------------------------------------------
+  std::string castTo(const ExprRef& e, const ScalarType& t, const std::string& accRef) {
+    std::string s = expr(e, accRef);
+    if (e->type == t || t.isBool()) return s;
+    return "((" + t.cName() + ")(" + s + "))";
+  }
+
+  std::string flatIndex(const std::string& tensor, const std::vector<ExprRef>& subs, const std::string& accRef) {
+    const TensorView& v = st_.views.at(tensor);
+    auto strides = makeStridesFromSizes(v.extents);
+    Affine total;
+    total.valid = true;
+    std::string extra;
+    for (size_t j = 0; j < subs.size(); ++j) {
+      Affine a = ir::toAffine(subs[j]);
+      if (a.valid) {
+        for (const auto& c : a.coef) total.coef[c.first] += c.second * strides[j];
+        total.constant += a.constant * strides[j];
+      } else {
+        extra += " + " + std::to_string(strides[j]) + " * (" + kc_.idx + ")(" + expr(subs[j], accRef) + ")";
+      }
+    }
+    return affineStr(total) + extra;
+  }
+
+  std::string loadStr(const ExprRef& e, const std::string& accRef) {
+    // the stage's own running value
+    if (e->name == st_.tensor && !accRef.empty() && e->args.size() == st_.lhsSubs.size()) {
+      bool same = true;
+      for (size_t i = 0; i < e->args.size(); ++i) same &= sameExpr(e->args[i], st_.lhsSubs[i]);
+      if (same) return accRef;
+    }
+    for (const auto& p : st_.promotions) {
+      if (p.tensor == e->name && activePromotions_.count(p.tensor)) {
+        return p.ldsName + "[" + ldsIndex(p, e->args) + "]";
+      }
+    }
+    return "p" + e->name + "[" + flatIndex(e->name, e->args, accRef) + "]";
+  }
+
+  std::string expr(const ExprRef& e, const std::string& accRef) {
+    switch (e->kind) {
+      case Expr::IntImm:
+        return std::to_string(e->ival);
+      case Expr::FloatImm:
+        return floatLiteral(e->fval, e->type);
+      case Expr::Var:
+        return "i_" + e->name;
+      case Expr::Load:
+        return loadStr(e, accRef);
+      case Expr::Cast:
+        return "((" + e->type.cName() + ")(" + expr(e->args[0], accRef) + "))";
+      case Expr::Unary:
+        return "(" + e->name + expr(e->args[0], accRef) + ")";
+      case Expr::Select:
+        return "(" + expr(e->args[0], accRef) + " ? " + castTo(e->args[1], e->type, accRef) + " : " +
+            castTo(e->args[2], e->type, accRef) + ")";
+      case Expr::Call: {
+        std::string s = e->name + "(";
+        for (size_t i = 0; i < e->args.size(); ++i) {
+          s += (i ? ", " : "") + castTo(e->args[i], e->type, accRef);
+        }
+        return s + ")";
+      }
+      case Expr::Binary: {
+        ScalarType mt = matchType(e->args[0]->type, e->args[1]->type);
+        if (e->name == "&&" || e->name == "||") {
+          return "(" + expr(e->args[0], accRef) + " " + e->name + " " + expr(e->args[1], accRef) + ")";
+        }
+        std::string a = castTo(e->args[0], mt, accRef), b = castTo(e->args[1], mt, accRef);
+        if (e->name == "min") return "__tc::tmin(" + a + ", " + b + ")";
+        if (e->name == "max") return "__tc::tmax(" + a + ", " + b + ")";
+        if (e->name == "/" && !mt.isFloat()) return "__tc::floordiv(" + a + ", " + b + ")";
+        if (e->name == "%" && !mt.isFloat()) return "__tc::floormod(" + a + ", " + b + ")";
+        if (e->name == "%") return std::string(mt.bits == 64 ? "fmod(" : "fmodf(") + a + ", " + b + ")";
+        return "(" + a + " " + e->name + " " + b + ")";
+      }
+    }
+    return "0";
+  }
+
+  static std::string combine(ReduceOp op, const std::string& a, const std::string& b) {
+    switch (op) {
+      case ReduceOp::Plus: return "(" + a + " + " + b + ")";
+      case ReduceOp::Times: return "(" + a + " * " + b + ")";
+      case ReduceOp::Min: return "__tc::tmin(" + a + ", " + b + ")";
+      case ReduceOp::Max: return "__tc::tmax(" + a + ", " + b + ")";
+      default: return b;
+    }
+  }
+  static std::string opStruct(ReduceOp op, const ScalarType& t) {
+    const char* n = op == ReduceOp::Plus ? "OpSum" : op == ReduceOp::Times ? "OpProd" : op == ReduceOp::Min ? "OpMin" : "OpMax";
+    return std::string("__tc::") + n + "<" + t.cName() + ">";
+  }
+
+  // --- LDS ------------------------------------------------------------------------------------
+  // lower corner of a promoted tensor's footprint in view dimension j, as C on tile indices
+  struct Footprint {
+    std::vector<Affine> coefs;          // subscript structure shared by all accesses
+    std::vector<int64_t> minConst;      // smallest constant per dimension over the accesses
+  };
+  std::map<std::string, Footprint> footprints_;
+
+  // span of a variable inside the region a promotion covers, and its low value as C
+  int64_t spanOf(const LoopVar& v, bool insideReductionTiles) const {
+    if (v.reduction && !insideReductionTiles) return v.extent;
+    return v.tile;
+  }
+  std::string lowOf(const LoopVar& v, bool insideReductionTiles) const {
+    if ((v.reduction && !insideReductionTiles) || v.numTiles == 1) return std::to_string(v.min);
+    return "(" + std::to_string(v.min) + " + " + tv(v) + " * " + std::to_string(v.tile) + ")";
+  }
+
+  std::string footprintLow(const Promotion& p, size_t j) const {
+    const Footprint& fp = footprints_.at(p.tensor);
+    std::ostringstream ss;
+    ss << fp.minConst[j];
+    for (const auto& c : fp.coefs[j].coef) {
+      const LoopVar& v = var(c.first);
+      if (c.second > 0) {
+        ss << " + " << c.second << " * " << lowOf(v, p.insideReductionTiles);
+      } else {
+        ss << " - " << -c.second << " * (" << lowOf(v, p.insideReductionTiles) << " + "
+           << spanOf(v, p.insideReductionTiles) - 1 << ")";
+      }
+    }
+    return ss.str();
+  }
+
+  std::string ldsIndex(const Promotion& p, const std::vector<ExprRef>& subs) {
+    std::ostringstream ss;
+    for (size_t j = 0; j < subs.size(); ++j) {
+      if (j) ss << " + ";
+      ss << "((" << affineStr(ir::toAffine(subs[j])) << ") - lo" << stageIdx_ << "_" << p.tensor << "_" << j << ")";
+      if (p.ldsStrides[j] != 1) ss << " * " << p.ldsStrides[j];
+    }
+    if (subs.empty()) ss << "0";
+    return ss.str();
+  }
+
+  // Decide which read-only operands of statement `s` to stage in LDS.
+  void planPromotions(const StageStmt& s, int64_t& ldsBudgetBytes) {
+    if (!kc_.opts.useSharedMemoryValue || s.redVars.empty()) return;
+    for (const auto& v : st_.vars) {
+      if (!v.reduction && !v.unrolled && v.perThread > 1) return; // needs a full register tile
+    }
+    bool reductionTiled = false;
+    for (const auto& r : s.redVars) reductionTiled |= var(r).numTiles > 1;
+    bool inside = reductionTiled &&
+        (!kc_.opts.hasSharedDepth || kc_.opts.sharedDepthValue > static_cast<uint32_t>(st_.numParallel));
+    // iterations of the statement inside the promoted region
+    std::set<std::string> stmtVars;
+    for (int i = 0; i < st_.numParallel; ++i) stmtVars.insert(st_.vars[i].name);
+    for (const auto& r : s.redVars) stmtVars.insert(r);
+    double iterations = 1;
+    for (const auto& n : stmtVars) iterations *= static_cast<double>(spanOf(var(n), inside));
+
+    std::map<std::string, std::vector<std::vector<Affine>>> accesses;
+    std::set<std::string> bad;
+    visit(s.rhs, [&](const ExprRef& e) {
+      if (e->kind != Expr::Load || e->name == st_.tensor) return;
+      std::vector<Affine> subs;
+      for (const auto& a : e->args) {
+        Affine x = ir::toAffine(a);
+        if (!x.valid) bad.insert(e->name);
+        subs.push_back(x);
+      }
+      accesses[e->name].push_back(subs);
+    });
+    struct Cand {
+      Promotion p;
+      Footprint fp;
+      int64_t bytes;
+    };
+    std::vector<Cand> cands;
+    for (const auto& acc : accesses) {
+      if (bad.count(acc.first)) continue;
+      const TensorView& view = st_.views.at(acc.first);
+      if (view.isOutput) continue; // may be written by another stage of this kernel
+      const auto& ref = acc.second.front();
+      bool sameShape = true;
+      for (const auto& a : acc.second) {
+        for (size_t j = 0; j < a.size(); ++j) sameShape &= a[j].coef == ref[j].coef;
+      }
+      if (!sameShape) continue;
+      Cand c;
+      c.p.tensor = acc.first;
+      c.p.ldsName = "lds" + std::to_string(stageIdx_) + "_" + acc.first;
+      c.p.insideReductionTiles = inside;
+      c.fp.coefs = ref;
+      int64_t elems = 1;
+      for (size_t j = 0; j < ref.size(); ++j) {
+        int64_t lo = ref[j].constant, hi = ref[j].constant;
+        for (const auto& a : acc.second) {
+          lo = std::min(lo, a[j].constant);
+          hi = std::max(hi, a[j].constant);
+        }
+        int64_t ext = 1 + (hi - lo);
+        for (const auto& cv : ref[j].coef) {
+          ext += std::abs(cv.second) * (spanOf(var(cv.first), inside) - 1);
+        }
+        c.fp.minConst.push_back(lo);
+        c.p.extents.push_back(ext);
+        elems *= ext;
+      }
+      c.p.reuse = static_cast<int64_t>(iterations * acc.second.size() / static_cast<double>(elems));
+      if (c.p.reuse < 2) continue;
+      // pad the innermost extent to an odd size when lanes walk a slower dimension
+      std::vector<int64_t> padded = c.p.extents;
+      if (!padded.empty() && padded.back() > 1 && padded.back() % 2 == 0 && lanesWalkOuterDim(ref)) {
+        padded.back() += 1;
+      }
+      c.p.ldsStrides = makeStridesFromSizes(padded);
+      c.p.elems = 1;
+      for (auto e : padded) c.p.elems *= e;
+      c.bytes = c.p.elems * view.type.bytes();
+      cands.push_back(c);
+    }
+    // most reused first, name as tie-break for determinism
+    std::sort(cands.begin(), cands.end(), [](const Cand& a, const Cand& b) {
+      return a.p.reuse != b.p.reuse ? a.p.reuse > b.p.reuse : a.p.tensor < b.p.tensor;
+    });
+    for (auto& c : cands) {
+      if (c.bytes <= ldsBudgetBytes) {
+        ldsBudgetBytes -= c.bytes;
+        footprints_[c.p.tensor] = c.fp;
+        st_.promotions.push_back(c.p);
+      }
+    }
+  }
+
+  bool lanesWalkOuterDim(const std::vector<Affine>& subs) const {
+    const LoopVar* x = nullptr;
+    for (const auto& v : st_.vars) {
+      if (v.threadAxis == 0) x = &v;
+    }
+    if (!x || subs.empty()) return false;
+    if (subs.back().coefOf(x->name) != 0) return false;
+    for (size_t j = 0; j + 1 < subs.size(); ++j) {
+      if (subs[j].coefOf(x->name) != 0) return true;
+    }
+    return false;
+  }
+
+  void emitLdsDecls() {
+    for (const auto& p : st_.promotions) {
+      em_.line("__shared__ " + st_.views.at(p.tensor).type.cName() + " " + p.ldsName + "[" +
+               std::to_string(p.elems) + "];");
+    }
+  }
+
+  void emitCopyIn(const Promotion& p) {
+    const TensorView& view = st_.views.at(p.tensor);
+    auto gStrides = makeStridesFromSizes(view.extents);
+    int64_t count = 1;
+    for (auto e : p.extents) count *= e;
+    for (size_t j = 0; j < p.extents.size(); ++j) {
+      em_.line("const int lo" + std::to_string(stageIdx_) + "_" + p.tensor + "_" + std::to_string(j) + " = " +
+               footprintLow(p, j) + ";");
+    }
+    if (kc_.opts.unrollCopySharedValue) em_.line("#pragma unroll");
+    em_.open("for (int c_ = tid_; c_ < " + std::to_string(count) + "; c_ += " + std::to_string(kc_.NT()) + ")");
+    int64_t div = count;
+    std::string cond, gidx, lidx;
+    for (size_t j = 0; j < p.extents.size(); ++j) {
+      div /= p.extents[j];
+      std::string l = "l" + std::to_string(j) + "_";
+      std::string e = "c_";
+      if (div > 1) e = "(" + e + " / " + std::to_string(div) + ")";
+      if (j > 0) e = e + " % " + std::to_string(p.extents[j]);
+      em_.line("const int " + l + " = " + e + ";");
+      std::string g = "g" + std::to_string(j) + "_";
+      em_.line("const int " + g + " = lo" + std::to_string(stageIdx_) + "_" + p.tensor + "_" + std::to_string(j) + " + " + l + ";");
+      cond += (j ? " && " : "") + std::string("(unsigned)") + g + " < " + std::to_string(view.extents[j]) + "u";
+      gidx += (j ? " + " : "") + g + (gStrides[j] != 1 ? " * " + std::to_string(gStrides[j]) : "");
+      lidx += (j ? " + " : "") + l + (p.ldsStrides[j] != 1 ? " * " + std::to_string(p.ldsStrides[j]) : "");
+    }
+    if (p.extents.empty()) {
+      cond = "true";
+      gidx = lidx = "0";
+    }
+    em_.line("if (" + cond + ") " + p.ldsName + "[" + lidx + "] = p" + p.tensor + "[" + gidx + "];");
+    em_.close();
+  }
+
+  // --- loops ----------------------------------------------------------------------------------
+  // Opens the per-thread point loop of `v` (uniform trip count across the block), declares
+  // i_<v> and returns the predicate term this variable contributes ("" when always valid).
+  std::string openPointLoop(const LoopVar& v, bool unrollPragma, int unrollFactor = 0) {
+    std::string q = "q_" + v.name;
+    std::string B = v.threadAxis >= 0 ? std::to_string(kc_.k.block[v.threadAxis]) : "1";
+    if (v.perThread > 1) {
+      if (unrollPragma) em_.line(unrollFactor > 1 ? "#pragma unroll " + std::to_string(unrollFactor) : "#pragma unroll");
+      em_.open("for (int " + q + " = 0; " + q + " < " + std::to_string(v.perThread) + "; ++" + q + ")");
+    } else {
+      em_.open("");
+    }
+    std::string qv = v.perThread > 1 ? q : "0";
+    std::string p;
+    if (v.threadAxis >= 0) {
+      p = qv == "0" ? std::string("(int)threadIdx.") + axisName(v.threadAxis)
+                    : "(" + qv + " * " + B + " + (int)threadIdx." + axisName(v.threadAxis) + ")";
+    } else {
+      p = qv;
+    }
+    std::string base = std::to_string(v.min);
+    if (v.numTiles > 1) base += " + " + tv(v) + " * " + std::to_string(v.tile);
+    em_.line("const int p_" + v.name + " = " + p + ";");
+    em_.line("const int " + iv(v) + " = " + base + " + p_" + v.name + ";");
+    std::string pred;
+    if (v.threadAxis >= 0 && v.perThread * kc_.k.block[v.threadAxis] != v.tile) {
+      pred = "p_" + v.name + " < " + std::to_string(v.tile);
+    }
+    if (v.partial()) {
+      pred += (pred.empty() ? "" : " && ") + iv(v) + " <= " + std::to_string(v.min + v.extent - 1);
+    }
+    return pred;
+  }
+
+  // Register-tile loops: opens loops over all unrolled parallel variables, defines `ok_` and
+  // the accumulator slot `a_`; the caller emits the body and then calls closeUnrolled().
+  int openUnrolled() {
+    em_.open("");
+    int opened = 1;
+    std::string pred = outerPred_;
+    std::string slot = "0";
+    for (int i = 0; i < st_.numParallel; ++i) {
+      const LoopVar& v = st_.vars[i];
+      if (!v.unrolled) continue;
+      std::string t = openPointLoop(v, true);
+      ++opened;
+      if (!t.empty()) pred += (pred.empty() ? "" : " && ") + t;
+      if (v.perThread > 1) slot = "(" + slot + ") * " + std::to_string(v.perThread) + " + q_" + v.name;
+    }
+    em_.line("const bool ok_ = " + (pred.empty() ? std::string("true") : pred) + ";");
+    em_.line("const int a_ = " + slot + ";");
+    return opened;
+  }
+  void closeN(int n) {
+    for (int i = 0; i < n; ++i) em_.close();
+  }
+
+  // thread axes this stage does not use must not duplicate its work
+  std::string idleAxesPred() const {
+    std::string p;
+    for (int a = 0; a < 3; ++a) {
+      if (kc_.k.block[a] == 1) continue;
+      bool used = false;
+      for (const auto& v : st_.vars) used |= v.threadAxis == a;
+      if (!used) p += (p.empty() ? "" : " && ") + std::string("threadIdx.") + axisName(a) + " == 0";
+    }
+    return p;
+  }
+
+  // --- statements -----------------------------------------------------------------------------
+  void emitPointwise(const StageStmt& s) {
+    int n = openUnrolled();
+    em_.line("if (ok_) acc_[a_] = " + castTo(s.rhs, accType_, accValid_ ? "acc_[a_]" : "") + ";");
+    closeN(n);
+  }
+
+  void preloadAcc() {
+    int n = openUnrolled();
+    em_.line("if (ok_) acc_[a_] = p" + st_.tensor + "[" + flatIndex(st_.tensor, st_.lhsSubs, "") + "];");
+    closeN(n);
+    accValid_ = true;
+  }
+
+  static bool readsOwnValue(const StageStmt& s, const StagePlan& st) {
+    bool r = false;
+    visit(s.rhs, [&](const ExprRef& e) { r |= e->kind == Expr::Load && e->name == st.tensor; });
+    return r;
+  }
+
+  void emitReduction(const StageStmt& s, int64_t unrollBudget) {
+    bool threadRed = false;
+    for (const auto& r : s.redVars) threadRed |= st_.threadReduction && var(r).threadAxis == 0;
+    std::string target = threadRed ? "part_" : "acc_";
+    std::string ident = ir::identityLiteral(s.op, accType_);
+    if (!s.init && !accValid_) preloadAcc();
+    {
+      int n = openUnrolled();
+      if (threadRed) {
+        em_.line("part_[a_] = " + ident + ";");
+        if (s.init) em_.line("acc_[a_] = " + ident + ";");
+      } else if (s.init) {
+        em_.line("acc_[a_] = " + ident + ";");
+      }
+      closeN(n);
+    }
+    accValid_ = true;
+    // promotions that cover the whole reduction go in front of the reduction loops
+    bool anyOutside = false, anyInside = false;
+    for (const auto& p : st_.promotions) (p.insideReductionTiles ? anyInside : anyOutside) = true;
+    auto copyIn = [&](bool inside) {
+      em_.line("__syncthreads();");
+      for (const auto& p : st_.promotions) {
+        if (p.insideReductionTiles == inside) {
+          emitCopyIn(p);
+          activePromotions_.insert(p.tensor);
+        }
+      }
+      em_.line("__syncthreads();");
+    };
+    int opened = 0;
+    if (anyOutside) {
+      em_.open("");
+      ++opened;
+      copyIn(false);
+    }
+    for (const auto& r : s.redVars) {
+      const LoopVar& v = var(r);
+      if (v.numTiles > 1) {
+        em_.open("for (int t_" + v.name + " = 0; t_" + v.name + " < " + std::to_string(v.numTiles) + "; ++t_" + v.name + ")");
+        ++opened;
+      }
+    }
+    if (anyInside) copyIn(true);
+    // point loops, innermost ones unrolled under the budget
+    std::vector<int> factors(s.redVars.size(), 0); // 0: no pragma, -1: full, >1: partial
+    int64_t remaining = std::max<int64_t>(1, unrollBudget / std::max<int64_t>(1, st_.accCount));
+    for (int i = static_cast<int>(s.redVars.size()) - 1; i >= 0; --i) {
+      const LoopVar& v = var(s.redVars[i]);
+      if (v.vectorLane) {
+        factors[i] = -1;
+        continue;
+      }
+      if (v.perThread <= remaining) {
+        factors[i] = -1;
+        remaining /= std::max<int64_t>(1, v.perThread);
+      } else {
+        if (remaining >= 2) factors[i] = static_cast<int>(remaining);
+        break;
+      }
+    }
+    std::string rpred;
+    int ropened = 0;
+    for (size_t i = 0; i < s.redVars.size(); ++i) {
+      const LoopVar& v = var(s.redVars[i]);
+      std::string t = openPointLoop(v, factors[i] != 0, factors[i] > 1 ? factors[i] : 0);
+      ++ropened;
+      if (!t.empty()) rpred += (rpred.empty() ? "" : " && ") + t;
+    }
+    {
+      int n = openUnrolled();
+      std::string cond = rpred.empty() ? "ok_" : "ok_ && " + rpred;
+      std::string rhs = castTo(s.rhs, accType_, "acc_[a_]");
+      em_.line("if (" + cond + ") " + target + "[a_] = " + combine(s.op, target + "[a_]", rhs) + ";");
+      closeN(n);
+    }
+    closeN(ropened);
+    closeN(opened);
+    for (const auto& p : st_.promotions) activePromotions_.erase(p.tensor);
+    if (threadRed) {
+      // every thread of the block reaches this point (uniform loops), as the barriers require
+      int n = openUnrolled();
+      em_.line("const " + accType_.cName() + " tot_ = __tc::blockAllReduceX<" + opStruct(s.op, accType_) + ", " +
+               std::to_string(kc_.k.block[0]) + ", " + std::to_string(kc_.k.block[1]) + ", " +
+               std::to_string(kc_.k.block[2]) + ">(part_[a_], red_scratch_);");
+      em_.line("acc_[a_] = " + combine(s.op, "acc_[a_]", "tot_") + ";");
+      closeN(n);
+    }
+  }
+
+  // --- whole stage ----------------------------------------------------------------------------
+  void plan(int64_t& ldsBudgetBytes) {
+    for (const auto& s : st_.stmts) {
+      if (!s.redVars.empty()) {
+        planPromotions(s, ldsBudgetBytes);
+        break;
+      }
+    }
+  }
+
+  void emit() {
+    accType_ = st_.views.at(st_.tensor).type;
+    em_.line("// stage " + std::to_string(stageIdx_) + ": " + st_.tensor);
+    em_.open("");
+    int opened = 1;
+    // sequential tile loops of parallel variables not handled at kernel level
+    for (int i = kc_.k.sharedDepth; i < st_.numParallel; ++i) {
+      const LoopVar& v = st_.vars[i];
+      if (v.numTiles > 1) {
+        em_.open("for (int t_" + v.name + " = 0; t_" + v.name + " < " + std::to_string(v.numTiles) + "; ++t_" + v.name + ")");
+        ++opened;
+      }
+    }
+    // per-thread point loops that stay loops
+    outerPred_ = idleAxesPredForCompute();
+    for (int i = 0; i < st_.numParallel; ++i) {
+      const LoopVar& v = st_.vars[i];
+      if (v.unrolled) continue;
+      std::string t = openPointLoop(v, false);
+      ++opened;
+      if (!t.empty()) outerPred_ += (outerPred_.empty() ? "" : " && ") + t;
+    }
+    em_.line(accType_.cName() + " acc_[" + std::to_string(st_.accCount) + "];");
+    if (st_.threadReduction) em_.line(accType_.cName() + " part_[" + std::to_string(st_.accCount) + "];");
+    accValid_ = false;
+    int64_t budget = kc_.opts.generic.hasUnroll ? static_cast<int64_t>(kc_.opts.generic.unrollValue) : 1;
+    for (const auto& s : st_.stmts) {
+      if (s.redVars.empty()) {
+        if (s.op != ReduceOp::None) {
+          // reduction operator without reduction indices: a single combine with the old value
+          if (!accValid_) preloadAcc();
+          int n = openUnrolled();
+          em_.line("if (ok_) acc_[a_] = " + combine(s.op, "acc_[a_]", castTo(s.rhs, accType_, "acc_[a_]")) + ";");
+          closeN(n);
+        } else {
+          if (!accValid_ && readsOwnValue(s, st_)) preloadAcc();
+          emitPointwise(s);
+          accValid_ = true;
+        }
+      } else {
+        emitReduction(s, budget);
+      }
+    }
+    // store
+    {
+      int n = openUnrolled();
+      std::string cond = "ok_";
+      if (st_.threadReduction) cond += " && threadIdx.x == 0";
+      em_.line("if (" + cond + ") p" + st_.tensor + "[" + flatIndex(st_.tensor, st_.lhsSubs, "") + "] = acc_[a_];");
+      closeN(n);
+    }
+    closeN(opened);
+  }
+
+  std::string idleAxesPredForCompute() const {
+    // With a thread-mapped reduction all threads must take part in the barriers; idle axes are
+    // filtered by the predicate rather than by skipping code.
+    return idleAxesPred();
+  }
+
+ private:
+  KernelCtx& kc_;
+  StagePlan& st_;
+  int stageIdx_;
+  Emitter& em_;
+  ScalarType accType_;
+  bool accValid_ = false;
+  std::string outerPred_;
+  std::set<std::string> activePromotions_;
+};
+
+// ------------------------------------------------------------------------------------------
+// mapping of one kernel
+// ------------------------------------------------------------------------------------------
+void mapKernel(KernelCtx& kc, const DeviceLimits& limits) {
+  const HipMappingOptions& o = kc.opts;
+  KernelPlan& k = kc.k;
+  TC_CHECK(!o.generic.hasTiling || !o.generic.tiling.empty()) << "tiling must hold at least one size";
+  for (size_t a = 0; a < 3; ++a) {
+    TC_CHECK_GT(o.grid[a], 0u) << "NYI: mapping to 0 blocks";
+    TC_CHECK_GT(o.block[a], 0u) << "NYI: mapping to 0 threads";
+  }
+  std::array<int64_t, 3> blockUse{{1, 1, 1}}, gridUse{{1, 1, 1}};
+  for (auto& st : k.stages) {
+    // tile sizes by band position (lanes do not take a position)
+    int pos = 0;
+    for (auto& v : st.vars) {
+      if (v.vectorLane) {
+        v.tile = v.extent;
+        v.numTiles = 1;
+        continue;
+      }
+      int64_t t = 0;
+      if (o.generic.hasTiling && pos < static_cast<int>(o.generic.tiling.size())) {
+        t = static_cast<int64_t>(o.generic.tiling[pos]);
+      }
+      ++pos;
+      // a lane-split variable is tiled in units of whole lane groups
+      const LoopVar* next = (&v + 1 < &st.vars[0] + st.vars.size()) ? &v + 1 : nullptr;
+      if (next && next->vectorLane && t > 0) t = std::max<int64_t>(1, t / next->extent);
+      v.tile = (t <= 0 || t > v.extent) ? v.extent : t;
+      v.numTiles = ceilDiv(v.extent, v.tile);
+    }
+    // blocks: outermost shared parallel variables, x first
+    int axis = 0;
+    for (int i = 0; i < st.numParallel && i < k.sharedDepth && axis < static_cast<int>(o.grid.size()); ++i) {
+      LoopVar& v = st.vars[i];
+      if (v.vectorLane) continue;
+      v.blockAxis = axis;
+      v.gridExtent = std::min<int64_t>(static_cast<int64_t>(o.grid[axis]), v.numTiles);
+      gridUse[axis] = std::max(gridUse[axis], v.gridExtent);
+      ++axis;
+    }
+    // threads: innermost variables, x first
+    bool hasReduction = false;
+    for (const auto& s : st.stmts) hasReduction |= !s.redVars.empty();
+    st.threadReduction = o.generic.matchLibraryCallsValue && hasReduction && o.block[0] > 1;
+    int taxis = 0;
+    int nb = static_cast<int>(o.block.size());
+    if (st.threadReduction) {
+      for (int i = static_cast<int>(st.vars.size()) - 1; i >= st.numParallel; --i) {
+        if (!st.vars[i].vectorLane) {
+          st.vars[i].threadAxis = 0;
+          break;
+        }
+      }
+      taxis = 1;
+    }
+    for (int i = st.numParallel - 1; i >= 0 && taxis < nb; --i) {
+      if (st.vars[i].vectorLane) continue;
+      st.vars[i].threadAxis = taxis++;
+    }
+    for (auto& v : st.vars) {
+      if (v.threadAxis >= 0) {
+        blockUse[v.threadAxis] =
+            std::max(blockUse[v.threadAxis], std::min<int64_t>(static_cast<int64_t>(o.block[v.threadAxis]), v.tile));
+      }
+    }
+  }
+  k.block = blockUse;
+  k.grid = gridUse;
+  TC_CHECK_LE(k.block[0] * k.block[1] * k.block[2], limits.maxThreadsPerBlock)
+      << "thread block of " << k.block[0] << "x" << k.block[1] << "x" << k.block[2] << " exceeds the device limit";
+  int64_t budget = o.generic.hasUnroll ? static_cast<int64_t>(o.generic.unrollValue) : 1;
+  for (auto& st : k.stages) {
+    for (auto& v : st.vars) {
+      v.perThread = v.threadAxis >= 0 ? ceilDiv(v.tile, k.block[v.threadAxis]) : v.tile;
+    }
+    // register tile: innermost parallel variables first, while the tile fits the budget
+    int64_t prod = 1;
+    for (int i = st.numParallel - 1; i >= 0; --i) {
+      LoopVar& v = st.vars[i];
+      if (v.vectorLane || prod * v.perThread <= std::max<int64_t>(budget, 1) || v.perThread == 1) {
+        if (prod * v.perThread > 1024) break;
+        v.unrolled = true;
+        prod *= v.perThread;
+      } else {
+        break;
+      }
+    }
+    st.accCount = prod;
+  }
+}
+
+std::string kernelSignature(const ir::Function& f, const std::string& name, int64_t nt) {
+  std::ostringstream ss;
+  ss << "extern \"C\" __global__ void __launch_bounds__(" << nt << ") " << name << "(";
+  bool first = true;
+  for (const auto& p : f.params) {
+    ss << (first ? "" : ", ") << "int " << p.first;
+    first = false;
+  }
+  for (const auto& t : f.outputs) {
+    ss << (first ? "" : ", ") << t.type.cName() << "* __restrict__ p" << t.name;
+    first = false;
+  }
+  for (const auto& t : f.inputs) {
+    ss << (first ? "" : ", ") << "const " << t.type.cName() << "* __restrict__ p" << t.name;
+    first = false;
+  }
+  ss << ")";
+  return ss.str();
+}
+
+void emitKernel(KernelCtx& kc, const DeviceLimits& limits, Emitter& em) {
+  KernelPlan& k = kc.k;
+  std::vector<StageCodegen> gens;
+  gens.reserve(k.stages.size());
+  int64_t ldsBudget = limits.ldsBytesPerBlock;
+  if (kc.opts.hasMaxSharedMemory) ldsBudget = std::min<int64_t>(ldsBudget, kc.opts.maxSharedMemoryValue);
+  int64_t scratchElems = 0;
+  ScalarType scratchType;
+  for (auto& st : k.stages) {
+    if (st.threadReduction) {
+      int64_t bx = k.block[0], rows = k.block[1] * k.block[2];
+      int64_t e = ((bx & (bx - 1)) == 0 && bx <= 64) ? 1 : (bx % 64 == 0 ? (bx / 64) * rows : bx * rows);
+      scratchElems = std::max(scratchElems, e);
+      ScalarType t = st.views.at(st.tensor).type;
+      if (t.bytes() > scratchType.bytes() || scratchElems == e) scratchType = t;
+    }
+  }
+  ldsBudget -= scratchElems * 8;
+  int64_t before = ldsBudget;
+  for (size_t i = 0; i < k.stages.size(); ++i) {
+    gens.emplace_back(kc, k.stages[i], static_cast<int>(i), em);
+    gens.back().plan(ldsBudget);
+  }
+  k.ldsBytes = (before - ldsBudget) + scratchElems * 8;
+
+  em.open(kernelSignature(kc.f, k.name, kc.NT()));
+  for (const auto& p : kc.f.params) em.line("(void)" + p.first + ";");
+  em.line("const int tid_ = threadIdx.x + " + std::to_string(k.block[0]) + " * (threadIdx.y + " +
+          std::to_string(k.block[1]) + " * threadIdx.z);");
+  em.line("(void)tid_;");
+  if (scratchElems > 0) {
+    // one scratch area typed per use; sized for the widest element
+    em.line("__shared__ double red_scratch_raw_[" + std::to_string(scratchElems) + "];");
+  }
+  for (auto& g : gens) g.emitLdsDecls();
+  // kernel-level tile loops over the shared parallel variables (taken from the first stage)
+  int opened = 0;
+  const StagePlan& s0 = k.stages.front();
+  for (int i = 0; i < k.sharedDepth && i < s0.numParallel; ++i) {
+    const LoopVar& v = s0.vars[i];
+    if (v.vectorLane || v.numTiles == 1) continue;
+    std::string t = "t_" + v.name;
+    if (v.blockAxis >= 0) {
+      std::string b = std::string("blockIdx.") + axisName(v.blockAxis);
+      if (v.gridExtent == v.numTiles) {
+        em.line("const int " + t + " = " + b + ";");
+      } else {
+        em.open("for (int " + t + " = " + b + "; " + t + " < " + std::to_string(v.numTiles) + "; " + t + " += " +
+                std::to_string(v.gridExtent) + ")");
+        ++opened;
+      }
+    } else {
+      em.open("for (int " + t + " = 0; " + t + " < " + std::to_string(v.numTiles) + "; ++" + t + ")");
+      ++opened;
+    }
+  }
+  for (size_t i = 0; i < k.stages.size(); ++i) {
+    if (i > 0) em.line("__syncthreads();");
+    if (k.stages[i].threadReduction) {
+      em.open("");
+      em.line(k.stages[i].views.at(k.stages[i].tensor).type.cName() + "* red_scratch_ = (" +
+              k.stages[i].views.at(k.stages[i].tensor).type.cName() + "*)red_scratch_raw_;");
+      gens[i].emit();
+      em.close();
+    } else {
+      gens[i].emit();
+    }
+  }
+  if (k.stages.size() > 1 && opened > 0) em.line("__syncthreads();");
+  for (int i = 0; i < opened; ++i) em.close();
+  em.close();
+}
+
+} // namespace
+
+MappedProgram mapToHip(
+    const ir::Function& f,
+    const HipMappingOptions& options,
+    const std::string& specializedName,
+    const DeviceLimits& limits) {
+  for (const auto& t : f.outputs) {
+    for (auto m : t.mins) {
+      TC_CHECK_EQ(m, 0) << "output " << t.name << " has a non-zero inferred lower bound; not supported";
+    }
+  }
+  // 1. stages
+  std::vector<RawStage> raw;
+  bool allowStageFusion = options.generic.intraTileScheduleOptions.fusionStrategy != FusionStrategy::Min ||
+      options.generic.outerScheduleOptions.fusionStrategy != FusionStrategy::Min;
+  for (const auto& s : f.statements) {
+    for (const auto& subs : accessesTo(s, s.tensor)) {
+      TC_CHECK(isIdentityAccess(subs, s.lhsVars))
+          << "statement on " << s.tensor << " reads its own output at other points; not supported";
+    }
+    bool merged = false;
+    if (!raw.empty() && allowStageFusion && sameBox(raw.back().first(), s)) {
+      raw.back().stmts.push_back(&s);
+      merged = true;
+    }
+    if (!merged) {
+      RawStage r;
+      r.stmts.push_back(&s);
+      raw.push_back(r);
+    }
+  }
+  // 2. kernels
+  struct Group {
+    std::vector<size_t> stages;
+    int depth;
+  };
+  std::vector<Group> groups;
+  FusionStrategy fs = options.generic.outerScheduleOptions.fusionStrategy;
+  for (size_t i = 0; i < raw.size(); ++i) {
+    bool joined = false;
+    if (!groups.empty() && fs != FusionStrategy::Min) {
+      Group& g = groups.back();
+      int d = g.depth;
+      for (size_t j : g.stages) {
+        d = std::min(d, sharedPrefix(raw[j], raw[i]));
+      }
+      int need = 1;
+      if (fs == FusionStrategy::Preserve3Coincident) {
+        size_t rank = raw[i].first().lhsVars.size();
+        for (size_t j : g.stages) rank = std::min(rank, raw[j].first().lhsVars.size());
+        need = static_cast<int>(std::min<size_t>(3, rank));
+      }
+      if (d >= need && d >= 1) {
+        g.stages.push_back(i);
+        g.depth = d;
+        joined = true;
+      }
+    }
+    if (!joined) {
+      groups.push_back(Group{{i}, static_cast<int>(raw[i].first().lhsVars.size())});
+    }
+  }
+  // 3. plans
+  MappedProgram prog;
+  for (const auto& p : f.params) {
+    prog.paramNames.push_back(p.first);
+    prog.paramValues.push_back(p.second);
+  }
+  int64_t maxNumel = 0;
+  for (const auto& t : f.inputs) maxNumel = std::max(maxNumel, t.numel());
+  for (const auto& t : f.outputs) maxNumel = std::max(maxNumel, t.numel());
+  TC_CHECK_LT(maxNumel, (1LL << 31)) << "tensors with 2^31 or more elements are not supported yet";
+
+  bool anyThreadReduction = false;
+  std::vector<std::unique_ptr<Emitter>> bodies;
+  for (size_t gi = 0; gi < groups.size(); ++gi) {
+    KernelPlan k;
+    k.name = specializedName + (gi == 0 ? "" : "_k" + std::to_string(gi));
+    bool single = groups[gi].stages.size() == 1;
+    for (size_t si : groups[gi].stages) {
+      StageBuilder b(f);
+      b.init(raw[si]);
+      if (single && options.collapseContiguousValue) b.collapse();
+      k.stages.push_back(std::move(b.st));
+    }
+    k.sharedDepth = single ? k.stages[0].numParallel : groups[gi].depth;
+    // later stages of a fused kernel adopt the first stage's names for the shared variables;
+    // their other variables get a stage suffix so nothing can collide
+    for (size_t si = 1; si < k.stages.size(); ++si) {
+      StagePlan& st = k.stages[si];
+      std::map<std::string, std::string> ren;
+      for (size_t vi = 0; vi < st.vars.size(); ++vi) {
+        ren[st.vars[vi].name] = static_cast<int>(vi) < k.sharedDepth
+            ? k.stages[0].vars[vi].name
+            : st.vars[vi].name + "_s" + std::to_string(si);
+      }
+      auto sub = [&](const ExprRef& e) -> ExprRef {
+        return e->kind == Expr::Var ? mkVar(ren.at(e->name)) : nullptr;
+      };
+      for (auto& v : st.vars) v.name = ren.at(v.name);
+      for (auto& e : st.lhsSubs) e = rewrite(e, sub);
+      for (auto& ss : st.stmts) {
+        ss.rhs = rewrite(ss.rhs, sub);
+        for (auto& r : ss.redVars) r = ren.at(r);
+      }
+    }
+    // vector lanes on the variable that will sit on threadIdx.x
+    if (options.vectorWidthValue > 1) {
+      for (auto& st : k.stages) {
+        bool hasRed = false;
+        for (const auto& s : st.stmts) hasRed |= !s.redVars.empty();
+        bool threadRed = options.generic.matchLibraryCallsValue && hasRed && options.block[0] > 1;
+        std::string target;
+        if (threadRed) {
+          target = st.vars.back().name;
+        } else if (st.numParallel > 0) {
+          target = st.vars[st.numParallel - 1].name;
+        }
+        // the shared prefix must keep its shape in every stage
+        bool inPrefix = !threadRed && !single && st.numParallel - 1 < k.sharedDepth;
+        if (!target.empty() && !inPrefix) {
+          StageBuilder b(f);
+          b.st = std::move(st);
+          int before = b.st.numParallel;
+          b.splitLanes(target, options.vectorWidthValue);
+          if (single) k.sharedDepth += b.st.numParallel - before;
+          st = std::move(b.st);
+        }
+      }
+    }
+    prog.kernels.push_back(std::move(k));
+  }
+  std::ostringstream src;
+  for (auto& k : prog.kernels) {
+    KernelCtx kc{f, options, k};
+    mapKernel(kc, limits);
+    for (const auto& st : k.stages) anyThreadReduction |= st.threadReduction;
+    bodies.emplace_back(new Emitter());
+    emitKernel(kc, limits, *bodies.back());
+  }
+  src << "// generated by the TC HIP mapper for gfx950; function " << f.name << "\n";
+  src << hip::deviceLibrary(anyThreadReduction);
+  for (const auto& b : bodies) src << "\n" << b->out.str();
+  prog.source = src.str();
+  return prog;
+}
+
+} // namespace mapper
+} // namespace tc
