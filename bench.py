@@ -1,0 +1,142 @@
+#!/usr/bin/env python3
+"""Benchmark of the TC HIP backend on one MI355X.
+
+One "step" = one launch of the compiled TC over one batch of synthetic, seeded inputs that are
+already resident in HBM.  The headline workload is the HBM-bound tensordot
+O(n,c1,c3,h,w) +=! I0(n,c1,r_c2,h,w) * I1(n,r_c2,c3,h,w) at N=32, C1=512, C2=8, C3=2, H=W=28;
+`--config` selects another of the five workloads, `--all` appends their figures under "others".
+Prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+FP32_PEAK_TFLOPS = 157.3       # MI355X fp32 matrix/vector, published
+
+
+def flops(name, shapes):
+    if "tensordot" in name:
+        n, c1, c2, h, w = shapes[0]
+        c3 = shapes[1][2]
+        return 2 * n * c1 * c2 * c3 * h * w
+    if "batch_matmul" in name:
+        b, n, m = shapes[0]
+        return 2 * b * n * m * shapes[1][2]
+    if "group_convolution" in name:
+        n, g, c, h, w = shapes[0]
+        _, f, _, kh, kw = shapes[1]
+        oh, ow = h - kh + 1, w - kw + 1
+        return n * g * f * oh * ow * (2 * c * kh * kw + 1)
+    m, n = shapes[0]
+    return 6 * m * n
+
+
+def measure(name, steps, warmup, options=None):
+    import torch
+    import tensorcomprehensions_amd as tc
+    from tests import workloads as W
+
+    src, entry, shapes, _, _ = W.CONFIGS[name]
+    ins = [torch.from_numpy(a).cuda() for a in W.make_inputs(name)]
+    opts = options or W.TUNED[name]
+    ex = tc.compile(src, entry, ins, opts)
+    outs = tc.prepare_outputs(src, entry, ins)
+    for _ in range(warmup):
+        tc.unchecked_run(ex, ins, outs)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()                       # same stream the kernels are launched on
+    for _ in range(steps):
+        tc.unchecked_run(ex, ins, outs)
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    kernel_ms = start.elapsed_time(stop) / steps
+    nbytes = W.algorithmic_bytes(name)
+    return {
+        "name": name, "options": opts, "wall_s": wall, "kernel_ms": kernel_ms, "bytes": nbytes,
+        "flops": flops(name, shapes), "launch": [ex.launch_bounds(k) for k in range(ex.num_kernels)],
+        "ins": ins, "outs": outs,
+    }
+
+
+def roofline(m):
+    gbs = m["bytes"] / (m["kernel_ms"] * 1e-3) / 1e9
+    tfl = m["flops"] / (m["kernel_ms"] * 1e-3) / 1e12
+    if "group_convolution" in m["name"]:
+        return {"bound": "mfma", "achieved": round(tfl, 3), "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(tfl / FP32_PEAK_TFLOPS, 4), "traffic": None}
+    return {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}
+
+
+def cpu_baseline(name, budget_s=15.0):
+    """The oracle's sequential loop nest (-O3 -march=native, one core) on the same inputs."""
+    from oracle import tc_oracle
+    from tests import workloads as W
+    src, entry, _, _, _ = W.CONFIGS[name]
+    ins = W.make_inputs(name)
+    tc_oracle.run(src, entry, ins, native=True)          # build + first touch
+    times = []
+    t_all = time.perf_counter()
+    while len(times) < 5 and time.perf_counter() - t_all < budget_s:
+        t0 = time.perf_counter()
+        tc_oracle.run(src, entry, ins, native=True)
+        times.append(time.perf_counter() - t0)
+    med = sorted(times)[len(times) // 2]
+    return {"value": round(W.algorithmic_bytes(name) / med / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"full {name} workload, median of {len(times)} runs of the sequential loop nest, {med * 1e3:.1f} ms each"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--config", default="c2_tensordot")
+    ap.add_argument("--options", default=None)
+    ap.add_argument("--all", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py measures one GPU: this backend has no multi-GPU path (run with --gpus 1)")
+    import torch
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    from tests import workloads as W
+
+    m = measure(a.config, a.steps, a.warmup, a.options)
+    value = m["bytes"] * a.steps / m["wall_s"] / 1e9
+    line = {
+        "metric": "per-TC kernel GB/s or TFLOP/s on 1 MI355X and % of roofline",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(m["wall_s"] * 1e3 / a.steps, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": a.config, "shapes": [list(s) for s in W.CONFIGS[a.config][2]],
+                   "options": m["options"], "launch": m["launch"], "algorithmic_bytes": m["bytes"]},
+        "roofline": roofline(m),
+        "device": torch.cuda.get_device_name(0),
+    }
+    if not a.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(a.config)
+        line["cpu_baseline"]["host_cores"] = os.cpu_count()
+    if a.all:
+        others = {}
+        for name in W.CONFIGS:
+            if name == a.config:
+                continue
+            o = measure(name, a.steps, a.warmup)
+            others[name] = {"kernel_us": round(o["kernel_ms"] * 1e3, 3), "roofline": roofline(o),
+                            "gflops": round(o["flops"] / (o["kernel_ms"] * 1e-3) / 1e9, 1), "launch": o["launch"]}
+        line["others"] = others
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
