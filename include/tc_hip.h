@@ -50,6 +50,10 @@ typedef struct tc_executor tc_executor_t;
 const char* tc_last_error(void);
 void tc_free(void* p); /* frees strings returned through char** parameters */
 
+/* tc::CompilerOptions (tc/utils/compiler_options.h:27-37) used by the calling thread's next
+ * calls: print warnings to stderr / turn warnings into errors.  Defaults: 1, 0. */
+void tc_set_compiler_options(int emit_warnings, int throw_warnings);
+
 /* tc::inferOutputTensorInfo (tc/core/compiler.h:88-92; tc::aten::inferOutputTensorInfo,
  * tc/aten/aten_compiler.h:35-38).  Writes up to `capacity` entries, *count = number of outputs. */
 int tc_infer_output_info(

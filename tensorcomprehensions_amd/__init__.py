@@ -23,7 +23,7 @@ from .mapping_options import MappingOptions, FusionStrategy
 
 __all__ = [
     "compile", "prepare_outputs", "infer_output_tensor_info", "run", "profile", "unchecked_run", "autotune",
-    "map_only", "lang_dump", "ShapeOnly", "Executor", "MappingOptions", "FusionStrategy", "ProfilingInfo", "TcError",
+    "map_only", "lang_dump", "set_compiler_options", "ShapeOnly", "Executor", "MappingOptions", "FusionStrategy", "ProfilingInfo", "TcError",
 ]
 
 ProfilingInfo = namedtuple("ProfilingInfo", ["cpu_overhead_us", "kernel_runtime_us"])
@@ -180,6 +180,11 @@ def profile(executor, inputs, outputs):
     _capi.check(_capi.lib().tc_executor_profile(executor._h, pin.ptr, len(pin), pout.ptr, len(pout), _stream(),
                                                 ctypes.byref(k), ctypes.byref(c)))
     return ProfilingInfo(c.value, k.value)
+
+
+def set_compiler_options(emit_warnings=True, throw_warnings=False):
+    """tc::CompilerOptions for this thread's following calls."""
+    _capi.lib().tc_set_compiler_options(int(emit_warnings), int(throw_warnings))
 
 
 def map_only(tc, entry_point, inputs, options=None):

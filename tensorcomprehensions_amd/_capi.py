@@ -64,6 +64,8 @@ def _declare(l):
     l.tc_last_error.restype = ctypes.c_char_p
     l.tc_free.argtypes = [ctypes.c_void_p]
     l.tc_free.restype = None
+    l.tc_set_compiler_options.argtypes = [ctypes.c_int, ctypes.c_int]
+    l.tc_set_compiler_options.restype = None
     l.tc_infer_output_info.argtypes = [ctypes.c_char_p, ctypes.c_char_p, tensors, ctypes.c_int,
                                        P(TensorInfo), ctypes.c_int, P(ctypes.c_int)]
     l.tc_compile.argtypes = [ctypes.c_char_p, ctypes.c_char_p, tensors, ctypes.c_int, ctypes.c_char_p,

@@ -23,6 +23,7 @@ struct tc_executor {
 namespace tc {
 namespace capi {
 thread_local std::string lastError;
+thread_local tc::CompilerOptions compilerOptions;
 
 char* dupString(const std::string& s) {
   char* p = static_cast<char*>(std::malloc(s.size() + 1));
@@ -66,12 +67,16 @@ const char* tc_last_error(void) {
 void tc_free(void* p) {
   std::free(p);
 }
+void tc_set_compiler_options(int emitWarnings, int throwWarnings) {
+  compilerOptions.emitWarnings = emitWarnings != 0;
+  compilerOptions.throwWarnings = throwWarnings != 0;
+}
 
 int tc_infer_output_info(
     const char* tcText, const char* entry, const tc_dl_tensor* const* inputs, int numInputs,
     tc_tensor_info* outputs, int capacity, int* count) {
   TC_CAPI_BEGIN
-  auto infos = tc::inferOutputTensorInfo(tcText, entry, constTensors(inputs, numInputs));
+  auto infos = tc::inferOutputTensorInfo(tcText, entry, constTensors(inputs, numInputs), compilerOptions);
   *count = static_cast<int>(infos.size());
   for (int i = 0; i < *count && i < capacity; ++i) {
     const tc::TensorInfo& t = infos[i];
@@ -91,7 +96,7 @@ int tc_compile(
     const char* options, tc_executor_t** executor) {
   TC_CAPI_BEGIN
   auto opts = tc::HipMappingOptions::fromText(options ? options : "naive");
-  auto ex = tc::compile<tc::HipBackend>(tcText, entry, constTensors(inputs, numInputs), opts);
+  auto ex = tc::compile<tc::HipBackend>(tcText, entry, constTensors(inputs, numInputs), opts, compilerOptions);
   *executor = new tc_executor{std::move(ex)};
   TC_CAPI_END
 }
@@ -101,7 +106,7 @@ int tc_compile_serialized_options(
     const void* options, size_t optionsSize, tc_executor_t** executor) {
   TC_CAPI_BEGIN
   tc::HipMappingOptions opts(std::string(static_cast<const char*>(options), optionsSize));
-  auto ex = tc::compile<tc::HipBackend>(tcText, entry, constTensors(inputs, numInputs), opts);
+  auto ex = tc::compile<tc::HipBackend>(tcText, entry, constTensors(inputs, numInputs), opts, compilerOptions);
   *executor = new tc_executor{std::move(ex)};
   TC_CAPI_END
 }
@@ -211,7 +216,7 @@ int tc_map(
   auto it = defs.find(entry);
   TC_CHECK(it != defs.end()) << "attempting to access undefined function " << entry;
   auto in = constTensors(inputs, numInputs);
-  tc::ir::Function f = tc::detail::translate(it->second, in, tc::CompilerOptions());
+  tc::ir::Function f = tc::detail::translate(it->second, in, compilerOptions);
   tc::detail::checkInputsCompliant(f, in);
   auto r = tc::HipBackend::compileWithTcMapper(
       f.name, f, in, tc::HipMappingOptions::fromText(options ? options : "naive"));
@@ -245,8 +250,7 @@ int tc_lang_dump(const char* text, const char* what, char** out) {
   } else if (w == "function") {
     ss << lang::Parser(text).parseFunction();
   } else if (w == "sema" || w == "sema_env" || w == "sema+env") {
-    tc::CompilerOptions quiet;
-    lang::Sema sema(quiet);
+    lang::Sema sema(compilerOptions);
     lang::TreeRef r = sema.checkFunction(lang::Parser(text).parseFunction());
     if (w != "sema_env") ss << r;
     if (w != "sema") ss << sema.dumpEnv();

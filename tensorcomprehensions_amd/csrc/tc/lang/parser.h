@@ -81,7 +81,8 @@ class Parser {
       do {
         clauses.push_back(parseWhereClause());
       } while (L.nextIf(','));
-      where = makeList(clauses.front()->range(), std::move(clauses));
+      SourceRange whereRange = clauses.front()->range();
+      where = makeList(whereRange, std::move(clauses));
     } else {
       where = makeList(L.cur().range);
     }
