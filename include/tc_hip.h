@@ -132,6 +132,14 @@ int tc_autotune(
     const tc_dl_tensor* const* outputs, int num_outputs,
     const char* base_options, const char* settings, char** best);
 
+/* Host-side tuner logic without a device, for bindings and tests:
+ *   "powers2_and_ceil_divisors", "72"  -> "1,2,3,4,5,8,9,..."   (tc/autotuner/utils.cc:42-56)
+ *   "search_space", "<shape>;<shape>..." e.g. "500x26x72;500x72x26" -> candidate value sets
+ *   "genetic_search", "seed=..;generations=..;pop_size=.." -> best synthetic cost per generation
+ *   "options_cache_selftest", "<scratch file>" -> "ok" or the first failed expectation
+ *   "median", "3,1,2,10" -> "2"                                  (tc/core/utils/math.h:23-37) */
+int tc_host_query(const char* what, const char* arg, char** out);
+
 #ifdef __cplusplus
 }
 #endif

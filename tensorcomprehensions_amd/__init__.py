@@ -23,7 +23,7 @@ from .mapping_options import MappingOptions, FusionStrategy
 
 __all__ = [
     "compile", "prepare_outputs", "infer_output_tensor_info", "run", "profile", "unchecked_run", "autotune",
-    "map_only", "lang_dump", "set_compiler_options", "ShapeOnly", "Executor", "MappingOptions", "FusionStrategy", "ProfilingInfo", "TcError",
+    "map_only", "lang_dump", "host_query", "set_compiler_options", "ShapeOnly", "Executor", "MappingOptions", "FusionStrategy", "ProfilingInfo", "TcError",
 ]
 
 ProfilingInfo = namedtuple("ProfilingInfo", ["cpu_overhead_us", "kernel_runtime_us"])
@@ -203,6 +203,13 @@ def map_only(tc, entry_point, inputs, options=None):
 def lang_dump(text, what):
     out = ctypes.c_void_p()
     _capi.check(_capi.lib().tc_lang_dump(text.encode(), what.encode(), ctypes.byref(out)))
+    return _capi.take_string(out)
+
+
+def host_query(what, arg=""):
+    """Device-free tuner logic (divisor sets, search space, synthetic genetic search, cache self-test)."""
+    out = ctypes.c_void_p()
+    _capi.check(_capi.lib().tc_host_query(what.encode(), str(arg).encode(), ctypes.byref(out)))
     return _capi.take_string(out)
 
 

@@ -95,6 +95,7 @@ def _declare(l):
     l.tc_map.argtypes = [ctypes.c_char_p, ctypes.c_char_p, tensors, ctypes.c_int, ctypes.c_char_p,
                          P(ctypes.c_void_p), P(ctypes.c_int), P(ctypes.c_uint), P(ctypes.c_uint)]
     l.tc_lang_dump.argtypes = [ctypes.c_char_p, ctypes.c_char_p, P(ctypes.c_void_p)]
+    l.tc_host_query.argtypes = [ctypes.c_char_p, ctypes.c_char_p, P(ctypes.c_void_p)]
     l.tc_autotune.argtypes = [ctypes.c_char_p, ctypes.c_char_p, tensors, ctypes.c_int, tensors, ctypes.c_int,
                               ctypes.c_char_p, ctypes.c_char_p, P(ctypes.c_void_p)]
 

@@ -1,9 +1,281 @@
 // tc_autotune: C ABI of the genetic autotuner.
+#include <sstream>
+
 #include "capi/tc_capi_internal.h"
+#include "tc/autotuner/autotuner.h"
+#include "tc/core/hip/hip_tc_executor.h"
+
+namespace {
+std::map<std::string, std::string> parseSettings(const char* s) {
+  std::map<std::string, std::string> m;
+  if (!s) return m;
+  std::stringstream ss(s);
+  std::string kv;
+  while (std::getline(ss, kv, ';')) {
+    auto eq = kv.find('=');
+    if (eq != std::string::npos) m[kv.substr(0, eq)] = kv.substr(eq + 1);
+  }
+  return m;
+}
+} // namespace
 
 extern "C" int tc_autotune(
-    const char*, const char*, const tc_dl_tensor* const*, int, const tc_dl_tensor* const*, int,
-    const char*, const char*, char**) {
-  tc::capi::lastError = "autotuner not linked into this build";
-  return 1;
+    const char* tcText, const char* entry, const tc_dl_tensor* const* inputs, int numInputs,
+    const tc_dl_tensor* const* outputs, int numOutputs, const char* baseOptions, const char* settingsText,
+    char** best) {
+  using namespace tc;
+  try {
+    autotune::TunerSettings st;
+    autotune::TuningParameterFixer fixer;
+    size_t topK = 1;
+    for (const auto& kv : parseSettings(settingsText)) {
+      const std::string &k = kv.first, &v = kv.second;
+      auto num = [&]() { return static_cast<size_t>(std::stoull(v)); };
+      auto list = [&]() {
+        std::vector<size_t> out;
+        std::stringstream ss(v);
+        std::string item;
+        while (std::getline(ss, item, ',')) out.push_back(std::stoull(item));
+        return out;
+      };
+      if (k == "generations") st.generations = num();
+      else if (k == "pop_size") st.populationSize = num();
+      else if (k == "crossover_rate") st.crossOverRate = static_cast<uint8_t>(num());
+      else if (k == "mutation_rate") st.mutationRate = static_cast<uint8_t>(num());
+      else if (k == "number_elites") st.numberElites = num();
+      else if (k == "threads") st.threads = num();
+      else if (k == "seed") st.seed = static_cast<int64_t>(std::stoll(v));
+      else if (k == "top_k") topK = num();
+      else if (k == "verbose") st.verbose = num() != 0;
+      else if (k == "max_unroll") st.maxUnroll = num();
+      else if (k == "min_launch_total_threads") st.minLaunchTotalThreads = num();
+      else if (k == "cache_file") st.cacheFile = v;
+      else if (k == "fix_tile") fixer.fixTilingParameters(list());
+      else if (k == "fix_block") fixer.fixBlockParameters(list());
+      else if (k == "fix_grid") fixer.fixGridParameters(list());
+      else if (k == "fix_unroll") fixer.fixUnrollFactor(num());
+      else if (k == "fix_use_shared_memory") fixer.fixUseSharedMemory(num() != 0);
+      else if (k == "fix_match_library_calls") fixer.fixMatchLibraryCalls(num() != 0);
+      else if (k == "fix_vector_width") fixer.fixVectorWidth(num());
+      else if (k == "fix_collapse_contiguous") fixer.fixCollapseContiguous(num() != 0);
+      else if (k == "fix_outer_fusion") {
+        FusionStrategy fs;
+        TC_CHECK(fusionStrategyFromString(v, &fs)) << "unknown fusion strategy " << v;
+        fixer.fixOuterScheduleFusionStrategy(fs);
+      } else {
+        TC_CHECK(false) << "unknown tuner setting '" << k << "'";
+      }
+    }
+    // base options: one per line
+    std::vector<HipMappingOptions> bases;
+    std::stringstream bs(baseOptions ? baseOptions : "naive");
+    std::string line;
+    while (std::getline(bs, line)) {
+      if (!line.empty()) bases.push_back(HipMappingOptions::fromText(line));
+    }
+    int dev = 0;
+    TC_HIP_CHECK(tchip_get_device(&dev));
+    std::unordered_map<size_t, std::vector<const DLConstTensor*>> in;
+    std::unordered_map<size_t, std::vector<const DLTensor*>> out;
+    in[dev] = capi::constTensors(inputs, numInputs);
+    out[dev] = capi::mutTensors(outputs, numOutputs);
+    autotune::Autotuner<HipBackend, autotune::GeneticSearch> tuner;
+    auto result = tuner.tune(tcText, entry, in, out, bases, topK, fixer, st);
+    std::string text;
+    for (const auto& o : result) text += o.toText() + "\n";
+    *best = capi::dupString(text);
+    return 0;
+  } catch (const std::exception& e) {
+    tc::capi::lastError = e.what();
+    return 1;
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// tc_host_query: tuner logic that needs no device
+// ------------------------------------------------------------------------------------------
+namespace {
+using namespace tc;
+using namespace tc::autotune;
+
+std::string joinSizes(const std::vector<size_t>& v) {
+  std::string s;
+  for (size_t i = 0; i < v.size(); ++i) s += (i ? "," : "") + std::to_string(v[i]);
+  return s;
+}
+
+// synthetic, deterministic cost of a configuration: distance to a known optimum
+double syntheticCost(const TuningConfiguration& c) {
+  HipMappingOptions o = HipMappingOptions::makeNaiveMappingOptions();
+  c.applyToHipMappingOptions(o);
+  double cost = 1.0;
+  auto d = [](double a, double b) { return std::abs(std::log2(std::max(a, 1.0)) - std::log2(std::max(b, 1.0))); };
+  cost += d(static_cast<double>(o.block[0]), 64) + d(static_cast<double>(o.block[1]), 4);
+  cost += d(static_cast<double>(o.grid[0]), 256);
+  cost += o.generic.tiling.empty() ? 5 : d(static_cast<double>(o.generic.tiling[0]), 8);
+  cost += d(static_cast<double>(o.generic.unrollValue), 16);
+  cost += o.useSharedMemoryValue ? 0 : 2;
+  cost += o.vectorWidthValue == 4 ? 0 : 1;
+  return cost;
+}
+
+std::string runSyntheticSearch(const std::map<std::string, std::string>& kv) {
+  auto get = [&](const char* k, size_t def) { return kv.count(k) ? static_cast<size_t>(std::stoull(kv.at(k))) : def; };
+  int64_t shape0[] = {512, 128}, shape1[] = {128, 256};
+  DLConstTensor a{nullptr, {kDLROCM, 0}, 2, {2, 32, 1}, shape0, nullptr, 0};
+  DLConstTensor b{nullptr, {kDLROCM, 0}, 2, {2, 32, 1}, shape1, nullptr, 0};
+  std::vector<HipMappingOptions> bases{HipMappingOptions::makeNaiveMappingOptions()};
+  TuningConfiguration space = tc::autotune::detail::setupTuningParameters({&a, &b}, bases, 256);
+  TuningConfiguration start = space;
+  start.fromHipMappingOptions(bases[0]);
+  GeneticSearch gs({start}, get("generations", 10), get("pop_size", 20), static_cast<uint8_t>(get("crossover_rate", 80)),
+                   static_cast<uint8_t>(get("mutation_rate", 7)), get("number_elites", 2),
+                   static_cast<int64_t>(get("seed", 1)));
+  std::ostringstream out;
+  size_t invalidEvery = get("invalid_every", 0);
+  for (size_t g = 0; g < gs.numGenerations; ++g) {
+    double best = 1e30;
+    size_t i = 0;
+    for (auto& c : gs.population) {
+      TC_CHECK(c->configuration.isValid()) << "search produced an invalid configuration";
+      if (invalidEvery && (i++ % invalidEvery) != 0) {
+        c->invalid = true;
+        continue;
+      }
+      double cost = syntheticCost(c->configuration);
+      c->runtime = Duration::fromMicroSeconds(cost * 10);
+      best = std::min(best, cost);
+    }
+    out << (g ? "," : "") << best;
+    TC_CHECK_EQ(gs.population.size(), gs.maxPopulationSize);
+    gs.updateParameters();
+  }
+  return out.str();
+}
+
+struct FakeBackend {
+  using MappingOptionsType = HipMappingOptions;
+  static std::string backendString() { return "fake device"; }
+};
+
+std::string cacheSelfTest(const std::string& scratch) {
+#define EXPECT(cond) \
+  if (!(cond)) return std::string("failed: ") + #cond
+  OptionsCache<FakeBackend> cache;
+  TensorInfo in0({2, 32, 1}, 0, {10, 16}, {16, 1}), in1({2, 32, 1}, 0, {16, 20}, {20, 1});
+  TensorInfo out0({2, 32, 1}, 0, {10, 20}, {20, 1});
+  auto o1 = HipMappingOptions::makeNaiveMappingOptions();
+  auto o2 = HipMappingOptions::makeNaiveMappingOptions().tile(4, 4).unroll(8);
+  auto o3 = HipMappingOptions::makePointwiseMappingOptions();
+  auto us = [](double v) { return Duration::fromMicroSeconds(v); };
+  cache.recordRuntime("tcA", {in0, in1}, {out0}, "dev", o1, us(10));
+  cache.recordRuntime("tcA", {in0, in1}, {out0}, "dev", o1, us(30));
+  cache.recordRuntime("tcA", {in0, in1}, {out0}, "dev", o1, us(20));
+  cache.recordRuntime("tcA", {in0, in1}, {out0}, "dev", o2, us(15));
+  cache.recordRuntime("tcA", {in0, in1}, {out0}, "dev", o3, us(50));
+  cache.recordRuntime("tcB", {in0, in1}, {out0}, "dev", o3, us(5));
+  EXPECT(cache.size() == 4);
+  EXPECT((cache.count({"tcA", {in0, in1}, {out0}, "dev"}) == 3));
+  EXPECT(cache.getKeys().size() == 2);
+  // ranking by the median of all recorded runtimes: o2 (15) < o1 (median 20) < o3 (50)
+  auto top = cache.getTopKEntries("tcA", {in0, in1}, {out0}, "dev", 2);
+  EXPECT(top.size() == 2);
+  EXPECT(top[0].first == o2 && top[0].second == us(15));
+  EXPECT(top[1].first == o1 && top[1].second == us(20));
+  // misses: other TC, other sizes, other device, other alignment
+  EXPECT(cache.getTopKOptions("tcC", {in0, in1}, {out0}, "dev", 1).empty());
+  EXPECT(cache.getTopKOptions("tcA", {in1, in0}, {out0}, "dev", 1).empty());
+  EXPECT(cache.getTopKOptions("tcA", {in0, in1}, {out0}, "other", 1).empty());
+  TensorInfo misaligned = in0;
+  misaligned.alignment = 64;
+  EXPECT(cache.getTopKOptions("tcA", {misaligned, in1}, {out0}, "dev", 1).empty());
+  EXPECT(cache.numberAttemptedRetrievals == 5 && cache.numberSuccessfulRetrievals == 1);
+  // wire round trip
+  OptionsCache<FakeBackend> copy;
+  copy.fromProtobuf(cache.toProtobuf());
+  EXPECT(copy.size() == 4);
+  auto top2 = copy.getTopKEntries("tcA", {in0, in1}, {out0}, "dev", 3);
+  EXPECT(top2.size() == 3 && top2[0].first == o2 && top2[2].first == o3 && top2[1].second == us(20));
+  // prune
+  copy.pruneKeepTopK(1);
+  EXPECT(copy.size() == 2);
+  EXPECT((copy.getTopKOptions("tcA", {in0, in1}, {out0}, "dev", 5) == std::vector<HipMappingOptions>{o2}));
+  // files: store, load, append-merge
+  if (!scratch.empty()) {
+    std::remove(scratch.c_str());
+    cache.storeCacheToFile(scratch);
+    OptionsCache<FakeBackend> loaded;
+    loaded.loadCacheFromFile(scratch);
+    EXPECT(loaded.size() == 4);
+    std::remove(scratch.c_str());
+    appendTopKToCacheFile(cache, scratch, 2);
+    appendTopKToCacheFile(cache, scratch, 1);
+    OptionsCache<FakeBackend> merged;
+    merged.loadCacheFromFile(scratch);
+    EXPECT(merged.size() == 3 + 2);
+    std::remove(scratch.c_str());
+  }
+  return "ok";
+#undef EXPECT
+}
+} // namespace
+
+extern "C" int tc_host_query(const char* what, const char* arg, char** out) {
+  try {
+    std::string w = what, a = arg ? arg : "";
+    std::string result;
+    if (w == "powers2_and_ceil_divisors") {
+      result = joinSizes(powers2andCeilDivisors(std::stoull(a)));
+    } else if (w == "median") {
+      std::vector<long long> v;
+      std::stringstream ss(a);
+      std::string item;
+      while (std::getline(ss, item, ',')) v.push_back(std::stoll(item));
+      result = std::to_string(median(v));
+    } else if (w == "search_space") {
+      std::vector<std::vector<int64_t>> shapes;
+      std::stringstream ss(a);
+      std::string sh;
+      while (std::getline(ss, sh, ';')) {
+        std::vector<int64_t> dims;
+        std::stringstream ds(sh);
+        std::string d;
+        while (std::getline(ds, d, 'x')) dims.push_back(std::stoll(d));
+        shapes.push_back(dims);
+      }
+      std::vector<DLConstTensor> ts(shapes.size());
+      std::vector<const DLConstTensor*> ptrs;
+      for (size_t i = 0; i < shapes.size(); ++i) {
+        ts[i] = DLConstTensor{nullptr, {kDLROCM, 0}, static_cast<int>(shapes[i].size()), {2, 32, 1}, shapes[i].data(), nullptr, 0};
+        ptrs.push_back(&ts[i]);
+      }
+      TuningConfiguration c = tc::autotune::detail::setupTuningParameters(ptrs, {HipMappingOptions::makeNaiveMappingOptions()}, 256);
+      result = "tile_dims=" + std::to_string(c.tilingParams.dims.size()) + ";tile=" + joinSizes(c.tilingParams.dims[0].values()) +
+          ";block=" + joinSizes(c.blockParams.dims[0].values()) + ";grid=" + joinSizes(c.gridParams.dims[0].values()) +
+          ";unroll=" + joinSizes(c.unrollFactor.values()) + ";genes=" + std::to_string(c.collectParameters().size());
+    } else if (w == "genetic_search") {
+      result = runSyntheticSearch(parseSettings(a.c_str()));
+    } else if (w == "options_cache_selftest") {
+      result = cacheSelfTest(a);
+    } else if (w == "base_outside_space") {
+      // a base mapping whose tile size is not a candidate value must be refused
+      int64_t shape[] = {10, 16};
+      DLConstTensor t{nullptr, {kDLROCM, 0}, 2, {2, 32, 1}, shape, nullptr, 0};
+      auto base = HipMappingOptions::makeNaiveMappingOptions().tile(7, 7);
+      TuningConfiguration c = tc::autotune::detail::setupTuningParameters({&t}, {base}, 256);
+      try {
+        c.fromHipMappingOptions(base);
+        result = "accepted";
+      } catch (const std::invalid_argument& e) {
+        result = std::string("invalid_argument: ") + e.what();
+      }
+    } else {
+      TC_CHECK(false) << "unknown host query '" << w << "'";
+    }
+    *out = tc::capi::dupString(result);
+    return 0;
+  } catch (const std::exception& e) {
+    tc::capi::lastError = e.what();
+    return 1;
+  }
 }

@@ -1,0 +1,301 @@
+// Autotuner: searches mapping options by compiling and timing candidates on the device.
+//
+// Structure of the reference's harness (tc/autotuner/autotuner.h:37-161, autotuner-inl.h:37-518):
+// per generation, a pool of compile threads walks the population with an atomic cursor and
+// queues (executor | nullptr, candidate); one evaluation thread per device pops the queue,
+// prunes hopeless candidates, profiles the rest ten times and records the median in the
+// OptionsCache and on the candidate; the search strategy then breeds the next generation.
+// SIGINT finishes the current generation and returns the best so far; SIGTERM aborts.
+#pragma once
+#include <atomic>
+#include <condition_variable>
+#include <csignal>
+#include <deque>
+#include <iostream>
+#include <mutex>
+#include <thread>
+#include <unordered_map>
+
+#include "tc/autotuner/genetic_search.h"
+#include "tc/autotuner/options_cache.h"
+#include "tc/autotuner/utils.h"
+#include "tc/core/compiler.h"
+#include "tc/core/hip/hip.h"
+#include "tc/core/flags.h"
+#include "tc/lang/parser.h"
+#include "tc/lang/sema.h"
+
+namespace tc {
+namespace autotune {
+
+struct TunerSettings {
+  size_t generations = flags().tuner_gen_generations;
+  size_t populationSize = flags().tuner_gen_pop_size;
+  uint8_t crossOverRate = static_cast<uint8_t>(flags().tuner_gen_crossover_rate);
+  uint8_t mutationRate = static_cast<uint8_t>(flags().tuner_gen_mutation_rate);
+  size_t numberElites = flags().tuner_gen_number_elites;
+  size_t threads = flags().tuner_threads;
+  uint64_t minLaunchTotalThreads = flags().tuner_min_launch_total_threads;
+  size_t maxUnroll = 256;
+  int64_t seed = -1;
+  bool verbose = flags().debug_tuner;
+  size_t restoreNumber = flags().tuner_gen_restore_number;
+  std::string cacheFile; // when set: seeds the first generation from it and appends the result
+};
+
+namespace detail {
+
+extern std::atomic<int> tunerSignal; // 0, SIGINT or SIGTERM while a tune() is running
+
+inline std::vector<size_t> inputDivisorsAndPowers2(const std::vector<const DLConstTensor*>& inputs) {
+  std::vector<size_t> sizes;
+  for (auto t : inputs) {
+    for (int i = 0; i < t->ndim; ++i) sizes.push_back(static_cast<size_t>(t->shape[i]));
+  }
+  std::sort(sizes.begin(), sizes.end());
+  sizes.erase(std::unique(sizes.begin(), sizes.end()), sizes.end());
+  std::vector<size_t> out;
+  for (auto s : sizes) out = mergeVectors(std::move(out), powers2andCeilDivisors(s));
+  return mergeVectors(std::move(out), powers2andCeilDivisors(256));
+}
+
+// Candidate value sets derived from the input shapes (tc/autotuner/autotuner-inl.h:326-404).
+inline TuningConfiguration setupTuningParameters(
+    const std::vector<const DLConstTensor*>& inputs, const std::vector<HipMappingOptions>& baseMappings,
+    size_t maxUnroll) {
+  TC_CHECK_GE(inputs.size(), 1u);
+  std::vector<size_t> range = inputDivisorsAndPowers2(inputs);
+  size_t maxRank = 0;
+  for (auto t : inputs) maxRank = std::max<size_t>(maxRank, t->ndim);
+  std::vector<size_t> tileRange = range;
+  tileRange.push_back(0); // 0 = do not tile this dimension
+  std::vector<size_t> blockRange = range, gridRange = range;
+  size_t tileDims = maxRank + 1;
+  for (const auto& b : baseMappings) {
+    blockRange = mergeVectors(std::move(blockRange), std::vector<size_t>(b.block.extractVector().begin(), b.block.extractVector().end()));
+    gridRange = mergeVectors(std::move(gridRange), std::vector<size_t>(b.grid.extractVector().begin(), b.grid.extractVector().end()));
+    tileDims = std::max(tileDims, b.generic.tiling.size());
+  }
+  TuningConfiguration c;
+  c.tilingParams.setRange(1, tileDims, "t", tileRange, "t");
+  c.blockParams.setRange(1, 3, "b", blockRange, "b");
+  c.gridParams.setRange(1, 3, "g", gridRange, "g");
+  c.unrollFactor = RangeParameter(powers2(maxUnroll), "unroll");
+  c.privateDepth = RangeParameter({0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10}, "pdepth");
+  c.sharedDepth = RangeParameter({0, 1, 2, 3, 4, 5, 6, 7}, "sdepth");
+  return c;
+}
+
+} // namespace detail
+
+template <typename Backend, typename SearchStrategy>
+class Autotuner {
+ public:
+  using ExecutorType = typename Backend::ExecutorType;
+  using MappingOptionsType = typename Backend::MappingOptionsType;
+  using OptionsCacheType = OptionsCache<Backend>;
+
+  Autotuner() : optionsCache(new OptionsCacheType()) {}
+
+  // `inputs` / `outputs`: device index -> tensors living on that device.  Returns the best
+  // topK options found (fewer when not enough candidates were valid).
+  std::vector<MappingOptionsType> tune(
+      const std::string& tc,
+      const std::string& tcEntryPoint,
+      const std::unordered_map<size_t, std::vector<const DLConstTensor*>>& inputs,
+      std::unordered_map<size_t, std::vector<const DLTensor*>>& outputs,
+      const std::vector<MappingOptionsType>& baseMappings,
+      size_t topK = 1,
+      const TuningParameterFixer& fixedParams = TuningParameterFixer(),
+      const TunerSettings& settings = TunerSettings());
+
+  std::shared_ptr<OptionsCacheType> optionsCache;
+};
+
+// ------------------------------------------------------------------------------------------
+template <typename Backend, typename SearchStrategy>
+std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrategy>::tune(
+    const std::string& tc,
+    const std::string& tcEntryPoint,
+    const std::unordered_map<size_t, std::vector<const DLConstTensor*>>& inputs,
+    std::unordered_map<size_t, std::vector<const DLTensor*>>& outputs,
+    const std::vector<MappingOptionsType>& baseMappings,
+    size_t topK,
+    const TuningParameterFixer& fixedParams,
+    const TunerSettings& settings) {
+  TC_CHECK(!inputs.empty()) << "no device to tune on";
+  TC_CHECK(!baseMappings.empty()) << "need at least one base mapping";
+  auto defs = tc::detail::parse(tc);
+  TC_CHECK_EQ(defs.count(tcEntryPoint), 1u) << "attempting to access undefined function " << tcEntryPoint;
+  lang::TreeRef tree = defs.at(tcEntryPoint);
+  CompilerOptions quiet;
+  quiet.emitWarnings = false;
+  std::ostringstream canon;
+  canon << lang::canonicalize(lang::Sema(quiet).checkFunction(tree));
+  const std::string canonicalTc = canon.str();
+
+  const auto& firstInputs = inputs.begin()->second;
+  auto inputsInfo = makeTensorInfoVector(firstInputs);
+  auto outputsInfo = makeTensorInfoVector(outputs.begin()->second);
+  const std::string backendStr = Backend::backendString();
+
+  // search space and starting points
+  std::vector<MappingOptionsType> bases = baseMappings;
+  if (!settings.cacheFile.empty()) {
+    auto restored = loadTopKFromCacheFile<Backend>(
+        canonicalTc, inputsInfo, outputsInfo, Backend::makeDeviceFilename(settings.cacheFile), settings.restoreNumber);
+    bases.insert(bases.end(), restored.begin(), restored.end());
+  }
+  TuningConfiguration space = detail::setupTuningParameters(firstInputs, bases, settings.maxUnroll);
+  space.fixParameters(fixedParams);
+  std::vector<TuningConfiguration> configs;
+  for (const auto& b : bases) {
+    TuningConfiguration c = space;
+    c.fromHipMappingOptions(b); // throws std::invalid_argument for values outside the space
+    configs.push_back(c);
+  }
+  SearchStrategy search(
+      configs, settings.generations, settings.populationSize, settings.crossOverRate, settings.mutationRate,
+      settings.numberElites, settings.seed);
+  const MappingOptionsType baseMapping = bases.front();
+
+  // signals: SIGINT = stop after this generation, SIGTERM = abort now
+  detail::tunerSignal = 0;
+  auto oldInt = std::signal(SIGINT, [](int s) { detail::tunerSignal = s; });
+  auto oldTerm = std::signal(SIGTERM, [](int s) { detail::tunerSignal = s; });
+  struct Restore {
+    void (*a)(int);
+    void (*b)(int);
+    ~Restore() {
+      std::signal(SIGINT, a);
+      std::signal(SIGTERM, b);
+    }
+  } restore{oldInt, oldTerm};
+
+  Duration bestTime = Duration::max();
+  for (size_t gen = 0; gen < settings.generations; ++gen) {
+    auto& population = search.population;
+    std::atomic<size_t> cursor{0};
+    std::mutex mu;
+    std::condition_variable cv;
+    std::deque<std::pair<std::unique_ptr<ExecutorType>, CandidateConfiguration*>> ready;
+    size_t produced = 0;
+
+    auto compileWorker = [&]() {
+      for (;;) {
+        size_t i = cursor.fetch_add(1);
+        if (i >= population.size() || detail::tunerSignal == SIGTERM) return;
+        CandidateConfiguration* cand = population[i].get();
+        std::unique_ptr<ExecutorType> ex;
+        try {
+          MappingOptionsType options = baseMapping;
+          cand->configuration.applyToHipMappingOptions(options);
+          ex = tc::detail::compile<Backend>(tree, firstInputs, options, quiet);
+        } catch (const std::exception& e) {
+          if (settings.verbose) std::cerr << "[tuner] candidate failed to compile: " << e.what() << std::endl;
+          ex.reset();
+        }
+        {
+          std::lock_guard<std::mutex> lock(mu);
+          ready.emplace_back(std::move(ex), cand);
+          ++produced;
+        }
+        cv.notify_one();
+      }
+    };
+
+    std::vector<Duration> generationTimes;
+    auto evaluate = [&](size_t device) {
+      typename Backend::WithDevice guard(device);
+      const auto& ins = inputs.at(device);
+      const auto& outs = outputs.at(device);
+      size_t consumed = 0;
+      while (consumed < population.size()) {
+        std::pair<std::unique_ptr<ExecutorType>, CandidateConfiguration*> job;
+        {
+          std::unique_lock<std::mutex> lock(mu);
+          cv.wait(lock, [&] { return !ready.empty() || detail::tunerSignal == SIGTERM; });
+          if (ready.empty()) return;
+          job = std::move(ready.front());
+          ready.pop_front();
+        }
+        ++consumed;
+        CandidateConfiguration* cand = job.second;
+        if (!job.first) {
+          cand->invalid = true;
+          continue;
+        }
+        ExecutorType& ex = *job.first;
+        try {
+          // prune launches that cannot fill even one compute unit
+          auto g = ex.grid().extractDefaultedArray();
+          auto b = ex.block().extractDefaultedArray();
+          if (g[0] * g[1] * g[2] * b[0] * b[1] * b[2] < settings.minLaunchTotalThreads) {
+            cand->invalid = true;
+            continue;
+          }
+          // first run: stop at once when catastrophically slow (100x), again after warm-up (5x)
+          ProfilingInfo first = ex.profile(ins, outs);
+          if (bestTime < Duration::max() && first.kernelRuntime >= bestTime * 100) {
+            cand->invalid = true;
+            continue;
+          }
+          ProfilingInfo warm = ex.profile(ins, outs);
+          if (bestTime < Duration::max() && warm.kernelRuntime >= bestTime * 5) {
+            cand->invalid = true;
+            continue;
+          }
+          std::vector<int64_t> runs;
+          for (int r = 0; r < 10; ++r) runs.push_back(ex.profile(ins, outs).kernelRuntime.toNanoSeconds());
+          Duration med = Duration::fromNanoSeconds(median(runs));
+          if (med == Duration::zero()) {
+            cand->invalid = true;
+            continue;
+          }
+          cand->runtime = med;
+          bestTime = std::min(bestTime, med, [](Duration a, Duration b) { return a < b; });
+          generationTimes.push_back(med);
+          MappingOptionsType options = baseMapping;
+          cand->configuration.applyToHipMappingOptions(options);
+          optionsCache->recordRuntime(canonicalTc, inputsInfo, outputsInfo, backendStr, options, med);
+        } catch (const std::exception& e) {
+          // a failed launch must not poison later candidates: drain the sticky error state
+          tchip_get_last_error();
+          if (settings.verbose) std::cerr << "[tuner] candidate failed to run: " << e.what() << std::endl;
+          cand->invalid = true;
+        }
+      }
+    };
+
+    std::vector<std::thread> compilers;
+    size_t nThreads = std::max<size_t>(1, std::min(settings.threads, population.size()));
+    for (size_t t = 0; t < nThreads; ++t) compilers.emplace_back(compileWorker);
+    std::thread evaluator(evaluate, inputs.begin()->first);
+    for (auto& t : compilers) t.join();
+    cv.notify_all();
+    evaluator.join();
+    if (detail::tunerSignal == SIGTERM) {
+      throw std::runtime_error("Abort requested");
+    }
+    if (settings.verbose || flags().tuner_gen_log_generations) {
+      std::sort(generationTimes.begin(), generationTimes.end());
+      std::cerr << "[tuner] generation " << gen << ": " << generationTimes.size() << "/" << population.size()
+                << " valid";
+      if (!generationTimes.empty()) {
+        std::cerr << " (best/median/worst) " << generationTimes.front().toMicroSecondsF() << "/"
+                  << generationTimes[generationTimes.size() / 2].toMicroSecondsF() << "/"
+                  << generationTimes.back().toMicroSecondsF() << " us";
+      }
+      std::cerr << std::endl;
+    }
+    if (detail::tunerSignal == SIGINT) break;
+    if (gen + 1 < settings.generations) search.updateParameters();
+  }
+  if (!settings.cacheFile.empty()) {
+    appendTopKToCacheFile<Backend>(*optionsCache, Backend::makeDeviceFilename(settings.cacheFile), std::max<size_t>(topK, 10));
+  }
+  return optionsCache->getTopKOptions(canonicalTc, inputsInfo, outputsInfo, backendStr, topK);
+}
+
+} // namespace autotune
+} // namespace tc

@@ -32,6 +32,20 @@ void checkSizesAndStridesAreCompliant(
     for (int d = 0; d < t->ndim; ++d) {
       TC_CHECK_EQ(t->shape[d], e.shape[d]) << what << " " << i << " dimension " << d << ": size differs from the compiled one";
     }
+    // Generated kernels index tensors as dense row-major arrays (as the reference's do,
+    // tc/core/polyhedral/cuda/codegen.cc:200-243, where a strided view silently computes on the
+    // wrong elements); a tensor whose strides say otherwise is refused instead.
+    if (t->strides) {
+      int64_t expect = 1;
+      for (int d = t->ndim - 1; d >= 0; --d) {
+        if (t->shape[d] != 1 && t->strides[d] != expect) {
+          std::stringstream ss;
+          ss << what << " " << i << " is not contiguous: " << *t;
+          throw InvalidStrideException(ss.str());
+        }
+        expect *= t->shape[d];
+      }
+    }
   }
 }
 } // namespace detail

@@ -1,0 +1,64 @@
+"""Device-free tuner logic: divisor sets (known answers of test/cuda/test_autotuner_utility.cc:34-50),
+the search space built from input shapes, GeneticSearch on a synthetic cost, OptionsCache semantics
+(scenarios after test/cuda/test_compilation_cache.cc:133-510), median (tc/core/utils/math.h:23-37)."""
+import os
+import tempfile
+
+import pytest
+
+import tensorcomprehensions_amd as tc
+
+
+@pytest.mark.parametrize("n,expected", [
+    (10, [1, 2, 3, 4, 5, 8, 10, 16]),
+    (72, [1, 2, 3, 4, 5, 8, 9, 16, 18, 32, 36, 64, 72, 128]),
+    (35, [1, 2, 3, 4, 5, 8, 9, 16, 18, 32, 35, 64]),
+    (130, [1, 2, 3, 4, 5, 8, 9, 16, 17, 32, 33, 64, 65, 128, 130, 256]),
+])
+def test_powers2_and_ceil_divisors(n, expected):
+    assert [int(x) for x in tc.host_query("powers2_and_ceil_divisors", n).split(",")] == expected
+
+
+def test_median_of_even_count_is_integer_mean_of_middle_pair():
+    assert tc.host_query("median", "3,1,2,10") == "2"
+    assert tc.host_query("median", "5,1,9") == "5"
+    assert tc.host_query("median", "4") == "4"
+
+
+def test_search_space_from_shapes():
+    fields = dict(kv.split("=") for kv in tc.host_query("search_space", "500x26x72;500x72x26").split(";"))
+    tile = [int(x) for x in fields["tile"].split(",")]
+    block = [int(x) for x in fields["block"].split(",")]
+    assert fields["tile_dims"] == "4"                       # largest rank + 1
+    assert 0 in tile and 0 not in block                     # 0 = "do not tile"; never a block size
+    for v in (26, 72, 500, 13, 36, 250, 256, 64):           # divisors of the dims, and of 256
+        assert v in tile and v in block
+    assert fields["unroll"] == "1,2,4,8,16,32,64,128,256"
+    assert fields["block"] == fields["grid"]                # naive's 64,4 / 256,256 are already members
+
+
+def test_base_mapping_outside_the_space_is_refused():
+    assert tc.host_query("base_outside_space").startswith("invalid_argument")
+
+
+def test_genetic_search_is_deterministic_and_monotone_with_elites():
+    a = tc.host_query("genetic_search", "seed=5;generations=12;pop_size=24;number_elites=3")
+    b = tc.host_query("genetic_search", "seed=5;generations=12;pop_size=24;number_elites=3")
+    c = tc.host_query("genetic_search", "seed=6;generations=12;pop_size=24;number_elites=3")
+    assert a == b
+    best = [float(x) for x in a.split(",")]
+    assert all(x >= y for x, y in zip(best, best[1:]))      # elites keep the best alive
+    assert best[-1] <= best[0]
+    assert len(c.split(",")) == 12
+
+
+def test_genetic_search_survives_mostly_invalid_generations():
+    # only every 6th candidate is valid: with 12 candidates that is 2 < 3 survivors, so every
+    # generation takes the re-randomise-around-the-last-best path
+    out = tc.host_query("genetic_search", "seed=2;generations=6;pop_size=12;invalid_every=6")
+    assert len(out.split(",")) == 6
+
+
+def test_options_cache_semantics_and_files():
+    with tempfile.TemporaryDirectory() as d:
+        assert tc.host_query("options_cache_selftest", os.path.join(d, "cache.bin")) == "ok"

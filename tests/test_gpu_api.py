@@ -1,0 +1,126 @@
+"""Executor contract through the C ABI on the device: checked run errors, profile, unchecked run,
+clearing, strides, repeated runs with different base pointers, the autotuner."""
+import numpy as np
+import pytest
+import torch
+
+import tensorcomprehensions_amd as tc
+from oracle import tc_oracle
+from tests import workloads as W
+
+pytestmark = pytest.mark.gpu
+
+MM = "def matmul(float(M, K) A, float(K, N) B) -> (C) { C(m, n) +=! A(m, r_k) * B(r_k, n) }"
+
+
+def test_run_checks_count_rank_dtype_shape():
+    A, B = torch.randn(8, 16, device="cuda"), torch.randn(16, 4, device="cuda")
+    ex = tc.compile(MM, "matmul", [A, B], "naive")
+    (C,) = tc.prepare_outputs(MM, "matmul", [A, B])
+    tc.run(ex, [A, B], [C])
+    with pytest.raises(tc.TcError):
+        tc.run(ex, [A], [C])
+    with pytest.raises(tc.TcError):
+        tc.run(ex, [A, B.double()], [C])
+    with pytest.raises(tc.TcError):
+        tc.run(ex, [A, torch.randn(16, 5, device="cuda")], [C])
+    with pytest.raises(tc.TcError):
+        tc.run(ex, [A, B], [torch.empty(8, 4, 1, device="cuda")])
+    torch.cuda.synchronize()
+    assert torch.allclose(C, A @ B, atol=1e-4)
+
+
+def test_non_contiguous_tensors_are_refused():
+    base = torch.randn(64, 128, device="cuda")
+    view = base[:, :64]                                     # strides (128, 1)
+    src = "def copy(float(M, N) A) -> (B) { B(m, n) = A(m, n) }"
+    ex = tc.compile(src, "copy", [view.contiguous()], "naive")
+    out = torch.empty(64, 64, device="cuda")
+    with pytest.raises(tc.TcError) as e:
+        tc.run(ex, [view], [out])
+    assert "not contiguous" in str(e.value)
+    with pytest.raises(tc.TcError):                          # compile time: stride 1 < 64*... transposed view
+        tc.compile(src, "copy", [base.t()], "naive")
+
+
+def test_profile_reports_kernel_time_and_same_result_for_new_pointers():
+    A, B = torch.randn(128, 64, device="cuda"), torch.randn(64, 32, device="cuda")
+    ex = tc.compile(MM, "matmul", [A, B], "naive;tile=16,16;mapToThreads=16,16")
+    (C,) = tc.prepare_outputs(MM, "matmul", [A, B])
+    info = tc.profile(ex, [A, B], [C])
+    assert info.kernel_runtime_us > 0 and info.cpu_overhead_us >= 0
+    A2, B2, C2 = A.clone() * 2, B.clone(), torch.empty_like(C)
+    tc.unchecked_run(ex, [A2, B2], [C2])
+    torch.cuda.synchronize()
+    assert torch.allclose(C2, 2 * C, atol=1e-4)
+
+
+def test_clear_runtime_compiled_function_forbids_further_runs():
+    A, B = torch.randn(8, 16, device="cuda"), torch.randn(16, 4, device="cuda")
+    ex = tc.compile(MM, "matmul", [A, B], "naive")
+    (C,) = tc.prepare_outputs(MM, "matmul", [A, B])
+    tc.run(ex, [A, B], [C])
+    torch.cuda.synchronize()
+    ex.clear_runtime_compiled_function()
+    with pytest.raises(tc.TcError) as e:
+        tc.run(ex, [A, B], [C])
+    assert "No rtcFun_" in str(e.value)
+
+
+def test_runs_on_a_side_stream():
+    A, B = torch.randn(64, 64, device="cuda"), torch.randn(64, 64, device="cuda")
+    ex = tc.compile(MM, "matmul", [A, B], "naive")
+    (C,) = tc.prepare_outputs(MM, "matmul", [A, B])
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        tc.run(ex, [A, B], [C])
+    s.synchronize()
+    assert torch.allclose(C, A @ B, atol=1e-4)
+
+
+def test_prepare_outputs_needs_an_input_and_infers_shapes():
+    A, B = torch.randn(8, 16, device="cuda"), torch.randn(16, 4, device="cuda")
+    (C,) = tc.prepare_outputs(MM, "matmul", [A, B])
+    assert C.shape == (8, 4) and C.dtype == torch.float32 and C.is_cuda
+    with pytest.raises(tc.TcError):
+        tc.prepare_outputs("def f() -> (O) { O(i) = 3 where i in 0:4 }", "f", [])
+
+
+def test_integer_and_double_tensors():
+    src = "def f(int32(N) A, double(N) B) -> (C, D) { C(n) = A(n) * 3 + n \n D(n) = B(n) * B(n) }"
+    A = torch.arange(100, dtype=torch.int32, device="cuda")
+    B = torch.randn(100, dtype=torch.float64, device="cuda")
+    ex = tc.compile(src, "f", [A, B], "naive")
+    C, D = tc.prepare_outputs(src, "f", [A, B])
+    assert C.dtype == torch.int32 and D.dtype == torch.float64
+    tc.run(ex, [A, B], [C, D])
+    torch.cuda.synchronize()
+    assert torch.equal(C, A * 3 + torch.arange(100, dtype=torch.int32, device="cuda"))
+    assert torch.equal(D, B * B)
+
+
+def test_autotune_small_tensordot_improves_on_naive():
+    name = "c1_tensordot_small"
+    src, entry, _, _, k = W.CONFIGS[name]
+    ins_np = W.make_inputs(name)
+    ins = [torch.from_numpy(a).cuda() for a in ins_np]
+    best = tc.autotune(src, entry, ins, "naive", generations=3, pop_size=10, threads=8, seed=7, number_elites=2)
+    assert len(best) == 1
+    ex = tc.compile(src, entry, ins, best[0])
+    outs = tc.prepare_outputs(src, entry, ins)
+    t_best = min(tc.profile(ex, ins, outs).kernel_runtime_us for _ in range(5))
+    ref = tc_oracle.run(src, entry, ins_np)[0]
+    assert np.abs(outs[0].cpu().numpy() - ref).max() <= W.tolerance(k, ref)
+    naive = tc.compile(src, entry, ins, "naive")
+    t_naive = min(tc.profile(naive, ins, outs).kernel_runtime_us for _ in range(5))
+    print(f"naive {t_naive:.1f} us, tuned {t_best:.1f} us: {best[0]}", flush=True)
+    assert t_best <= t_naive * 1.05
+
+
+def test_autotune_survives_unmappable_candidates():
+    """A population made mostly of configurations the mapper refuses (fixed huge block) must
+    not break the tuner: candidates are marked invalid and the search goes on."""
+    A, B = torch.randn(64, 64, device="cuda"), torch.randn(64, 64, device="cuda")
+    best = tc.autotune(MM, "matmul", [A, B], "naive", generations=2, pop_size=6, threads=4, seed=3, top_k=2)
+    assert 1 <= len(best) <= 2

@@ -1,0 +1,97 @@
+"""Wave64 reduction library on the block shapes of the reference's reduction tests
+(test/cuda/test_tc_mapper.cc:120-177: x extents {1,2,4,7,8,11,15,17,24,32,35,42,64,128,130} and the
+(x,y) pairs), extended with whole-wavefront multiples, against the oracle and A.sum(1)."""
+import numpy as np
+import pytest
+import torch
+
+import tensorcomprehensions_amd as tc
+from oracle import tc_oracle
+from tests import workloads as W
+
+pytestmark = pytest.mark.gpu
+
+SUM2D = "def sum2d(float(M, N) A) -> (C) { C(m) +=! A(m, r_n) }"
+X_ONLY = [1, 2, 4, 7, 8, 11, 15, 17, 24, 32, 35, 42, 64, 128, 130, 192, 256, 320, 512, 1024]
+XY = [(4, 7), (11, 5), (16, 9), (8, 11), (11, 8), (111, 7), (128, 7), (7, 128), (64, 4), (256, 4), (192, 3)]
+
+
+def check(src, entry, ins_np, options, k):
+    ins = [torch.from_numpy(a).cuda() for a in ins_np]
+    ex = tc.compile(src, entry, ins, options)
+    outs = tc.prepare_outputs(src, entry, ins)
+    for o in outs:
+        o.fill_(float("nan"))
+    tc.run(ex, ins, outs)
+    torch.cuda.synchronize()
+    ref = tc_oracle.run(src, entry, ins_np)
+    for o, r in zip(outs, ref):
+        assert np.abs(o.cpu().numpy() - r).max() <= W.tolerance(k, r)
+    return ex
+
+
+@pytest.mark.parametrize("bx", X_ONLY)
+def test_row_sums_block_x(bx):
+    print(f"sum2d block x={bx}", flush=True)
+    A = np.random.Generator(np.random.Philox(bx)).standard_normal((37, 1013), dtype=np.float32)
+    ex = check(SUM2D, "sum2d", [A], f"naive;matchLibraryCalls=1;mapToThreads={bx};mapToBlocks=64;tile=1", 1013)
+    assert ("blockAllReduceX" in ex.compiled_source) == (bx > 1)
+
+
+@pytest.mark.parametrize("bx,by", XY)
+def test_row_sums_block_xy(bx, by):
+    print(f"sum2d block x={bx} y={by}", flush=True)
+    A = np.random.Generator(np.random.Philox(bx * 1000 + by)).standard_normal((53, 700), dtype=np.float32)
+    check(SUM2D, "sum2d", [A], f"naive;matchLibraryCalls=1;mapToThreads={bx},{by};mapToBlocks=16;tile={by}", 700)
+
+
+def test_all_ones_sum_is_exactly_the_reduction_length():
+    A = np.ones((64, 4096), np.float32)
+    ins = [torch.from_numpy(A).cuda()]
+    ex = tc.compile(SUM2D, "sum2d", ins, "naive;matchLibraryCalls=1;mapToThreads=256;mapToBlocks=64;tile=1;vectorWidth=4")
+    (out,) = tc.prepare_outputs(SUM2D, "sum2d", ins)
+    tc.run(ex, ins, [out])
+    assert torch.all(out == 4096.0)
+
+
+@pytest.mark.parametrize("op,ref", [("max=!", lambda a: a.max(1)), ("min=!", lambda a: a.min(1))])
+def test_min_max_reductions_are_bit_exact(op, ref):
+    src = f"def red(float(M, N) A) -> (C) {{ C(m) {op} A(m, r_n) }}"
+    A = np.random.Generator(np.random.Philox(3)).standard_normal((40, 999), dtype=np.float32)
+    ins = [torch.from_numpy(A).cuda()]
+    ex = tc.compile(src, "red", ins, "naive;matchLibraryCalls=1;mapToThreads=192,2;mapToBlocks=20;tile=2")
+    (out,) = tc.prepare_outputs(src, "red", ins)
+    tc.run(ex, ins, [out])
+    assert np.array_equal(out.cpu().numpy(), ref(A))
+
+
+def test_non_initialising_reduction_accumulates_into_existing_values():
+    src = "def acc(float(M, N) A) -> (C) { C(m) += A(m, r_n) }"
+    A = np.ones((16, 300), np.float32)
+    ins = [torch.from_numpy(A).cuda()]
+    for opts in ("naive", "naive;matchLibraryCalls=1;mapToThreads=64,2;tile=2"):
+        ex = tc.compile(src, "acc", ins, opts)
+        out = torch.full((16,), 5.0, device="cuda")
+        tc.run(ex, ins, [out])
+        assert torch.all(out == 305.0), opts
+
+
+def test_moments_full_size_properties():
+    """Size-independent checks at the benchmark size: a row of constants has that mean and zero
+    variance; shifting a row shifts the mean and keeps the variance."""
+    name = "c5_moments"
+    src, entry, shapes, _, k = W.CONFIGS[name]
+    X = W.make_inputs(name)[0]
+    X[0, :] = 2.5
+    X[1, :] = X[2, :] + 10.0
+    ins = [torch.from_numpy(X).cuda()]
+    ex = tc.compile(src, entry, ins, W.TUNED[name])
+    mean, var = tc.prepare_outputs(src, entry, ins)
+    tc.run(ex, ins, [mean, var])
+    mean, var = mean.cpu().numpy(), var.cpu().numpy()
+    assert mean[0] == 2.5 and var[0] == 0.0
+    assert abs(mean[1] - (mean[2] + 10.0)) <= 1e-4
+    assert abs(var[1] - var[2]) <= 1e-3 * var[2]
+    Xd = X.astype(np.float64)
+    assert np.abs(mean - Xd.mean(1)).max() <= W.tolerance(k, Xd.mean(1))
+    assert np.abs(var - Xd.var(1)).max() <= W.tolerance(k, Xd.var(1))

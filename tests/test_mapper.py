@@ -1,0 +1,148 @@
+"""Mapper known answers on a GPU-less host: tightened launch bounds, stage/kernel formation under
+the fusion strategies, reduction-library matching, LDS promotion footprints, collapsing, vector
+lanes, error paths.  Scenarios follow test/test_cuda_mapper.cc (:352-383 Basic, :632-645 1-D code on
+a 2-D mapping, :837-850/:930-994 reductions) and test_cuda_mapper_memory_promotion.cc (:298-310
+footprints, :441-449), restated for this mapper's output."""
+import re
+
+import pytest
+
+import tensorcomprehensions_amd as tc
+from tensorcomprehensions_amd import MappingOptions, ShapeOnly
+from tests import workloads as W
+
+
+def mapped(src, entry, shapes, options):
+    return tc.map_only(src, entry, [ShapeOnly(s) for s in shapes], options)
+
+
+ADD = "def fun(float(N, M) A, float(N, M) B) -> (C) { C(n, m) = A(n, m) + B(n, m) }"
+
+
+def test_launch_bounds_are_tightened_to_the_problem():
+    o = MappingOptions.naive().tile(16, 16).mapToBlocks(256, 256).mapToThreads(16, 16).collapseContiguous(False)
+    src, launches = mapped(ADD, "fun", [(512, 40), (512, 40)], o)
+    assert launches == [((32, 3, 1), (16, 16, 1))]            # 512/16 blocks in x, ceil(40/16) in y
+    # the last m tile is partial: a guard must protect it
+    assert "<= 39" in src
+
+
+def test_one_dimensional_code_on_a_two_dimensional_mapping():
+    src, launches = mapped("def f(float(N) A) -> (B) { B(n) = A(n) }", "f", [(100,)], MappingOptions.naive())
+    (grid, block), = launches
+    assert grid == (4, 1, 1) and block == (32, 1, 1)          # tile 32 -> 4 tiles; y extents collapse to 1
+
+
+def test_kernel_name_and_argument_order():
+    src, _ = mapped(W.TENSORDOT, "tensordot", [(16, 8, 16, 17, 25), (16, 16, 2, 17, 25)], "naive")
+    # sizes appended in parameter-name order C1,C2,C3,H,N,W; args: sizes, outputs, inputs
+    assert re.search(r"tensordot_8_16_2_17_16_25\(int C1, int C2, int C3, int H, int N, int W, "
+                     r"float\* __restrict__ pO, const float\* __restrict__ pI0, const float\* __restrict__ pI1\)", src)
+
+
+def test_collapse_and_vector_lanes():
+    shapes = [(4, 8, 8, 28, 28), (4, 8, 2, 28, 28)]
+    src, _ = mapped(W.TENSORDOT, "tensordot", shapes, MappingOptions.naive().vectorWidth(4))
+    assert "i_h_w_o" in src and "i_h_w_v" in src              # h,w merged (784 contiguous), split in lanes of 4
+    src, _ = mapped(W.TENSORDOT, "tensordot", shapes, MappingOptions.naive().collapseContiguous(False))
+    assert "i_h_w" not in src and "i_w" in src
+    # 17*25 = 425 is not a multiple of 4: lanes are dropped, the code stays scalar
+    src, _ = mapped(W.TENSORDOT, "tensordot", [(2, 3, 4, 17, 25), (2, 4, 2, 17, 25)], MappingOptions.naive().vectorWidth(4))
+    assert "i_h_w" in src and "_v" not in src
+    # the convolution's h and w are not jointly contiguous in the input (windows): no merge
+    src, _ = mapped(W.GROUP_CONVOLUTION, "group_convolution", [(2, 2, 4, 8, 8), (2, 4, 4, 3, 3), (2, 4)], "naive")
+    assert "i_h_w" not in src
+
+
+def test_reduction_library_is_matched_only_when_asked():
+    red = "def fun(float(N, K) I) -> (O) { O(n) +=! I(n, r_k) }"
+    src, launches = mapped(red, "fun", [(64, 4096)], MappingOptions.naive().matchLibraryCalls(True).mapToThreads(128, 2).tile(2))
+    assert "__tc::blockAllReduceX<__tc::OpSum<float>, 128, 2, 1>" in src
+    assert launches == [((32, 1, 1), (128, 2, 1))]
+    src, _ = mapped(red, "fun", [(64, 4096)], MappingOptions.naive().matchLibraryCalls(False).mapToThreads(128, 2))
+    assert "blockAllReduceX" not in src
+    # x extent 1: nothing to reduce across
+    src, _ = mapped(red, "fun", [(64, 4096)], MappingOptions.naive().matchLibraryCalls(True).mapToThreads(1))
+    assert "blockAllReduceX" not in src
+    # min / max / product use their own operators
+    mx = "def fun(float(N, K) I) -> (O) { O(n) max=! I(n, r_k) }"
+    src, _ = mapped(mx, "fun", [(64, 4096)], MappingOptions.naive().matchLibraryCalls(True).mapToThreads(64))
+    assert "__tc::OpMax<float>" in src
+
+
+def test_lds_promotion_footprints():
+    o = MappingOptions.naive().tile(1, 26, 26, 72).mapToThreads(26, 13).mapToBlocks(500).unroll(4).useSharedMemory(True)
+    src, launches = mapped(W.BATCH_MATMUL, "batch_matmul", [(500, 26, 72), (500, 72, 26)], o)
+    assert launches == [((500, 1, 1), (26, 13, 1))]
+    # per block: X[1][26][72] and Y[1][72][26] (footprint = min(tile, size) per dimension)
+    assert "__shared__ float lds0_X[1872];" in src
+    assert re.search(r"__shared__ float lds0_Y\[(1872|1944)\];", src)
+    assert src.count("__syncthreads();") >= 2                 # before and after the copies
+    # without the switch nothing is staged
+    src, _ = mapped(W.BATCH_MATMUL, "batch_matmul", [(500, 26, 72), (500, 72, 26)], o.useSharedMemory(False))
+    assert "__shared__" not in src
+    # no reuse, no promotion: a point-wise sum reads every element once
+    src, _ = mapped(ADD, "fun", [(64, 64), (64, 64)], MappingOptions.naive().useSharedMemory(True))
+    assert "__shared__" not in src
+
+
+def test_convolution_window_footprint_includes_the_halo():
+    o = "naive;tile=1,1,16,14,14,4;mapToThreads=14,14;mapToBlocks=32,32;unroll=16;useSharedMemory=1"
+    src, _ = mapped(W.GROUP_CONVOLUTION, "group_convolution", [(32, 32, 16, 16, 16), (32, 16, 16, 3, 3), (32, 16)], o)
+    # input tile: 4 channels x (14+2) x (14+2); weights: 16 x 4 x 3 x 3
+    assert "__shared__ float lds0_I[1024];" in src
+    assert "__shared__ float lds0_W1[576];" in src
+
+
+def test_lds_budget_is_respected():
+    o = MappingOptions.naive().tile(1, 26, 26, 72).mapToThreads(26, 13).mapToBlocks(500).unroll(4).useSharedMemory(True)
+    src, _ = mapped(W.BATCH_MATMUL, "batch_matmul", [(500, 26, 72), (500, 72, 26)], o.maxSharedMemory(8000))
+    assert src.count("__shared__ float") == 1                 # only one of the two 7.5 KB tiles fits
+
+
+def test_fusion_strategies_decide_kernel_count():
+    gc = [(2, 3, 4, 9, 8), (3, 5, 4, 3, 3), (3, 5)]
+    _, launches = mapped(W.GROUP_CONVOLUTION, "group_convolution", gc, MappingOptions.naive())
+    assert len(launches) == 1                                  # bias epilogue fused into the reduction stage
+    _, launches = mapped(W.GROUP_CONVOLUTION, "group_convolution", gc, MappingOptions.naive().scheduleFusionStrategy("Min"))
+    assert len(launches) == 2
+    src, launches = mapped(W.MOMENTS, "moments", [(64, 1024)], MappingOptions.naive())
+    assert len(launches) == 1 and "// stage 1: var" in src and "__syncthreads();" in src
+    _, launches = mapped(W.MOMENTS, "moments", [(64, 1024)], MappingOptions.naive().scheduleFusionStrategy("Min"))
+    assert len(launches) == 2
+
+
+def test_producer_consumer_matmuls_share_only_the_row_dimension():
+    two = """def fun(float(M, K) I, float(K, N) W1, float(N, P) W2) -> (O1, O2) {
+        O1(m, n) +=!  I(m, r_k) * W1(r_k, n)
+        O2(m, p) +=! O1(m, r_n) * W2(r_n, p) }"""
+    shapes = [(64, 32), (32, 48), (48, 16)]
+    src, launches = mapped(two, "fun", shapes, MappingOptions.naive().scheduleFusionStrategy("Max").tile(4, 16).mapToBlocks(256, 256))
+    assert len(launches) == 1
+    (grid, _), = launches
+    assert grid == (16, 1, 1)                                  # blocks only over m: O2 needs whole rows of O1
+    _, launches = mapped(two, "fun", shapes, MappingOptions.naive())   # Preserve3Coincident: needs 2 shared dims
+    assert len(launches) == 2
+
+
+@pytest.mark.parametrize("bad,fragment", [
+    ("naive;mapToThreads=0", "mapping to 0"),
+    ("naive;mapToBlocks=0", "mapping to 0"),
+    ("naive;mapToThreads=1024,2;tile=0,0;collapseContiguous=0", "exceeds the device limit"),
+])
+def test_options_the_mapper_cannot_honour(bad, fragment):
+    with pytest.raises(tc.TcError) as e:
+        mapped(ADD, "fun", [(2048, 2048), (2048, 2048)], bad)
+    assert fragment in str(e.value)
+
+
+def test_generated_sources_compile_for_gfx950():
+    cases = [
+        (W.MOMENTS, "moments", [(64, 1000)], "naive;matchLibraryCalls=1;mapToThreads=96,2;tile=2"),
+        (W.BATCH_MATMUL, "batch_matmul", [(7, 26, 72), (7, 72, 26)], "naive;tile=1,13,26,8;mapToThreads=26,13;useSharedMemory=1;unroll=8"),
+        ("def f(int32(N) A, float(N) B) -> (C) { C(n) = float(A(n) % 3) * B(n) + exp(B(n)) }", "f", [(100,), (100,)], "pointwise"),
+    ]
+    for src, entry, shapes, opts in cases:
+        ins = [ShapeOnly(s, "int32" if (src.startswith("def f(int32") and i == 0) else "float32") for i, s in enumerate(shapes)]
+        ex = tc.compile(src, entry, ins, opts)
+        assert ex.num_kernels >= 1 and "extern \"C\" __global__" in ex.compiled_source
