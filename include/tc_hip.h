@@ -93,6 +93,15 @@ int tc_executor_profile(
     const tc_dl_tensor* const* outputs, int num_outputs, void* stream,
     double* kernel_us, double* cpu_overhead_us);
 
+/* `repeats` back-to-back launches between one pair of events on `stream`, raw pointers, no
+ * checks; *total_us = device time of all of them.  For kernels shorter than a host launch round
+ * trip; the reference's benchmark loop (tc/benchmarks/benchmark_fixture.h:201-241) times single
+ * launches at whole-microsecond resolution instead. */
+int tc_executor_profile_repeated(
+    const tc_executor_t* executor,
+    const void* const* inputs, int num_inputs, void* const* outputs, int num_outputs, void* stream,
+    int repeats, double* total_us);
+
 /* TcExecutor::compiledSource, CudaTcExecutor::grid()/block() (cuda_tc_executor.h:52-60) */
 const char* tc_executor_source(const tc_executor_t* executor);
 int tc_executor_num_kernels(const tc_executor_t* executor);

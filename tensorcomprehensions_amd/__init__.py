@@ -22,7 +22,7 @@ from ._capi import TcError
 from .mapping_options import MappingOptions, FusionStrategy
 
 __all__ = [
-    "compile", "prepare_outputs", "infer_output_tensor_info", "run", "profile", "unchecked_run", "autotune",
+    "compile", "prepare_outputs", "infer_output_tensor_info", "run", "profile", "profile_repeated", "unchecked_run", "autotune",
     "map_only", "lang_dump", "host_query", "set_compiler_options", "ShapeOnly", "Executor", "MappingOptions", "FusionStrategy", "ProfilingInfo", "TcError",
 ]
 
@@ -180,6 +180,16 @@ def profile(executor, inputs, outputs):
     _capi.check(_capi.lib().tc_executor_profile(executor._h, pin.ptr, len(pin), pout.ptr, len(pout), _stream(),
                                                 ctypes.byref(k), ctypes.byref(c)))
     return ProfilingInfo(c.value, k.value)
+
+
+def profile_repeated(executor, inputs, outputs, repeats):
+    """Device time in microseconds of `repeats` back-to-back launches (one event pair around all)."""
+    ins = (ctypes.c_void_p * max(len(inputs), 1))(*[t.data_ptr() for t in inputs])
+    outs = (ctypes.c_void_p * max(len(outputs), 1))(*[t.data_ptr() for t in outputs])
+    total = ctypes.c_double(0)
+    _capi.check(_capi.lib().tc_executor_profile_repeated(executor._h, ins, len(inputs), outs, len(outputs), _stream(),
+                                                         int(repeats), ctypes.byref(total)))
+    return total.value
 
 
 def set_compiler_options(emit_warnings=True, throw_warnings=False):

@@ -77,6 +77,9 @@ def _declare(l):
                                             P(ctypes.c_void_p), ctypes.c_int, ctypes.c_void_p]
     l.tc_executor_profile.argtypes = [ctypes.c_void_p, tensors, ctypes.c_int, tensors, ctypes.c_int,
                                       ctypes.c_void_p, P(ctypes.c_double), P(ctypes.c_double)]
+    l.tc_executor_profile_repeated.argtypes = [ctypes.c_void_p, P(ctypes.c_void_p), ctypes.c_int,
+                                               P(ctypes.c_void_p), ctypes.c_int, ctypes.c_void_p, ctypes.c_int,
+                                               P(ctypes.c_double)]
     l.tc_executor_source.argtypes = [ctypes.c_void_p]
     l.tc_executor_source.restype = ctypes.c_char_p
     l.tc_executor_num_kernels.argtypes = [ctypes.c_void_p]

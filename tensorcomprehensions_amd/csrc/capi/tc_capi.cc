@@ -147,6 +147,19 @@ int tc_executor_profile(
   TC_CAPI_END
 }
 
+int tc_executor_profile_repeated(
+    const tc_executor_t* ex, const void* const* inputs, int numInputs, void* const* outputs, int numOutputs,
+    void* stream, int repeats, double* totalUs) {
+  TC_CAPI_BEGIN
+  TC_CHECK(ex && ex->impl) << "null executor";
+  tc::HipRuntimeInformation info;
+  info.stream = stream;
+  tc::Duration d = ex->impl->profileRepeated(
+      std::vector<const void*>(inputs, inputs + numInputs), std::vector<void*>(outputs, outputs + numOutputs), repeats, info);
+  *totalUs = d.toMicroSecondsF();
+  TC_CAPI_END
+}
+
 const char* tc_executor_source(const tc_executor_t* ex) {
   return ex && ex->impl ? ex->impl->compiledSource.c_str() : "";
 }

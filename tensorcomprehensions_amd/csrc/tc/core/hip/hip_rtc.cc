@@ -61,7 +61,8 @@ Duration HipRTCFunction::Launch(
     std::vector<int> params,
     std::vector<void*> outputs,
     std::vector<const void*> inputs,
-    bool profile) const {
+    bool profile,
+    int repeats) const {
   TC_CHECK(!cleared_) << "launch of a cleared RTC function";
   int dev = 0;
   TC_HIP_CHECK(tchip_get_device(&dev));
@@ -79,8 +80,8 @@ Duration HipRTCFunction::Launch(
   if (profile) {
     TC_HIP_CHECK(tchip_event_create(&start));
     TC_HIP_CHECK(tchip_event_create(&stop));
-    TC_HIP_CHECK(tchip_event_record(start, stream));
   }
+  std::vector<tchip_function_t> fns;
   for (const auto& k : kernels) {
     auto key = std::make_pair(dev, k.name);
     auto it = functions_.find(key);
@@ -89,7 +90,15 @@ Duration HipRTCFunction::Launch(
       TC_HIP_CHECK(tchip_module_get_function(modules_[dev], k.name.c_str(), &fn));
       it = functions_.emplace(key, fn).first;
     }
-    TC_HIP_CHECK(tchip_launch(it->second, k.grid.data(), k.block.data(), 0, stream, args.data()));
+    fns.push_back(it->second);
+  }
+  if (profile) {
+    TC_HIP_CHECK(tchip_event_record(start, stream));
+  }
+  for (int r = 0; r < repeats; ++r) {
+    for (size_t i = 0; i < kernels.size(); ++i) {
+      TC_HIP_CHECK(tchip_launch(fns[i], kernels[i].grid.data(), kernels[i].block.data(), 0, stream, args.data()));
+    }
   }
   if (profile) {
     float ms = 0;

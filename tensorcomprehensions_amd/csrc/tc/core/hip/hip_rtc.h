@@ -28,13 +28,16 @@ class HipRTCFunction {
   // Launches the kernels in order on `stream` with arguments (params..., outputs..., inputs...).
   // With profile=true the launches are bracketed by events and the elapsed device time is
   // returned after synchronising; otherwise returns Duration::max() without synchronising.
+  // `repeats` > 1 issues the whole launch sequence that many times back to back (between the
+  // events when profiling): the way to time kernels shorter than a launch round trip.
   Duration Launch(
       const std::vector<HipKernelLaunch>& kernels,
       tchip_stream_t stream,
       std::vector<int> params,
       std::vector<void*> outputs,
       std::vector<const void*> inputs,
-      bool profile = false) const;
+      bool profile = false,
+      int repeats = 1) const;
 
   void clear();
   const std::string& code() const { return code_; }

@@ -68,6 +68,16 @@ void HipTcExecutor::uncheckedRun(
   rtcFun_->Launch(result_.kernels, info.stream, result_.parameters, outputs, inputs, false);
 }
 
+Duration HipTcExecutor::profileRepeated(
+    const std::vector<const void*>& inputs,
+    const std::vector<void*>& outputs,
+    int repeats,
+    HipRuntimeInformation info) const {
+  TC_CHECK(rtcFun_) << "No rtcFun_ attached, cannot launch";
+  TC_CHECK_GE(repeats, 1);
+  return rtcFun_->Launch(result_.kernels, info.stream, result_.parameters, outputs, inputs, true, repeats);
+}
+
 ProfilingInfo HipTcExecutor::profileUnchecked(
     const std::vector<const void*>& inputs,
     const std::vector<void*>& outputs,

@@ -25,6 +25,14 @@ class HipTcExecutor : public TcExecutor<HipBackend> {
       const std::vector<void*>& outputs,
       HipRuntimeInformation info = HipRuntimeInformation()) const override;
 
+  // Total device time of `repeats` back-to-back launches (one pair of events around all of
+  // them); divide by `repeats` for a per-launch figure that is free of host launch latency.
+  Duration profileRepeated(
+      const std::vector<const void*>& inputs,
+      const std::vector<void*>& outputs,
+      int repeats,
+      HipRuntimeInformation info = HipRuntimeInformation()) const;
+
   // Unloads the JIT-compiled module; the executor cannot run afterwards.
   void clearRuntimeCompiledFunction() {
     if (rtcFun_) {

@@ -1,6 +1,7 @@
 #include "tc/core/mapper/mapper.h"
 
 #include <algorithm>
+#include <cctype>
 #include <cstdio>
 #include <functional>
 #include <set>
@@ -535,7 +536,14 @@ class StageCodegen {
         return p.ldsName + "[" + ldsIndex(p, e->args) + "]";
       }
     }
-    return "p" + e->name + "[" + flatIndex(e->name, e->args, accRef) + "]";
+    std::string global = "p" + e->name + "[" + flatIndex(e->name, e->args, accRef) + "]";
+    if (inCachedReduction_) {
+      auto it = regCaches.find(global);
+      if (it != regCaches.end()) {
+        return it->second.name + "[" + cacheSlot_ + "]";
+      }
+    }
+    return global;
   }
 
   std::string expr(const ExprRef& e, const std::string& accRef) {
@@ -678,6 +686,13 @@ class StageCodegen {
       const TensorView& view = st_.views.at(acc.first);
       if (view.isOutput) continue; // may be written by another stage of this kernel
       const auto& ref = acc.second.front();
+      // an operand every thread of the block reads at the same address goes through the scalar
+      // data cache (s_load into SGPRs); staging it in LDS would only add traffic
+      bool uniform = true;
+      for (const auto& sub : ref) {
+        for (const auto& cv : sub.coef) uniform &= var(cv.first).threadAxis < 0 || cv.second == 0;
+      }
+      if (uniform) continue;
       bool sameShape = true;
       for (const auto& a : acc.second) {
         for (size_t j = 0; j < a.size(); ++j) sameShape &= a[j].coef == ref[j].coef;
@@ -758,28 +773,55 @@ class StageCodegen {
       em_.line("const int lo" + std::to_string(stageIdx_) + "_" + p.tensor + "_" + std::to_string(j) + " = " +
                footprintLow(p, j) + ";");
     }
-    if (kc_.opts.unrollCopySharedValue) em_.line("#pragma unroll");
-    em_.open("for (int c_ = tid_; c_ < " + std::to_string(count) + "; c_ += " + std::to_string(kc_.NT()) + ")");
-    int64_t div = count;
+    // Two phases per chunk of iterations: all global loads first (unconditional, from a clamped
+    // address, so they are issued back to back and their latencies overlap), then the LDS stores.
+    int64_t iters = ceilDiv(count, kc_.NT());
+    int64_t chunk = std::min<int64_t>(iters, kc_.opts.unrollCopySharedValue ? 32 : 16);
+    std::string ty = view.type.cName();
+    auto decompose = [&](const std::string& itExpr, std::string& cond, std::string& gidx, std::string& lidx) {
+      em_.line("const int c_ = (" + itExpr + ") * " + std::to_string(kc_.NT()) + " + tid_;");
+      int64_t div = count;
+      cond.clear();
+      gidx.clear();
+      lidx.clear();
+      for (size_t j = 0; j < p.extents.size(); ++j) {
+        div /= p.extents[j];
+        std::string l = "l" + std::to_string(j) + "_";
+        std::string e = "c_";
+        if (div > 1) e = "(" + e + " / " + std::to_string(div) + ")";
+        if (j > 0) e = e + " % " + std::to_string(p.extents[j]);
+        em_.line("const int " + l + " = " + e + ";");
+        std::string g = "g" + std::to_string(j) + "_";
+        em_.line("const int " + g + " = lo" + std::to_string(stageIdx_) + "_" + p.tensor + "_" + std::to_string(j) + " + " + l + ";");
+        cond += (j ? " && " : "") + std::string("(unsigned)") + g + " < " + std::to_string(view.extents[j]) + "u";
+        gidx += (j ? " + " : "") + g + (gStrides[j] != 1 ? " * " + std::to_string(gStrides[j]) : "");
+        lidx += (j ? " + " : "") + l + (p.ldsStrides[j] != 1 ? " * " + std::to_string(p.ldsStrides[j]) : "");
+      }
+      if (p.extents.empty()) {
+        cond = "true";
+        gidx = lidx = "0";
+      }
+      cond = "c_ < " + std::to_string(count) + " && " + cond;
+    };
+    bool chunked = iters > chunk;
+    if (chunked) {
+      em_.open("for (int cb_ = 0; cb_ < " + std::to_string(iters) + "; cb_ += " + std::to_string(chunk) + ")");
+    } else {
+      em_.open("");
+    }
+    std::string base = chunked ? "cb_ + " : "";
+    em_.line(ty + " stage_[" + std::to_string(chunk) + "];");
     std::string cond, gidx, lidx;
-    for (size_t j = 0; j < p.extents.size(); ++j) {
-      div /= p.extents[j];
-      std::string l = "l" + std::to_string(j) + "_";
-      std::string e = "c_";
-      if (div > 1) e = "(" + e + " / " + std::to_string(div) + ")";
-      if (j > 0) e = e + " % " + std::to_string(p.extents[j]);
-      em_.line("const int " + l + " = " + e + ";");
-      std::string g = "g" + std::to_string(j) + "_";
-      em_.line("const int " + g + " = lo" + std::to_string(stageIdx_) + "_" + p.tensor + "_" + std::to_string(j) + " + " + l + ";");
-      cond += (j ? " && " : "") + std::string("(unsigned)") + g + " < " + std::to_string(view.extents[j]) + "u";
-      gidx += (j ? " + " : "") + g + (gStrides[j] != 1 ? " * " + std::to_string(gStrides[j]) : "");
-      lidx += (j ? " + " : "") + l + (p.ldsStrides[j] != 1 ? " * " + std::to_string(p.ldsStrides[j]) : "");
-    }
-    if (p.extents.empty()) {
-      cond = "true";
-      gidx = lidx = "0";
-    }
-    em_.line("if (" + cond + ") " + p.ldsName + "[" + lidx + "] = p" + p.tensor + "[" + gidx + "];");
+    em_.line("#pragma unroll");
+    em_.open("for (int it_ = 0; it_ < " + std::to_string(chunk) + "; ++it_)");
+    decompose(base + "it_", cond, gidx, lidx);
+    em_.line("stage_[it_] = p" + p.tensor + "[(" + cond + ") ? (" + gidx + ") : 0];");
+    em_.close();
+    em_.line("#pragma unroll");
+    em_.open("for (int it_ = 0; it_ < " + std::to_string(chunk) + "; ++it_)");
+    decompose(base + "it_", cond, gidx, lidx);
+    em_.line("if (c_ < " + std::to_string(count) + ") " + p.ldsName + "[" + lidx + "] = stage_[it_];");
+    em_.close();
     em_.close();
   }
 
@@ -919,6 +961,8 @@ class StageCodegen {
     // point loops, innermost ones unrolled under the budget
     std::vector<int> factors(s.redVars.size(), 0); // 0: no pragma, -1: full, >1: partial
     int64_t remaining = std::max<int64_t>(1, unrollBudget / std::max<int64_t>(1, st_.accCount));
+    bool cached = !regCaches.empty() && &s == cachedStmt_;
+    if (cached) remaining = 1 << 30; // register-cached operands need fully unrolled loops
     for (int i = static_cast<int>(s.redVars.size()) - 1; i >= 0; --i) {
       const LoopVar& v = var(s.redVars[i]);
       if (v.vectorLane) {
@@ -944,7 +988,25 @@ class StageCodegen {
     {
       int n = openUnrolled();
       std::string cond = rpred.empty() ? "ok_" : "ok_ && " + rpred;
+      if (cached) {
+        // slot of this (register-tile element, reduction iteration) in the per-thread cache
+        std::string rlin = "0";
+        int64_t rcount = 1;
+        for (const auto& r : s.redVars) {
+          const LoopVar& v = var(r);
+          rcount *= v.perThread;
+          if (v.perThread > 1) rlin = "(" + rlin + ") * " + std::to_string(v.perThread) + " + q_" + v.name;
+        }
+        cacheSlot_ = "a_ * " + std::to_string(rcount) + " + " + rlin;
+        for (const auto& c : regCaches) {
+          if (c.second.producer) {
+            em_.line("if (" + cond + ") " + c.second.name + "[" + cacheSlot_ + "] = " + c.first + ";");
+          }
+        }
+        inCachedReduction_ = true;
+      }
       std::string rhs = castTo(s.rhs, accType_, "acc_[a_]");
+      inCachedReduction_ = false;
       em_.line("if (" + cond + ") " + target + "[a_] = " + combine(s.op, target + "[a_]", rhs) + ";");
       closeN(n);
     }
@@ -960,6 +1022,69 @@ class StageCodegen {
       em_.line("acc_[a_] = " + combine(s.op, "acc_[a_]", "tot_") + ";");
       closeN(n);
     }
+  }
+
+  // --- register caches shared between stages -----------------------------------------------------
+  struct RegCache {
+    std::string name;
+    bool producer = false;
+  };
+  std::map<std::string, RegCache> regCaches; // printed global load -> cache
+  const StageStmt* cachedStmt_ = nullptr;
+
+  const StageStmt* firstReduction() const {
+    for (const auto& s : st_.stmts) {
+      if (!s.redVars.empty()) return &s;
+    }
+    return nullptr;
+  }
+
+  // Loop structure + addressing of the stage's reduction statement in position-independent
+  // form: two stages with equal signatures make every thread touch the same addresses at the
+  // same loop counters.  Empty when the stage cannot take part in register caching.
+  std::string cacheSignature(std::vector<std::pair<std::string, std::string>>& loads) {
+    const StageStmt* s = firstReduction();
+    if (!s) return "";
+    std::map<std::string, std::string> canon;
+    std::ostringstream sig;
+    for (size_t i = 0; i < st_.vars.size(); ++i) {
+      const LoopVar& v = st_.vars[i];
+      bool mine = !v.reduction || std::find(s->redVars.begin(), s->redVars.end(), v.name) != s->redVars.end();
+      if (!mine) return "";
+      if (v.reduction && v.numTiles != 1) return "";
+      if (!v.reduction && !v.unrolled && v.perThread > 1) return "";
+      canon[v.name] = "v" + std::to_string(i);
+      sig << v.min << "," << v.extent << "," << v.tile << "," << v.numTiles << "," << v.blockAxis << ","
+          << v.threadAxis << "," << v.perThread << "," << v.unrolled << "," << v.vectorLane << "," << v.reduction << ";";
+    }
+    visit(s->rhs, [&](const ExprRef& e) {
+      if (e->kind != Expr::Load) return;
+      const TensorView& view = st_.views.at(e->name);
+      if (view.isOutput) return;
+      for (const auto& a : e->args) {
+        if (!ir::toAffine(a).valid) return;
+      }
+      std::string text = "p" + e->name + "[" + flatIndex(e->name, e->args, "") + "]";
+      // position-independent spelling of the same address
+      std::string key = text;
+      for (const auto& c : canon) {
+        std::string from = "i_" + c.first, to = "#" + c.second;
+        for (size_t pos = key.find(from); pos != std::string::npos; pos = key.find(from, pos + to.size())) {
+          size_t end = pos + from.size();
+          bool boundary = end >= key.size() || !(std::isalnum(static_cast<unsigned char>(key[end])) || key[end] == '_');
+          if (boundary) key.replace(pos, from.size(), to);
+        }
+      }
+      loads.emplace_back(key, text);
+    });
+    return sig.str();
+  }
+
+  int64_t cacheSlots() const {
+    const StageStmt* s = firstReduction();
+    int64_t n = st_.accCount;
+    for (const auto& r : s->redVars) n *= var(r).perThread;
+    return n;
   }
 
   // --- whole stage ----------------------------------------------------------------------------
@@ -1041,6 +1166,8 @@ class StageCodegen {
   bool accValid_ = false;
   std::string outerPred_;
   std::set<std::string> activePromotions_;
+  bool inCachedReduction_ = false;
+  std::string cacheSlot_;
 };
 
 // ------------------------------------------------------------------------------------------
@@ -1181,6 +1308,40 @@ void emitKernel(KernelCtx& kc, const DeviceLimits& limits, Emitter& em) {
   }
   k.ldsBytes = (before - ldsBudget) + scratchElems * 8;
 
+  // Register promotion across stages (usePrivateMemory): an input that several stages read with
+  // the same loop structure and addresses is loaded once, by the first of them, into a
+  // per-thread register array that lives across the stages of one block iteration.
+  std::vector<std::string> cacheDecls;
+  if (kc.opts.usePrivateMemoryValue && gens.size() >= 2) {
+    std::vector<std::string> sigs(gens.size());
+    std::vector<std::vector<std::pair<std::string, std::string>>> loads(gens.size());
+    for (size_t i = 0; i < gens.size(); ++i) sigs[i] = gens[i].cacheSignature(loads[i]);
+    std::map<std::string, std::string> produced; // canonical load -> cache name
+    for (size_t i = 0; i < gens.size(); ++i) {
+      if (sigs[i].empty() || sigs[i] != sigs[0]) continue;
+      if (gens[i].cacheSlots() > 256) continue;
+      for (const auto& l : loads[i]) {
+        bool sharedLater = false;
+        for (size_t j = 0; j < gens.size(); ++j) {
+          if (j == i || sigs[j] != sigs[i]) continue;
+          for (const auto& m : loads[j]) sharedLater |= m.first == l.first;
+        }
+        if (!sharedLater) continue;
+        auto it = produced.find(l.first);
+        bool producer = it == produced.end();
+        if (producer) {
+          std::string name = "rcache" + std::to_string(produced.size()) + "_";
+          it = produced.emplace(l.first, name).first;
+          std::string tensor = l.second.substr(1, l.second.find('[') - 1);
+          cacheDecls.push_back(k.stages[i].views.at(tensor).type.cName() + " " + name + "[" +
+                               std::to_string(gens[i].cacheSlots()) + "];");
+        }
+        gens[i].regCaches[l.second] = StageCodegen::RegCache{it->second, producer};
+        gens[i].cachedStmt_ = gens[i].firstReduction();
+      }
+    }
+  }
+
   em.open(kernelSignature(kc.f, k.name, kc.NT()));
   for (const auto& p : kc.f.params) em.line("(void)" + p.first + ";");
   em.line("const int tid_ = threadIdx.x + " + std::to_string(k.block[0]) + " * (threadIdx.y + " +
@@ -1212,6 +1373,7 @@ void emitKernel(KernelCtx& kc, const DeviceLimits& limits, Emitter& em) {
       ++opened;
     }
   }
+  for (const auto& d : cacheDecls) em.line(d);
   for (size_t i = 0; i < k.stages.size(); ++i) {
     if (i > 0) em.line("__syncthreads();");
     if (k.stages[i].threadReduction) {
