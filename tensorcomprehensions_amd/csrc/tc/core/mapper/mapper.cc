@@ -434,6 +434,68 @@ struct StageBuilder {
   }
 };
 
+// Decides whether a stage is a dense fp32 contraction the matrix cores can take and assigns the
+// variable roles.  Needs: first statement `out +=(!) A(...) * B(...)` with affine subscripts,
+// float operands, at least one parallel variable private to each operand; later statements are
+// point-wise epilogues.
+bool classifyContraction(StagePlan& st) {
+  if (st.stmts.empty()) return false;
+  const StageStmt& s = st.stmts[0];
+  if (s.redVars.empty() || s.op != ReduceOp::Plus) return false;
+  for (size_t i = 1; i < st.stmts.size(); ++i) {
+    if (!st.stmts[i].redVars.empty()) return false;
+  }
+  ScalarType f32{ScalarType::Float, 32};
+  if (st.views.at(st.tensor).type != f32) return false;
+  const ExprRef& e = s.rhs;
+  if (e->kind != Expr::Binary || e->name != "*" || e->args[0]->kind != Expr::Load || e->args[1]->kind != Expr::Load) {
+    return false;
+  }
+  for (const auto& l : e->args) {
+    if (l->type != f32 || l->name == st.tensor) return false;
+    for (const auto& a : l->args) {
+      if (!ir::toAffine(a).valid) return false;
+    }
+  }
+  auto mentions = [](const ExprRef& load, const std::string& v) {
+    bool m = false;
+    visit(load, [&](const ExprRef& x) { m |= x->kind == Expr::Var && x->name == v; });
+    return m;
+  };
+  std::vector<std::string> onlyA, onlyB, batch, k;
+  for (const auto& v : st.vars) {
+    if (v.vectorLane) return false;
+    bool a = mentions(e->args[0], v.name), b = mentions(e->args[1], v.name);
+    if (v.reduction) {
+      k.push_back(v.name);
+    } else if (a && !b) {
+      onlyA.push_back(v.name);
+    } else if (b && !a) {
+      onlyB.push_back(v.name);
+    } else {
+      batch.push_back(v.name);
+    }
+  }
+  if (onlyA.empty() || onlyB.empty() || k.empty()) return false;
+  st.mfma = true;
+  st.mfmaM = onlyA;
+  st.mfmaN = onlyB;
+  st.mfmaBatch = batch;
+  st.mfmaK = k;
+  st.mfmaSwapOperands = false;
+  // The 16 lanes of a row group hold 16 consecutive N positions of the output tile: put the
+  // output's innermost (contiguous) index on the N side so that stores coalesce.
+  std::string innermost;
+  for (const auto& v : st.vars) {
+    if (!v.reduction) innermost = v.name;
+  }
+  if (std::find(onlyA.begin(), onlyA.end(), innermost) != onlyA.end()) {
+    std::swap(st.mfmaM, st.mfmaN);
+    st.mfmaSwapOperands = true;
+  }
+  return true;
+}
+
 // ------------------------------------------------------------------------------------------
 // code emission
 // ------------------------------------------------------------------------------------------
@@ -650,11 +712,11 @@ class StageCodegen {
   void planPromotions(const StageStmt& s, int64_t& ldsBudgetBytes) {
     if (!kc_.opts.useSharedMemoryValue || s.redVars.empty()) return;
     for (const auto& v : st_.vars) {
-      if (!v.reduction && !v.unrolled && v.perThread > 1) return; // needs a full register tile
+      if (!st_.mfma && !v.reduction && !v.unrolled && v.perThread > 1) return; // needs a full register tile
     }
     bool reductionTiled = false;
     for (const auto& r : s.redVars) reductionTiled |= var(r).numTiles > 1;
-    bool inside = reductionTiled &&
+    bool inside = reductionTiled && !st_.mfma &&
         (!kc_.opts.hasSharedDepth || kc_.opts.sharedDepthValue > static_cast<uint32_t>(st_.numParallel));
     // iterations of the statement inside the promoted region
     std::set<std::string> stmtVars;
@@ -688,7 +750,7 @@ class StageCodegen {
       const auto& ref = acc.second.front();
       // an operand every thread of the block reads at the same address goes through the scalar
       // data cache (s_load into SGPRs); staging it in LDS would only add traffic
-      bool uniform = true;
+      bool uniform = !st_.mfma; // on the matrix cores every operand element differs per lane
       for (const auto& sub : ref) {
         for (const auto& cv : sub.coef) uniform &= var(cv.first).threadAxis < 0 || cv.second == 0;
       }
@@ -1097,9 +1159,134 @@ class StageCodegen {
     }
   }
 
+  // Declares i_<v> (and p_<v>) for every variable of `group` from the flattened position `pos`
+  // inside the block tile (row-major over the group's tile extents, last variable fastest) and
+  // returns the predicate "position exists".
+  std::string decodeGroup(const std::vector<std::string>& group, const std::string& pos) {
+    int64_t total = 1;
+    for (const auto& n : group) total *= var(n).tile;
+    std::string pred = pos + " < " + std::to_string(total);
+    int64_t div = total;
+    for (const auto& n : group) {
+      const LoopVar& v = var(n);
+      div /= v.tile;
+      std::string e = pos;
+      if (div > 1) e = "(" + e + " / " + std::to_string(div) + ")";
+      if (&n != &group.front()) e = e + " % " + std::to_string(v.tile);
+      std::string base = std::to_string(v.min);
+      if (v.numTiles > 1) base += " + " + tv(v) + " * " + std::to_string(v.tile);
+      em_.line("const int p_" + v.name + " = " + e + ";");
+      em_.line("const int " + iv(v) + " = " + base + " + p_" + v.name + ";");
+      if (v.partial()) pred += " && " + iv(v) + " <= " + std::to_string(v.min + v.extent - 1);
+    }
+    return pred;
+  }
+
+  void emitMfma() {
+    const StageStmt& s = st_.stmts[0];
+    auto tileProduct = [&](const std::vector<std::string>& g) {
+      int64_t t = 1;
+      for (const auto& n : g) t *= var(n).tile;
+      return t;
+    };
+    int64_t MT = tileProduct(st_.mfmaM), NT = tileProduct(st_.mfmaN), BT = tileProduct(st_.mfmaBatch),
+            KT = tileProduct(st_.mfmaK);
+    int64_t numMT = ceilDiv(MT, 16), numNT = ceilDiv(NT, 16), ksteps = ceilDiv(KT, 4);
+    int64_t tiles = BT * numMT * numNT;
+    const ExprRef& loadA = s.rhs->args[st_.mfmaSwapOperands ? 1 : 0]; // holds the M-side variables
+    const ExprRef& loadB = s.rhs->args[st_.mfmaSwapOperands ? 0 : 1]; // holds the N-side variables
+    em_.line("// matrix cores: " + std::to_string(tiles) + " tiles of 16x16 per block, " + std::to_string(ksteps) +
+             " steps of v_mfma_f32_16x16x4_f32 each, " + std::to_string(st_.waves) + " wavefront(s)");
+    int opened = 0;
+    if (!st_.promotions.empty()) {
+      em_.open("");
+      ++opened;
+      em_.line("__syncthreads();");
+      for (const auto& p : st_.promotions) {
+        emitCopyIn(p);
+        activePromotions_.insert(p.tensor);
+      }
+      em_.line("__syncthreads();");
+    }
+    em_.line("const int lm_ = threadIdx.x & 15, lj_ = threadIdx.x >> 4;");
+    em_.open("for (int tl_ = threadIdx.y; tl_ < " + std::to_string(tiles) + "; tl_ += " + std::to_string(st_.waves) + ")");
+    ++opened;
+    em_.line("const int nt_ = tl_ % " + std::to_string(numNT) + ", mt_ = (tl_ / " + std::to_string(numNT) + ") % " +
+             std::to_string(numMT) + ", bt_ = tl_ / " + std::to_string(numNT * numMT) + ";");
+    std::string bok = st_.mfmaBatch.empty() ? "true" : decodeGroup(st_.mfmaBatch, "bt_");
+    em_.line("const bool bok_ = " + bok + ";");
+    em_.line("const int npos_ = nt_ * 16 + lm_;");
+    em_.line("const bool nok_ = bok_ && " + decodeGroup(st_.mfmaN, "npos_") + ";");
+    em_.line("__tc::floatx4 c_ = {0.0f, 0.0f, 0.0f, 0.0f};");
+    if (!s.init) {
+      // accumulate into the existing output values
+      em_.line("#pragma unroll");
+      em_.open("for (int r_ = 0; r_ < 4; ++r_)");
+      em_.line("const int mpos_ = mt_ * 16 + 4 * lj_ + r_;");
+      em_.line("const bool mok_ = " + decodeGroup(st_.mfmaM, "mpos_") + ";");
+      em_.line("if (nok_ && mok_) c_[r_] = p" + st_.tensor + "[" + flatIndex(st_.tensor, st_.lhsSubs, "") + "];");
+      em_.close();
+    }
+    {
+      em_.open("");
+      em_.line("const int mposa_ = mt_ * 16 + lm_;");
+      em_.line("const bool moka_ = bok_ && " + decodeGroup(st_.mfmaM, "mposa_") + ";");
+      em_.line(ksteps <= 64 ? "#pragma unroll" : "#pragma unroll 4");
+      em_.open("for (int ks_ = 0; ks_ < " + std::to_string(ksteps) + "; ++ks_)");
+      em_.line("const int kk_ = ks_ * 4 + lj_;");
+      em_.line("const bool kok_ = " + decodeGroup(st_.mfmaK, "kk_") + ";");
+      em_.line("const float a_ = (moka_ && kok_) ? " + loadStr(loadA, "") + " : 0.0f;");
+      em_.line("const float b_ = (nok_ && kok_) ? " + loadStr(loadB, "") + " : 0.0f;");
+      em_.line("c_ = __builtin_amdgcn_mfma_f32_16x16x4f32(a_, b_, c_, 0, 0, 0);");
+      em_.close();
+      em_.close();
+    }
+    // epilogue and store: lane holds rows 4*lj_ .. 4*lj_+3 of column lm_
+    em_.line("#pragma unroll");
+    em_.open("for (int r_ = 0; r_ < 4; ++r_)");
+    em_.line("const int mpos_ = mt_ * 16 + 4 * lj_ + r_;");
+    em_.line("const bool okr_ = nok_ && " + decodeGroup(st_.mfmaM, "mpos_") + ";");
+    em_.line(accType_.cName() + " acc_[1];");
+    em_.line("acc_[0] = c_[r_];");
+    outerPred_ = "okr_";
+    accValid_ = true;
+    for (size_t i = 1; i < st_.stmts.size(); ++i) {
+      const StageStmt& e = st_.stmts[i];
+      if (e.op != ReduceOp::None) {
+        int n = openUnrolled();
+        em_.line("if (ok_) acc_[a_] = " + combine(e.op, "acc_[a_]", castTo(e.rhs, accType_, "acc_[a_]")) + ";");
+        closeN(n);
+      } else {
+        emitPointwise(e);
+      }
+    }
+    {
+      int n = openUnrolled();
+      em_.line("if (ok_) p" + st_.tensor + "[" + flatIndex(st_.tensor, st_.lhsSubs, "") + "] = acc_[a_];");
+      closeN(n);
+    }
+    em_.close();
+    closeN(opened);
+    for (const auto& p : st_.promotions) activePromotions_.erase(p.tensor);
+  }
+
   void emit() {
     accType_ = st_.views.at(st_.tensor).type;
     em_.line("// stage " + std::to_string(stageIdx_) + ": " + st_.tensor);
+    if (st_.mfma) {
+      em_.open("");
+      int openedTiles = 1;
+      for (int i = kc_.k.sharedDepth; i < st_.numParallel; ++i) {
+        const LoopVar& v = st_.vars[i];
+        if (v.numTiles > 1) {
+          em_.open("for (int t_" + v.name + " = 0; t_" + v.name + " < " + std::to_string(v.numTiles) + "; ++t_" + v.name + ")");
+          ++openedTiles;
+        }
+      }
+      emitMfma();
+      closeN(openedTiles);
+      return;
+    }
     em_.open("");
     int opened = 1;
     // sequential tile loops of parallel variables not handled at kernel level
@@ -1212,6 +1399,21 @@ void mapKernel(KernelCtx& kc, const DeviceLimits& limits) {
       gridUse[axis] = std::max(gridUse[axis], v.gridExtent);
       ++axis;
     }
+    if (st.mfma) {
+      // one wavefront per 16x16 output tile; the block holds as many wavefronts as the block
+      // option has threads; the reduction is consumed whole (no reduction tiling)
+      for (auto& v : st.vars) {
+        if (v.reduction) {
+          v.tile = v.extent;
+          v.numTiles = 1;
+        }
+      }
+      int64_t threads = static_cast<int64_t>(o.block[0] * o.block[1] * o.block[2]);
+      st.waves = std::max<int64_t>(1, std::min<int64_t>(16, threads / 64));
+      blockUse[0] = std::max<int64_t>(blockUse[0], 64);
+      blockUse[1] = std::max<int64_t>(blockUse[1], st.waves);
+      continue;
+    }
     // threads: innermost variables, x first
     bool hasReduction = false;
     for (const auto& s : st.stmts) hasReduction |= !s.redVars.empty();
@@ -1246,6 +1448,10 @@ void mapKernel(KernelCtx& kc, const DeviceLimits& limits) {
   for (auto& st : k.stages) {
     for (auto& v : st.vars) {
       v.perThread = v.threadAxis >= 0 ? ceilDiv(v.tile, k.block[v.threadAxis]) : v.tile;
+    }
+    if (st.mfma) {
+      st.accCount = 1;
+      continue;
     }
     // register tile: innermost parallel variables first, while the tile fits the budget
     int64_t prod = 1;
@@ -1498,9 +1704,13 @@ MappedProgram mapToHip(
         for (auto& r : ss.redVars) r = ren.at(r);
       }
     }
+    if (options.useMfmaValue) {
+      for (auto& st : k.stages) classifyContraction(st);
+    }
     // vector lanes on the variable that will sit on threadIdx.x
     if (options.vectorWidthValue > 1) {
       for (auto& st : k.stages) {
+        if (st.mfma) continue;
         bool hasRed = false;
         for (const auto& s : st.stmts) hasRed |= !s.redVars.empty();
         bool threadRed = options.generic.matchLibraryCallsValue && hasRed && options.block[0] > 1;

@@ -84,6 +84,13 @@ struct StagePlan {
   bool threadReduction = false;      // innermost reduction variable mapped to threadIdx.x
   std::vector<Promotion> promotions;
   int64_t accCount = 1;              // register-tile size
+  // Matrix-core mapping of a dense contraction `out +=! A * B` (useMfma): parallel variables
+  // found only in A form the M side, only in B the N side, the rest are batch; each wavefront
+  // computes 16x16 output tiles with v_mfma_f32_16x16x4_f32 over the flattened reduction.
+  bool mfma = false;
+  std::vector<std::string> mfmaM, mfmaN, mfmaBatch, mfmaK;
+  bool mfmaSwapOperands = false;     // the first factor of the product is the N-side operand
+  int64_t waves = 1;
 };
 
 struct KernelPlan {

@@ -1,0 +1,101 @@
+"""Matrix-core (v_mfma_f32_16x16x4_f32) emission for dense contractions against the oracle:
+lane layout, partial tiles in M, N and K, batch variables, epilogues, accumulation into existing
+outputs.  Integer-valued inputs make the comparison bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+import tensorcomprehensions_amd as tc
+from oracle import tc_oracle
+from tests import workloads as W
+
+pytestmark = pytest.mark.gpu
+
+MM = "def matmul(float(M, K) A, float(K, N) B) -> (C) { C(m, n) +=! A(m, r_k) * B(r_k, n) }"
+TMM = "def tmm(float(M, K) A, float(N, K) B) -> (C) { C(m, n) +=! A(m, r_k) * B(n, r_k) }"
+
+
+def run(src, entry, ins_np, options, outs_init=None):
+    ins = [torch.from_numpy(a).cuda() for a in ins_np]
+    ex = tc.compile(src, entry, ins, options)
+    assert "__builtin_amdgcn_mfma_f32_16x16x4f32" in ex.compiled_source
+    outs = tc.prepare_outputs(src, entry, ins)
+    for i, o in enumerate(outs):
+        if outs_init is not None:
+            o.copy_(torch.from_numpy(outs_init[i]))
+        else:
+            o.fill_(float("nan"))
+    tc.run(ex, ins, outs)
+    torch.cuda.synchronize()
+    return [o.cpu().numpy() for o in outs]
+
+
+def ints(shape, seed):
+    return np.random.Generator(np.random.Philox(seed)).integers(-4, 5, size=shape).astype(np.float32)
+
+
+@pytest.mark.parametrize("m,k,n", [(16, 4, 16), (16, 16, 16), (32, 8, 48), (26, 72, 26), (5, 3, 7), (17, 33, 65), (64, 130, 20)])
+@pytest.mark.parametrize("waves", [1, 4])
+def test_matmul_shapes_exact(m, k, n, waves):
+    print(f"mfma matmul {m}x{k}x{n} waves={waves}", flush=True)
+    A, B = ints((m, k), m * 100 + k), ints((k, n), n)
+    opts = f"naive;tile=32,32;mapToThreads=64,{waves};mapToBlocks=64,64;useMfma=1"
+    (C,) = run(MM, "matmul", [A, B], opts)
+    assert np.array_equal(C, A @ B)
+    (Ct,) = run(TMM, "tmm", [A, np.ascontiguousarray(B.T)], opts)
+    assert np.array_equal(Ct, A @ B)
+
+
+def test_matmul_with_lds_operands_and_untiled_problem():
+    A, B = ints((50, 40), 1), ints((40, 30), 2)
+    (C,) = run(MM, "matmul", [A, B], "naive;tile=0,0;mapToThreads=64,2;mapToBlocks=1;useMfma=1;useSharedMemory=1")
+    assert np.array_equal(C, A @ B)
+
+
+def test_accumulate_into_existing_output():
+    src = "def mmacc(float(M, K) A, float(K, N) B) -> (C) { C(m, n) += A(m, r_k) * B(r_k, n) }"
+    A, B = ints((20, 12), 3), ints((12, 18), 4)
+    C0 = ints((20, 18), 5)
+    (C,) = run(src, "mmacc", [A, B], "naive;tile=32,32;mapToThreads=64;useMfma=1", outs_init=[C0])
+    assert np.array_equal(C, C0 + A @ B)
+
+
+@pytest.mark.parametrize("opts", [
+    "naive;tile=1,26,26;mapToThreads=64,4;mapToBlocks=500;useMfma=1",
+    "naive;tile=1,26,26;mapToThreads=64,4;mapToBlocks=500;useMfma=1;useSharedMemory=1",
+    "naive;tile=2,26,26;mapToThreads=64,8;mapToBlocks=500;useMfma=1;useSharedMemory=1",
+])
+def test_batch_matmul(opts):
+    X, Y = ints((9, 26, 72), 6), ints((9, 72, 26), 7)
+    (Z,) = run(W.BATCH_MATMUL, "batch_matmul", [X, Y], opts)
+    assert np.array_equal(Z, np.einsum("bnm,bmk->bnk", X, Y))
+
+
+@pytest.mark.parametrize("opts", [
+    "naive;tile=1,1,16,14,14;mapToThreads=64,4;mapToBlocks=32,32;useMfma=1;useSharedMemory=1",
+    "naive;tile=1,1,16,14,14;mapToThreads=64,2;mapToBlocks=32,32;useMfma=1",
+    "naive;tile=1,2,8,7,14;mapToThreads=64,4;mapToBlocks=32,32;useMfma=1;useSharedMemory=1",
+])
+def test_group_convolution_with_bias_epilogue(opts):
+    I, Wt, B = ints((3, 4, 6, 16, 16), 8), ints((4, 16, 6, 3, 3), 9), ints((4, 16), 10)
+    (O,) = run(W.GROUP_CONVOLUTION, "group_convolution", [I, Wt, B], opts)
+    (ref,) = tc_oracle.run(W.GROUP_CONVOLUTION, "group_convolution", [I, Wt, B])
+    assert np.array_equal(O, ref)
+
+
+def test_full_size_configs_within_tolerance():
+    for name, opts in (("c3_batch_matmul", "naive;tile=1,26,26;mapToThreads=64,4;mapToBlocks=500;useMfma=1;useSharedMemory=1"),
+                       ("c4_group_convolution", "naive;tile=1,1,16,14,14;mapToThreads=64,4;mapToBlocks=32,32;useMfma=1;useSharedMemory=1")):
+        src, entry, _, _, k = W.CONFIGS[name]
+        ins = W.make_inputs(name)
+        got = run(src, entry, ins, opts)
+        ref = tc_oracle.run(src, entry, ins)
+        for g, r in zip(got, ref):
+            assert np.abs(g - r).max() <= W.tolerance(k, r), name
+
+
+def test_non_contractions_fall_back_to_the_vector_path():
+    src = "def add(float(N, M) A, float(N, M) B) -> (C) { C(n, m) = A(n, m) + B(n, m) }"
+    A = torch.randn(32, 32, device="cuda")
+    ex = tc.compile(src, "add", [A, A], "naive;useMfma=1")
+    assert "mfma" not in ex.compiled_source
