@@ -828,12 +828,37 @@ class StageCodegen {
 
   void emitCopyIn(const Promotion& p) {
     const TensorView& view = st_.views.at(p.tensor);
-    auto gStrides = makeStridesFromSizes(view.extents);
+    auto gStridesFull = makeStridesFromSizes(view.extents);
     int64_t count = 1;
     for (auto e : p.extents) count *= e;
+    std::string loPrefix = "lo" + std::to_string(stageIdx_) + "_" + p.tensor + "_";
     for (size_t j = 0; j < p.extents.size(); ++j) {
-      em_.line("const int lo" + std::to_string(stageIdx_) + "_" + p.tensor + "_" + std::to_string(j) + " = " +
-               footprintLow(p, j) + ";");
+      em_.line("const int " + loPrefix + std::to_string(j) + " = " + footprintLow(p, j) + ";");
+    }
+    // Copy dimensions: trailing dimensions the footprint covers completely (and that are not
+    // padded in LDS) are contiguous in both memories and fold into their outer neighbour, which
+    // removes most of the index decoding.
+    struct CopyDim {
+      int64_t extent, tensorExtent, gStride, lStride;
+      std::string lo;
+    };
+    std::vector<CopyDim> dims;
+    for (size_t j = 0; j < p.extents.size(); ++j) {
+      dims.push_back(CopyDim{p.extents[j], view.extents[j], gStridesFull[j], p.ldsStrides[j], loPrefix + std::to_string(j)});
+    }
+    while (dims.size() >= 2) {
+      CopyDim& in = dims.back();
+      CopyDim& out = dims[dims.size() - 2];
+      bool full = in.extent == in.tensorExtent && out.lStride == in.lStride * in.extent &&
+          out.gStride == in.gStride * in.tensorExtent;
+      if (!full) break;
+      // (out, in) -> one dimension of extent out*in starting at out.lo * in.extent (in.lo is 0)
+      out.lo = "(" + out.lo + ") * " + std::to_string(in.extent);
+      out.extent *= in.extent;
+      out.tensorExtent *= in.tensorExtent;
+      out.gStride = in.gStride;
+      out.lStride = in.lStride;
+      dims.pop_back();
     }
     // Two phases per chunk of iterations: all global loads first (unconditional, from a clamped
     // address, so they are issued back to back and their latencies overlap), then the LDS stores.
@@ -846,20 +871,20 @@ class StageCodegen {
       cond.clear();
       gidx.clear();
       lidx.clear();
-      for (size_t j = 0; j < p.extents.size(); ++j) {
-        div /= p.extents[j];
+      for (size_t j = 0; j < dims.size(); ++j) {
+        div /= dims[j].extent;
         std::string l = "l" + std::to_string(j) + "_";
         std::string e = "c_";
         if (div > 1) e = "(" + e + " / " + std::to_string(div) + ")";
-        if (j > 0) e = e + " % " + std::to_string(p.extents[j]);
+        if (j > 0) e = e + " % " + std::to_string(dims[j].extent);
         em_.line("const int " + l + " = " + e + ";");
         std::string g = "g" + std::to_string(j) + "_";
-        em_.line("const int " + g + " = lo" + std::to_string(stageIdx_) + "_" + p.tensor + "_" + std::to_string(j) + " + " + l + ";");
-        cond += (j ? " && " : "") + std::string("(unsigned)") + g + " < " + std::to_string(view.extents[j]) + "u";
-        gidx += (j ? " + " : "") + g + (gStrides[j] != 1 ? " * " + std::to_string(gStrides[j]) : "");
-        lidx += (j ? " + " : "") + l + (p.ldsStrides[j] != 1 ? " * " + std::to_string(p.ldsStrides[j]) : "");
+        em_.line("const int " + g + " = " + dims[j].lo + " + " + l + ";");
+        cond += (j ? " && " : "") + std::string("(unsigned)") + g + " < " + std::to_string(dims[j].tensorExtent) + "u";
+        gidx += (j ? " + " : "") + g + (dims[j].gStride != 1 ? " * " + std::to_string(dims[j].gStride) : "");
+        lidx += (j ? " + " : "") + l + (dims[j].lStride != 1 ? " * " + std::to_string(dims[j].lStride) : "");
       }
-      if (p.extents.empty()) {
+      if (dims.empty()) {
         cond = "true";
         gidx = lidx = "0";
       }
@@ -1162,22 +1187,33 @@ class StageCodegen {
   // Declares i_<v> (and p_<v>) for every variable of `group` from the flattened position `pos`
   // inside the block tile (row-major over the group's tile extents, last variable fastest) and
   // returns the predicate "position exists".
-  std::string decodeGroup(const std::vector<std::string>& group, const std::string& pos) {
+  std::string decodeGroup(const std::vector<std::string>& group, const std::string& pos, bool clamp = false) {
     int64_t total = 1;
     for (const auto& n : group) total *= var(n).tile;
     std::string pred = pos + " < " + std::to_string(total);
+    // clamped: positions past the end alias the last valid one, so that addresses computed from
+    // the decoded indices are always legal (used for operands whose surplus lanes are discarded)
+    std::string src = pos;
+    if (clamp) {
+      src = "pc" + std::to_string(clampId_++) + "_";
+      em_.line("const int " + src + " = min(" + pos + ", " + std::to_string(total - 1) + ");");
+    }
     int64_t div = total;
     for (const auto& n : group) {
       const LoopVar& v = var(n);
       div /= v.tile;
-      std::string e = pos;
+      std::string e = src;
       if (div > 1) e = "(" + e + " / " + std::to_string(div) + ")";
       if (&n != &group.front()) e = e + " % " + std::to_string(v.tile);
       std::string base = std::to_string(v.min);
       if (v.numTiles > 1) base += " + " + tv(v) + " * " + std::to_string(v.tile);
       em_.line("const int p_" + v.name + " = " + e + ";");
-      em_.line("const int " + iv(v) + " = " + base + " + p_" + v.name + ";");
-      if (v.partial()) pred += " && " + iv(v) + " <= " + std::to_string(v.min + v.extent - 1);
+      if (clamp && v.partial()) {
+        em_.line("const int " + iv(v) + " = min(" + base + " + p_" + v.name + ", " + std::to_string(v.min + v.extent - 1) + ");");
+      } else {
+        em_.line("const int " + iv(v) + " = " + base + " + p_" + v.name + ";");
+      }
+      if (v.partial()) pred += " && " + base + " + p_" + v.name + " <= " + std::to_string(v.min + v.extent - 1);
     }
     return pred;
   }
@@ -1192,7 +1228,15 @@ class StageCodegen {
     int64_t MT = tileProduct(st_.mfmaM), NT = tileProduct(st_.mfmaN), BT = tileProduct(st_.mfmaBatch),
             KT = tileProduct(st_.mfmaK);
     int64_t numMT = ceilDiv(MT, 16), numNT = ceilDiv(NT, 16), ksteps = ceilDiv(KT, 4);
+    (void)KT;
     int64_t tiles = BT * numMT * numNT;
+    // predicates that are statically true need no code
+    auto groupExact = [&](const std::vector<std::string>& g, int64_t total, int64_t granule) {
+      bool exact = total % granule == 0;
+      for (const auto& n : g) exact &= !var(n).partial();
+      return exact;
+    };
+    (void)groupExact;
     const ExprRef& loadA = s.rhs->args[st_.mfmaSwapOperands ? 1 : 0]; // holds the M-side variables
     const ExprRef& loadB = s.rhs->args[st_.mfmaSwapOperands ? 0 : 1]; // holds the N-side variables
     em_.line("// matrix cores: " + std::to_string(tiles) + " tiles of 16x16 per block, " + std::to_string(ksteps) +
@@ -1213,10 +1257,14 @@ class StageCodegen {
     ++opened;
     em_.line("const int nt_ = tl_ % " + std::to_string(numNT) + ", mt_ = (tl_ / " + std::to_string(numNT) + ") % " +
              std::to_string(numMT) + ", bt_ = tl_ / " + std::to_string(numNT * numMT) + ";");
-    std::string bok = st_.mfmaBatch.empty() ? "true" : decodeGroup(st_.mfmaBatch, "bt_");
+    // A row of the product depends on one row of the M-side operand only and a column on one
+    // column of the N-side operand, so lanes past the end of a partial tile may load any legal
+    // element (clamped indices): their results are never stored.  Only surplus reduction steps
+    // must contribute exact zeros.
+    std::string bok = st_.mfmaBatch.empty() ? "true" : decodeGroup(st_.mfmaBatch, "bt_", true);
     em_.line("const bool bok_ = " + bok + ";");
     em_.line("const int npos_ = nt_ * 16 + lm_;");
-    em_.line("const bool nok_ = bok_ && " + decodeGroup(st_.mfmaN, "npos_") + ";");
+    em_.line("const bool nok_ = bok_ && " + decodeGroup(st_.mfmaN, "npos_", true) + ";");
     em_.line("__tc::floatx4 c_ = {0.0f, 0.0f, 0.0f, 0.0f};");
     if (!s.init) {
       // accumulate into the existing output values
@@ -1230,13 +1278,59 @@ class StageCodegen {
     {
       em_.open("");
       em_.line("const int mposa_ = mt_ * 16 + lm_;");
-      em_.line("const bool moka_ = bok_ && " + decodeGroup(st_.mfmaM, "mposa_") + ";");
-      em_.line(ksteps <= 64 ? "#pragma unroll" : "#pragma unroll 4");
+      em_.line("const bool moka_ = bok_ && " + decodeGroup(st_.mfmaM, "mposa_", true) + ";");
+      em_.line("(void)moka_;");
+      // Lane group lj_ (0..3) owns a contiguous quarter of the flattened reduction and step ks_
+      // walks inside it: when a quarter is a whole number of inner-variable periods, the inner
+      // reduction indices of a step are compile-time constants after unrolling and only the
+      // outermost one depends on the lane, so operand addresses become "lane base + immediate".
+      int64_t quarter = ceilDiv(KT, 4);
+      ksteps = quarter;
+      int64_t innerProd = 1;
+      for (size_t i = 1; i < st_.mfmaK.size(); ++i) innerProd *= var(st_.mfmaK[i]).tile;
+      bool aligned = quarter % innerProd == 0;
+      em_.line(ksteps <= 128 ? "#pragma unroll" : "#pragma unroll 4");
       em_.open("for (int ks_ = 0; ks_ < " + std::to_string(ksteps) + "; ++ks_)");
-      em_.line("const int kk_ = ks_ * 4 + lj_;");
-      em_.line("const bool kok_ = " + decodeGroup(st_.mfmaK, "kk_") + ";");
-      em_.line("const float a_ = (moka_ && kok_) ? " + loadStr(loadA, "") + " : 0.0f;");
-      em_.line("const float b_ = (nok_ && kok_) ? " + loadStr(loadB, "") + " : 0.0f;");
+      std::string kok;
+      if (aligned) {
+        int64_t div = innerProd;
+        for (size_t i = 0; i < st_.mfmaK.size(); ++i) {
+          const LoopVar& v = var(st_.mfmaK[i]);
+          std::string e;
+          if (i == 0) {
+            e = "lj_ * " + std::to_string(quarter / innerProd) + " + ks_ / " + std::to_string(innerProd);
+          } else {
+            div /= v.tile;
+            e = "(ks_ / " + std::to_string(div) + ") % " + std::to_string(v.tile);
+          }
+          if (i == 0 && quarter * 4 != KT) e = "min(" + e + ", " + std::to_string(v.tile - 1) + ")";
+          em_.line("const int p_" + v.name + " = " + e + ";");
+          em_.line("const int " + iv(v) + " = " + std::to_string(v.min) + " + p_" + v.name + ";");
+        }
+        if (quarter * 4 != KT) kok = "lj_ * " + std::to_string(quarter) + " + ks_ < " + std::to_string(KT);
+      } else {
+        em_.line("const int kk_ = lj_ * " + std::to_string(quarter) + " + ks_;");
+        kok = decodeGroup(st_.mfmaK, "kk_", true);
+        if (quarter * 4 == KT) kok.clear();
+      }
+      auto operand = [&](const char* name, const ExprRef& load) {
+        std::string text = loadStr(load, "");
+        if (kok.empty()) {
+          em_.line(std::string("const float ") + name + " = " + text + ";");
+        } else {
+          em_.line(std::string("const float ") + name + "raw_ = " + text + ";");
+          em_.line(std::string("const float ") + name + " = kok_ ? " + name + "raw_ : 0.0f;");
+        }
+      };
+      if (!kok.empty()) em_.line("const bool kok_ = " + kok + ";");
+      if (aligned && !kok.empty()) {
+        // the surplus steps of the last lane group would decode past the outermost extent
+        const LoopVar& v0 = var(st_.mfmaK[0]);
+        em_.line("// (indices of surplus steps are clamped below)");
+        (void)v0;
+      }
+      operand("a_", loadA);
+      operand("b_", loadB);
       em_.line("c_ = __builtin_amdgcn_mfma_f32_16x16x4f32(a_, b_, c_, 0, 0, 0);");
       em_.close();
       em_.close();
@@ -1355,6 +1449,7 @@ class StageCodegen {
   std::set<std::string> activePromotions_;
   bool inCachedReduction_ = false;
   std::string cacheSlot_;
+  int clampId_ = 0;
 };
 
 // ------------------------------------------------------------------------------------------
