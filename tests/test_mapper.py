@@ -48,7 +48,7 @@ def test_collapse_and_vector_lanes():
     assert "i_h_w" not in src and "i_w" in src
     # 17*25 = 425 is not a multiple of 4: lanes are dropped, the code stays scalar
     src, _ = mapped(W.TENSORDOT, "tensordot", [(2, 3, 4, 17, 25), (2, 4, 2, 17, 25)], MappingOptions.naive().vectorWidth(4))
-    assert "i_h_w" in src and "_v" not in src
+    assert "i_h_w" in src and "i_h_w_v" not in src
     # the convolution's h and w are not jointly contiguous in the input (windows): no merge
     src, _ = mapped(W.GROUP_CONVOLUTION, "group_convolution", [(2, 2, 4, 8, 8), (2, 4, 4, 3, 3), (2, 4)], "naive")
     assert "i_h_w" not in src
