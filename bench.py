@@ -65,14 +65,44 @@ def measure(name, steps, warmup, options=None):
     }
 
 
+COPY_TC = "def copy(float(N) I) -> (O) { O(i) = I(i) }"
+COPY_ELEMS = 64 * 1024 * 1024           # 256 MiB read + 256 MiB written per launch
+
+
+def calibrate_copy(steps):
+    """A plain copy through the same backend: what FETCH_SIZE / WRITE_SIZE read for a kernel whose
+    HBM traffic is known (268 435 456 B each way) scales the counters of the measured kernel."""
+    import torch
+    import tensorcomprehensions_amd as tc
+    src = torch.ones(COPY_ELEMS, device="cuda")
+    ex = tc.compile(COPY_TC, "copy", [src], "naive;tile=4096;mapToThreads=256;mapToBlocks=16384;vectorWidth=4;unroll=16")
+    (dst,) = tc.prepare_outputs(COPY_TC, "copy", [src])
+    us = tc.profile_repeated(ex, [src], [dst], steps) / steps
+    torch.cuda.synchronize()
+    sys.stderr.write(f"copy calibration: {2 * 4 * COPY_ELEMS / us / 1e3:.1f} GB/s, {us:.1f} us per launch\n")
+
+
+def measured_traffic(name):
+    """HBM bytes per launch from the committed counter summary of this workload, if there is one."""
+    short = {"c2_tensordot": "tensordot_c2", "c3_batch_matmul": "batch_matmul_c3",
+             "c4_group_convolution": "group_convolution_c4", "c5_moments": "moments_c5"}.get(name)
+    path = os.path.join(ROOT, "profiles", f"{short}_hbm_traffic.txt")
+    if not short or not os.path.exists(path):
+        return None
+    for line in open(path):
+        if line.startswith("traffic_bytes_per_launch:"):
+            return int(line.split(":")[1])
+    return None
+
+
 def roofline(m):
     gbs = m["bytes"] / (m["kernel_ms"] * 1e-3) / 1e9
     tfl = m["flops"] / (m["kernel_ms"] * 1e-3) / 1e12
     if "group_convolution" in m["name"]:
         return {"bound": "mfma", "achieved": round(tfl, 3), "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(tfl / FP32_PEAK_TFLOPS, 4), "traffic": None}
+                "frac": round(tfl / FP32_PEAK_TFLOPS, 4), "traffic": measured_traffic(m["name"])}
     return {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}
+            "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": measured_traffic(m["name"])}
 
 
 def cpu_baseline(name, budget_s=15.0):
@@ -102,6 +132,8 @@ def main():
     ap.add_argument("--options", default=None)
     ap.add_argument("--all", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also launch a plain copy kernel of known size (reference point for HBM byte counters)")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py measures one GPU: this backend has no multi-GPU path (run with --gpus 1)")
@@ -109,6 +141,8 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     from tests import workloads as W
 
+    if a.calibrate:
+        calibrate_copy(a.steps)
     m = measure(a.config, a.steps, a.warmup, a.options)
     value = m["bytes"] * a.steps / m["wall_s"] / 1e9
     line = {
