@@ -61,7 +61,9 @@ TuningConfiguration::TuningConfiguration()
       privateDepth({0}, "pdepth"),
       sharedDepth({0}, "sdepth"),
       vectorWidth({1, 2, 4}, "vector width"),
-      collapseContiguous(RangeParameter::boolean("collapse contiguous")) {
+      collapseContiguous(RangeParameter::boolean("collapse contiguous")),
+      useMfma(RangeParameter::boolean("use mfma")),
+      prefetchShared(RangeParameter::boolean("prefetch shared")) {
   tilingParams.setRange(1, 1, "t", {0}, "t");
   blockParams.setRange(1, 3, "b", {1}, "b");
   gridParams.setRange(1, 3, "g", {1}, "g");
@@ -88,7 +90,7 @@ std::vector<RangeParameter*> TuningConfiguration::collectParameters() {
   multi(gridParams);
   for (auto* x : {&unrollFactor, &tileImperfectlyNested, &useSharedMemory, &usePrivateMemory, &unrollCopyShared,
                   &useReadOnlyCache, &matchLibraryCalls, &privateDepth, &sharedDepth, &vectorWidth,
-                  &collapseContiguous}) {
+                  &collapseContiguous, &useMfma, &prefetchShared}) {
     p.push_back(x);
   }
   return p;
@@ -124,6 +126,8 @@ void TuningConfiguration::fromHipMappingOptions(const HipMappingOptions& o) {
   sharedDepth.selectFromValue(o.sharedDepthValue);
   vectorWidth.selectFromValue(o.vectorWidthValue);
   collapseContiguous.selectFromValue(o.collapseContiguousValue);
+  useMfma.selectFromValue(o.useMfmaValue);
+  prefetchShared.selectFromValue(o.prefetchSharedValue);
 }
 
 void TuningConfiguration::applyToHipMappingOptions(HipMappingOptions& o) const {
@@ -145,6 +149,8 @@ void TuningConfiguration::applyToHipMappingOptions(HipMappingOptions& o) const {
   o.sharedDepth(static_cast<uint32_t>(sharedDepth.value()));
   o.vectorWidth(static_cast<uint32_t>(vectorWidth.value()));
   o.collapseContiguous(collapseContiguous.value());
+  o.useMfma(useMfma.value());
+  o.prefetchShared(prefetchShared.value());
 }
 
 void TuningConfiguration::fixParameters(const TuningParameterFixer& f) {

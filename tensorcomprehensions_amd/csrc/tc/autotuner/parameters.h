@@ -83,7 +83,7 @@ class TuningConfiguration {
   RangeParameter tileImperfectlyNested;
   RangeParameter useSharedMemory, usePrivateMemory, unrollCopyShared, useReadOnlyCache, matchLibraryCalls;
   RangeParameter privateDepth, sharedDepth;
-  RangeParameter vectorWidth, collapseContiguous;
+  RangeParameter vectorWidth, collapseContiguous, useMfma, prefetchShared;
 
  private:
   std::vector<std::function<bool(const TuningConfiguration&)>> validators_;

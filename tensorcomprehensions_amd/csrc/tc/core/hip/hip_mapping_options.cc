@@ -35,7 +35,7 @@ std::string HipMappingOptions::toText() const {
   if (hasPrivateDepth) ss << ";privateDepth=" << privateDepthValue;
   if (hasSharedDepth) ss << ";sharedDepth=" << sharedDepthValue;
   ss << ";vectorWidth=" << vectorWidthValue << ";collapseContiguous=" << collapseContiguousValue
-     << ";useMfma=" << useMfmaValue;
+     << ";useMfma=" << useMfmaValue << ";prefetchShared=" << prefetchSharedValue;
   return ss.str();
 }
 
@@ -86,6 +86,7 @@ HipMappingOptions HipMappingOptions::fromText(const std::string& text) {
     else if (k == "vectorWidth") o.vectorWidth(static_cast<uint32_t>(std::stoul(v)));
     else if (k == "collapseContiguous") o.collapseContiguous(b());
     else if (k == "useMfma") o.useMfma(b());
+    else if (k == "prefetchShared") o.prefetchShared(b());
     else TC_CHECK(false) << "unknown mapping option '" << k << "'";
   }
   return o;
@@ -126,7 +127,8 @@ std::ostream& operator<<(std::ostream& os, const HipMappingOptionsAsCpp& p) {
   if (o.hasSharedDepth) os << in << ".sharedDepth(" << o.sharedDepthValue << ")\n";
   os << in << ".vectorWidth(" << o.vectorWidthValue << ")\n"
      << in << ".collapseContiguous(" << bs(o.collapseContiguousValue) << ")\n"
-     << in << ".useMfma(" << bs(o.useMfmaValue) << ")";
+     << in << ".useMfma(" << bs(o.useMfmaValue) << ")\n"
+     << in << ".prefetchShared(" << bs(o.prefetchSharedValue) << ")";
   return os;
 }
 

@@ -7,7 +7,9 @@
 //   * presets use blocks that are multiples of the 64-lane wavefront,
 //   * extra fields (numbers 11+ on the wire): vectorWidth (adjacent elements per thread along the
 //     contiguous dimension), collapseContiguous (merge loop dimensions that are jointly contiguous
-//     in every tensor before mapping), useMfma (matrix-core tiles for dense contractions).
+//     in every tensor before mapping), useMfma (matrix-core tiles for dense contractions),
+//     prefetchShared (software-pipelined LDS staging: the next block tile's global loads are
+//     in flight while the current one is computed).
 #pragma once
 #include <algorithm>
 #include <array>
@@ -80,6 +82,7 @@ class HipMappingOptions : public GenericOptionsFluent<HipMappingOptions> {
   uint32_t vectorWidthValue = 1;
   bool collapseContiguousValue = true;
   bool useMfmaValue = false;
+  bool prefetchSharedValue = false;
 
   HipMappingOptions() = default;
   // from a serialized HipMappingOptionsProto
@@ -92,7 +95,8 @@ class HipMappingOptions : public GenericOptionsFluent<HipMappingOptions> {
         (!hasMaxSharedMemory || maxSharedMemoryValue == o.maxSharedMemoryValue) &&
         useReadOnlyCacheValue == o.useReadOnlyCacheValue && privateDepthValue == o.privateDepthValue &&
         sharedDepthValue == o.sharedDepthValue && vectorWidthValue == o.vectorWidthValue &&
-        collapseContiguousValue == o.collapseContiguousValue && useMfmaValue == o.useMfmaValue;
+        collapseContiguousValue == o.collapseContiguousValue && useMfmaValue == o.useMfmaValue &&
+        prefetchSharedValue == o.prefetchSharedValue;
   }
   bool operator!=(const HipMappingOptions& o) const { return !(*this == o); }
 
@@ -140,6 +144,7 @@ class HipMappingOptions : public GenericOptionsFluent<HipMappingOptions> {
   }
   HipMappingOptions& collapseContiguous(bool b) { collapseContiguousValue = b; return *this; }
   HipMappingOptions& useMfma(bool b) { useMfmaValue = b; return *this; }
+  HipMappingOptions& prefetchShared(bool b) { prefetchSharedValue = b; return *this; }
 
   std::string toProtobufSerializedString() const {
     protowire::Writer w;
@@ -156,6 +161,7 @@ class HipMappingOptions : public GenericOptionsFluent<HipMappingOptions> {
     w.varint(11, vectorWidthValue);
     w.boolean(12, collapseContiguousValue);
     w.boolean(13, useMfmaValue);
+    w.boolean(14, prefetchSharedValue);
     return w.str();
   }
   void fromProto(const std::string& s) {
@@ -175,6 +181,7 @@ class HipMappingOptions : public GenericOptionsFluent<HipMappingOptions> {
         case 11: vectorWidthValue = static_cast<uint32_t>(r.value()); break;
         case 12: collapseContiguousValue = r.value() != 0; break;
         case 13: useMfmaValue = r.value() != 0; break;
+        case 14: prefetchSharedValue = r.value() != 0; break;
         default: break;
       }
     }

@@ -529,7 +529,15 @@ class StageCodegen {
 
   // --- naming -------------------------------------------------------------------------------
   std::string iv(const LoopVar& v) const { return "i_" + v.name; }
-  std::string tv(const LoopVar& v) const { return v.numTiles > 1 ? "t_" + v.name : "0"; }
+  std::string tv(const LoopVar& v) const {
+    auto it = tileOverride.find(v.name);
+    if (it != tileOverride.end()) return it->second;
+    return v.numTiles > 1 ? "t_" + v.name : "0";
+  }
+  // while emitting the loads of a prefetched tile: tile-index expression to use for a variable
+  std::map<std::string, std::string> tileOverride;
+  // LDS staging is driven by the kernel-level pipeline: stages only declare footprint origins
+  bool suppressCopy = false;
 
   const LoopVar& var(const std::string& n) const {
     for (const auto& v : st_.vars) {
@@ -599,6 +607,10 @@ class StageCodegen {
       }
     }
     std::string global = "p" + e->name + "[" + flatIndex(e->name, e->args, accRef) + "]";
+    if (kc_.opts.useReadOnlyCacheValue && !st_.views.at(e->name).isOutput && ntLoads_) {
+      // streaming read of an input that is never written: keep it out of the way of cached data
+      global = "__builtin_nontemporal_load(&" + global + ")";
+    }
     if (inCachedReduction_) {
       auto it = regCaches.find(global);
       if (it != regCaches.end()) {
@@ -826,6 +838,85 @@ class StageCodegen {
     }
   }
 
+  std::string loPrefix(const Promotion& p) const { return "lo" + std::to_string(stageIdx_) + "_" + p.tensor + "_"; }
+
+  void declareLows(const Promotion& p) {
+    for (size_t j = 0; j < p.extents.size(); ++j) {
+      em_.line("const int " + loPrefix(p) + std::to_string(j) + " = " + footprintLow(p, j) + ";");
+    }
+  }
+
+  int64_t copyIterations(const Promotion& p) const {
+    int64_t count = 1;
+    for (auto e : p.extents) count *= e;
+    return ceilDiv(count, kc_.NT());
+  }
+
+  // Whole-footprint variants used by the software pipeline: every thread keeps its share of the
+  // tile in `regs` between the load and the store phase.  Footprint origins must be in scope.
+  void emitCopyLoads(const Promotion& p, const std::string& regs) { emitCopyPhase(p, regs, true); }
+  void emitCopyStores(const Promotion& p, const std::string& regs) { emitCopyPhase(p, regs, false); }
+
+  struct CopyDim {
+    int64_t extent, tensorExtent, gStride, lStride;
+    std::string lo;
+  };
+  std::vector<CopyDim> copyDims(const Promotion& p) const {
+    const TensorView& view = st_.views.at(p.tensor);
+    auto gStridesFull = makeStridesFromSizes(view.extents);
+    std::vector<CopyDim> dims;
+    for (size_t j = 0; j < p.extents.size(); ++j) {
+      dims.push_back(CopyDim{p.extents[j], view.extents[j], gStridesFull[j], p.ldsStrides[j], loPrefix(p) + std::to_string(j)});
+    }
+    while (dims.size() >= 2) {
+      CopyDim& in = dims.back();
+      CopyDim& out = dims[dims.size() - 2];
+      bool full = in.extent == in.tensorExtent && out.lStride == in.lStride * in.extent &&
+          out.gStride == in.gStride * in.tensorExtent;
+      if (!full) break;
+      out.lo = "(" + out.lo + ") * " + std::to_string(in.extent);
+      out.extent *= in.extent;
+      out.tensorExtent *= in.tensorExtent;
+      out.gStride = in.gStride;
+      out.lStride = in.lStride;
+      dims.pop_back();
+    }
+    return dims;
+  }
+
+  void emitCopyPhase(const Promotion& p, const std::string& regs, bool loads) {
+    int64_t count = 1;
+    for (auto e : p.extents) count *= e;
+    std::vector<CopyDim> dims = copyDims(p);
+    em_.line("#pragma unroll");
+    em_.open("for (int it_ = 0; it_ < " + std::to_string(copyIterations(p)) + "; ++it_)");
+    em_.line("const int c_ = it_ * " + std::to_string(kc_.NT()) + " + tid_;");
+    int64_t div = count;
+    std::string cond = "c_ < " + std::to_string(count), gidx, lidx;
+    for (size_t j = 0; j < dims.size(); ++j) {
+      div /= dims[j].extent;
+      std::string l = "l" + std::to_string(j) + "_";
+      std::string e = "c_";
+      if (div > 1) e = "(" + e + " / " + std::to_string(div) + ")";
+      if (j > 0) e = e + " % " + std::to_string(dims[j].extent);
+      em_.line("const int " + l + " = " + e + ";");
+      if (loads) {
+        std::string g = "g" + std::to_string(j) + "_";
+        em_.line("const int " + g + " = " + dims[j].lo + " + " + l + ";");
+        cond += " && (unsigned)" + g + " < " + std::to_string(dims[j].tensorExtent) + "u";
+        gidx += (j ? " + " : "") + g + (dims[j].gStride != 1 ? " * " + std::to_string(dims[j].gStride) : "");
+      }
+      lidx += (j ? " + " : "") + l + (dims[j].lStride != 1 ? " * " + std::to_string(dims[j].lStride) : "");
+    }
+    if (dims.empty()) gidx = lidx = "0";
+    if (loads) {
+      em_.line(regs + "[it_] = p" + p.tensor + "[(" + cond + ") ? (" + gidx + ") : 0];");
+    } else {
+      em_.line("if (c_ < " + std::to_string(count) + ") " + p.ldsName + "[" + lidx + "] = " + regs + "[it_];");
+    }
+    em_.close();
+  }
+
   void emitCopyIn(const Promotion& p) {
     const TensorView& view = st_.views.at(p.tensor);
     auto gStridesFull = makeStridesFromSizes(view.extents);
@@ -1022,6 +1113,15 @@ class StageCodegen {
     bool anyOutside = false, anyInside = false;
     for (const auto& p : st_.promotions) (p.insideReductionTiles ? anyInside : anyOutside) = true;
     auto copyIn = [&](bool inside) {
+      if (suppressCopy && !inside) {
+        for (const auto& p : st_.promotions) {
+          if (!p.insideReductionTiles) {
+            declareLows(p);
+            activePromotions_.insert(p.tensor);
+          }
+        }
+        return;
+      }
       em_.line("__syncthreads();");
       for (const auto& p : st_.promotions) {
         if (p.insideReductionTiles == inside) {
@@ -1110,6 +1210,9 @@ class StageCodegen {
       closeN(n);
     }
   }
+
+  const std::vector<Promotion>& promotions() const { return st_.promotions; }
+  std::string promotionType(const Promotion& p) const { return st_.views.at(p.tensor).type.cName(); }
 
   // --- register caches shared between stages -----------------------------------------------------
   struct RegCache {
@@ -1245,12 +1348,19 @@ class StageCodegen {
     if (!st_.promotions.empty()) {
       em_.open("");
       ++opened;
-      em_.line("__syncthreads();");
-      for (const auto& p : st_.promotions) {
-        emitCopyIn(p);
-        activePromotions_.insert(p.tensor);
+      if (suppressCopy) {
+        for (const auto& p : st_.promotions) {
+          declareLows(p);
+          activePromotions_.insert(p.tensor);
+        }
+      } else {
+        em_.line("__syncthreads();");
+        for (const auto& p : st_.promotions) {
+          emitCopyIn(p);
+          activePromotions_.insert(p.tensor);
+        }
+        em_.line("__syncthreads();");
       }
-      em_.line("__syncthreads();");
     }
     em_.line("const int lm_ = threadIdx.x & 15, lj_ = threadIdx.x >> 4;");
     em_.open("for (int tl_ = threadIdx.y; tl_ < " + std::to_string(tiles) + "; tl_ += " + std::to_string(st_.waves) + ")");
@@ -1339,10 +1449,12 @@ class StageCodegen {
     em_.line("#pragma unroll");
     em_.open("for (int r_ = 0; r_ < 4; ++r_)");
     em_.line("const int mpos_ = mt_ * 16 + 4 * lj_ + r_;");
-    em_.line("const bool okr_ = nok_ && " + decodeGroup(st_.mfmaM, "mpos_") + ";");
+    // indices are clamped to legal points, so the epilogue's loads need no branch (four
+    // independent rows are then fetched together); only the store is predicated
+    em_.line("const bool okr_ = nok_ && " + decodeGroup(st_.mfmaM, "mpos_", true) + ";");
     em_.line(accType_.cName() + " acc_[1];");
     em_.line("acc_[0] = c_[r_];");
-    outerPred_ = "okr_";
+    outerPred_ = "";
     accValid_ = true;
     for (size_t i = 1; i < st_.stmts.size(); ++i) {
       const StageStmt& e = st_.stmts[i];
@@ -1354,11 +1466,7 @@ class StageCodegen {
         emitPointwise(e);
       }
     }
-    {
-      int n = openUnrolled();
-      em_.line("if (ok_) p" + st_.tensor + "[" + flatIndex(st_.tensor, st_.lhsSubs, "") + "] = acc_[a_];");
-      closeN(n);
-    }
+    em_.line("if (okr_) p" + st_.tensor + "[" + flatIndex(st_.tensor, st_.lhsSubs, "") + "] = acc_[0];");
     em_.close();
     closeN(opened);
     for (const auto& p : st_.promotions) activePromotions_.erase(p.tensor);
@@ -1450,6 +1558,7 @@ class StageCodegen {
   bool inCachedReduction_ = false;
   std::string cacheSlot_;
   int clampId_ = 0;
+  bool ntLoads_ = true;
 };
 
 // ------------------------------------------------------------------------------------------
@@ -1488,7 +1597,8 @@ void mapKernel(KernelCtx& kc, const DeviceLimits& limits) {
     int axis = 0;
     for (int i = 0; i < st.numParallel && i < k.sharedDepth && axis < static_cast<int>(o.grid.size()); ++i) {
       LoopVar& v = st.vars[i];
-      if (v.vectorLane) continue;
+      // a variable with a single tile has nothing to distribute and does not use up an axis
+      if (v.vectorLane || v.numTiles == 1) continue;
       v.blockAxis = axis;
       v.gridExtent = std::min<int64_t>(static_cast<int64_t>(o.grid[axis]), v.numTiles);
       gridUse[axis] = std::max(gridUse[axis], v.gridExtent);
@@ -1653,26 +1763,76 @@ void emitKernel(KernelCtx& kc, const DeviceLimits& limits, Emitter& em) {
     em.line("__shared__ double red_scratch_raw_[" + std::to_string(scratchElems) + "];");
   }
   for (auto& g : gens) g.emitLdsDecls();
-  // kernel-level tile loops over the shared parallel variables (taken from the first stage)
+  // kernel-level tile loops over the shared parallel variables (taken from the first stage):
+  // first the tile indices that are plain block ids, then the loops, outermost first
   int opened = 0;
   const StagePlan& s0 = k.stages.front();
+  std::vector<const LoopVar*> loops;
   for (int i = 0; i < k.sharedDepth && i < s0.numParallel; ++i) {
     const LoopVar& v = s0.vars[i];
     if (v.vectorLane || v.numTiles == 1) continue;
-    std::string t = "t_" + v.name;
-    if (v.blockAxis >= 0) {
-      std::string b = std::string("blockIdx.") + axisName(v.blockAxis);
-      if (v.gridExtent == v.numTiles) {
-        em.line("const int " + t + " = " + b + ";");
-      } else {
-        em.open("for (int " + t + " = " + b + "; " + t + " < " + std::to_string(v.numTiles) + "; " + t + " += " +
-                std::to_string(v.gridExtent) + ")");
-        ++opened;
-      }
+    if (v.blockAxis >= 0 && v.gridExtent == v.numTiles) {
+      em.line("const int t_" + v.name + " = blockIdx." + axisName(v.blockAxis) + ";");
     } else {
-      em.open("for (int " + t + " = 0; " + t + " < " + std::to_string(v.numTiles) + "; ++" + t + ")");
-      ++opened;
+      loops.push_back(&v);
     }
+  }
+  auto loopHeader = [&](const LoopVar& v, std::string& start, std::string& step) {
+    start = v.blockAxis >= 0 ? std::string("blockIdx.") + axisName(v.blockAxis) : "0";
+    step = v.blockAxis >= 0 ? std::to_string(v.gridExtent) : "1";
+    std::string t = "t_" + v.name;
+    return "for (int " + t + " = " + start + "; " + t + " < " + std::to_string(v.numTiles) + "; " + t + " += " + step + ")";
+  };
+  // Software pipeline over the innermost kernel-level loop (prefetchShared): the global loads of
+  // the next tile's LDS footprints are issued before the current tile is computed and land in
+  // registers; they are written to LDS after the computation, between two barriers.
+  bool pipelined = false;
+  if (kc.opts.prefetchSharedValue && k.stages.size() == 1 && !loops.empty() && !gens[0].promotions().empty()) {
+    int64_t regs = 0;
+    pipelined = true;
+    for (const auto& p : gens[0].promotions()) {
+      pipelined &= !p.insideReductionTiles;
+      regs += gens[0].copyIterations(p);
+    }
+    pipelined &= regs <= 96;
+  }
+  for (size_t li = 0; li < loops.size(); ++li) {
+    const LoopVar& v = *loops[li];
+    std::string start, step;
+    std::string header = loopHeader(v, start, step);
+    if (!(pipelined && li + 1 == loops.size())) {
+      em.open(header);
+      ++opened;
+      continue;
+    }
+    StageCodegen& g = gens[0];
+    std::string t = "t_" + v.name;
+    em.open("");
+    ++opened;
+    for (const auto& p : g.promotions()) {
+      em.line(g.promotionType(p) + " pf_" + p.tensor + "_[" + std::to_string(g.copyIterations(p)) + "];");
+    }
+    em.open("");
+    em.line("const int " + t + " = " + start + ";");
+    for (const auto& p : g.promotions()) {
+      g.declareLows(p);
+      g.emitCopyLoads(p, "pf_" + p.tensor + "_");
+    }
+    for (const auto& p : g.promotions()) g.emitCopyStores(p, "pf_" + p.tensor + "_");
+    em.close();
+    em.open(header);
+    ++opened;
+    em.line("__syncthreads();");
+    em.line("const bool more_ = " + t + " + " + step + " < " + std::to_string(v.numTiles) + ";");
+    em.open("if (more_)");
+    g.tileOverride[v.name] = "(" + t + " + " + step + ")";
+    for (const auto& p : g.promotions()) {
+      g.declareLows(p);
+      g.emitCopyLoads(p, "pf_" + p.tensor + "_");
+    }
+    g.tileOverride.clear();
+    em.close();
+    g.suppressCopy = true;
   }
   for (const auto& d : cacheDecls) em.line(d);
   for (size_t i = 0; i < k.stages.size(); ++i) {
@@ -1686,6 +1846,13 @@ void emitKernel(KernelCtx& kc, const DeviceLimits& limits, Emitter& em) {
     } else {
       gens[i].emit();
     }
+  }
+  if (pipelined) {
+    StageCodegen& g = gens[0];
+    em.line("__syncthreads();");
+    em.open("if (more_)");
+    for (const auto& p : g.promotions()) g.emitCopyStores(p, "pf_" + p.tensor + "_");
+    em.close();
   }
   if (k.stages.size() > 1 && opened > 0) em.line("__syncthreads();");
   for (int i = 0; i < opened; ++i) em.close();

@@ -75,6 +75,7 @@ class MappingOptions:
     def vectorWidth(self, n): return self._set("vectorWidth", int(n))
     def collapseContiguous(self, b): return self._set("collapseContiguous", _b(b))
     def useMfma(self, b): return self._set("useMfma", _b(b))
+    def prefetchShared(self, b): return self._set("prefetchShared", _b(b))
 
     def to_text(self):
         return ";".join(self._parts)

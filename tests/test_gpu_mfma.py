@@ -99,3 +99,35 @@ def test_non_contractions_fall_back_to_the_vector_path():
     A = torch.randn(32, 32, device="cuda")
     ex = tc.compile(src, "add", [A, A], "naive;useMfma=1")
     assert "mfma" not in ex.compiled_source
+
+
+@pytest.mark.parametrize("opts", [
+    "naive;tile=1,1,16,14,14;mapToThreads=64,4;mapToBlocks=3,2;useMfma=1;useSharedMemory=1;prefetchShared=1",
+    "naive;tile=1,1,16,14,14;mapToThreads=64,4;mapToBlocks=2,4;useMfma=1;useSharedMemory=1;prefetchShared=1",
+    "naive;tile=1,1,16,14,14;mapToThreads=64,2;mapToBlocks=1,1;useMfma=1;useSharedMemory=1;prefetchShared=1",
+])
+def test_prefetched_lds_staging_matches(opts):
+    """Software-pipelined staging: blocks loop over several tiles, loading the next tile's
+    footprints while the current one is computed."""
+    I, Wt, B = ints((3, 4, 6, 16, 16), 18), ints((4, 16, 6, 3, 3), 19), ints((4, 16), 20)
+    ins = [torch.from_numpy(a).cuda() for a in (I, Wt, B)]
+    ex = tc.compile(W.GROUP_CONVOLUTION, "group_convolution", ins, opts)
+    assert "more_" in ex.compiled_source
+    (O,) = tc.prepare_outputs(W.GROUP_CONVOLUTION, "group_convolution", ins)
+    O.fill_(float("nan"))
+    tc.run(ex, ins, [O])
+    torch.cuda.synchronize()
+    (ref,) = tc_oracle.run(W.GROUP_CONVOLUTION, "group_convolution", [I, Wt, B])
+    assert np.array_equal(O.cpu().numpy(), ref)
+
+
+def test_prefetched_lds_staging_on_the_vector_path():
+    X, Y = ints((9, 26, 72), 26), ints((9, 72, 26), 27)
+    opts = "naive;tile=1,26,26,72;mapToThreads=26,13;mapToBlocks=2;unroll=4;useSharedMemory=1;prefetchShared=1"
+    ins = [torch.from_numpy(a).cuda() for a in (X, Y)]
+    ex = tc.compile(W.BATCH_MATMUL, "batch_matmul", ins, opts)
+    assert "more_" in ex.compiled_source and "mfma" not in ex.compiled_source
+    (Z,) = tc.prepare_outputs(W.BATCH_MATMUL, "batch_matmul", ins)
+    tc.run(ex, ins, [Z])
+    torch.cuda.synchronize()
+    assert np.array_equal(Z.cpu().numpy(), np.einsum("bnm,bmk->bnk", X, Y))
