@@ -1,31 +1,140 @@
 // Implementation of the thin HIP C ABI declared in include/tchip.h.
+//
+// The HIP runtime and hipRTC are bound at run time, not at link time: a process must talk to one
+// HIP runtime only (streams, events and modules are objects of the runtime that created them),
+// and a host framework such as PyTorch ships and loads its own copy.  The loader therefore
+// prefers a runtime that is already mapped into the process and only falls back to the system
+// one (ROCm's libamdhip64.so.N / libhiprtc.so.N).
 #include "tchip.h"
 
+#include <dlfcn.h>
 #include <hip/hip_runtime_api.h>
 #include <hip/hiprtc.h>
 
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <string>
 #include <vector>
 
 namespace {
 thread_local std::string g_lastError;
 
+struct HipApi {
+  void* hipLib = nullptr;
+  void* rtcLib = nullptr;
+  std::string loadError;
+#define TCHIP_FN(name) decltype(&::name) name = nullptr
+  TCHIP_FN(hipGetDeviceCount);
+  TCHIP_FN(hipGetDevice);
+  TCHIP_FN(hipSetDevice);
+  hipError_t (*hipGetDevicePropertiesFn)(hipDeviceProp_t*, int) = nullptr;
+  TCHIP_FN(hipDeviceSynchronize);
+  TCHIP_FN(hipStreamSynchronize);
+  TCHIP_FN(hipModuleLoadData);
+  TCHIP_FN(hipModuleGetFunction);
+  TCHIP_FN(hipModuleUnload);
+  TCHIP_FN(hipModuleLaunchKernel);
+  TCHIP_FN(hipEventCreate);
+  TCHIP_FN(hipEventRecord);
+  TCHIP_FN(hipEventSynchronize);
+  TCHIP_FN(hipEventElapsedTime);
+  TCHIP_FN(hipEventDestroy);
+  TCHIP_FN(hipGetLastError);
+  TCHIP_FN(hipGetErrorString);
+  TCHIP_FN(hiprtcCreateProgram);
+  TCHIP_FN(hiprtcCompileProgram);
+  TCHIP_FN(hiprtcGetProgramLogSize);
+  TCHIP_FN(hiprtcGetProgramLog);
+  TCHIP_FN(hiprtcGetCodeSize);
+  TCHIP_FN(hiprtcGetCode);
+  TCHIP_FN(hiprtcDestroyProgram);
+  TCHIP_FN(hiprtcGetErrorString);
+#undef TCHIP_FN
+
+  static void* openFirst(const std::vector<const char*>& names) {
+    for (const char* n : names) { // a copy the process already uses wins
+      if (void* h = dlopen(n, RTLD_NOW | RTLD_GLOBAL | RTLD_NOLOAD)) return h;
+    }
+    for (const char* n : names) {
+      if (void* h = dlopen(n, RTLD_NOW | RTLD_GLOBAL)) return h;
+    }
+    return nullptr;
+  }
+  template <typename F>
+  bool bind(void* lib, const char* sym, F& out) {
+    out = reinterpret_cast<F>(dlsym(lib, sym));
+    if (!out) loadError += std::string(loadError.empty() ? "missing symbols: " : ", ") + sym;
+    return out != nullptr;
+  }
+  HipApi() {
+    hipLib = openFirst({"libamdhip64.so", "libamdhip64.so.7", "libamdhip64.so.6", "/opt/rocm/lib/libamdhip64.so"});
+    rtcLib = openFirst({"libhiprtc.so", "libhiprtc.so.7", "libhiprtc.so.6", "/opt/rocm/lib/libhiprtc.so"});
+    if (!hipLib) loadError = "cannot load the HIP runtime (libamdhip64.so)";
+    if (!rtcLib) loadError += std::string(loadError.empty() ? "" : "; ") + "cannot load hipRTC (libhiprtc.so)";
+    if (hipLib) {
+#define TCHIP_BIND(name) bind(hipLib, #name, name)
+      TCHIP_BIND(hipGetDeviceCount);
+      TCHIP_BIND(hipGetDevice);
+      TCHIP_BIND(hipSetDevice);
+      bind(hipLib, "hipGetDevicePropertiesR0600", hipGetDevicePropertiesFn);
+      TCHIP_BIND(hipDeviceSynchronize);
+      TCHIP_BIND(hipStreamSynchronize);
+      TCHIP_BIND(hipModuleLoadData);
+      TCHIP_BIND(hipModuleGetFunction);
+      TCHIP_BIND(hipModuleUnload);
+      TCHIP_BIND(hipModuleLaunchKernel);
+      TCHIP_BIND(hipEventCreate);
+      TCHIP_BIND(hipEventRecord);
+      TCHIP_BIND(hipEventSynchronize);
+      TCHIP_BIND(hipEventElapsedTime);
+      TCHIP_BIND(hipEventDestroy);
+      TCHIP_BIND(hipGetLastError);
+      TCHIP_BIND(hipGetErrorString);
+#undef TCHIP_BIND
+    }
+    if (rtcLib) {
+#define TCHIP_BIND(name) bind(rtcLib, #name, name)
+      TCHIP_BIND(hiprtcCreateProgram);
+      TCHIP_BIND(hiprtcCompileProgram);
+      TCHIP_BIND(hiprtcGetProgramLogSize);
+      TCHIP_BIND(hiprtcGetProgramLog);
+      TCHIP_BIND(hiprtcGetCodeSize);
+      TCHIP_BIND(hiprtcGetCode);
+      TCHIP_BIND(hiprtcDestroyProgram);
+      TCHIP_BIND(hiprtcGetErrorString);
+#undef TCHIP_BIND
+    }
+  }
+};
+
+HipApi& api() {
+  static HipApi a;
+  return a;
+}
+
+constexpr int kNotLoaded = 20000;
+bool hipReady() {
+  if (api().loadError.empty()) return true;
+  g_lastError = api().loadError;
+  return false;
+}
+
 int fail(hipError_t e, const char* what) {
-  g_lastError = std::string(what) + ": " + hipGetErrorString(e);
+  g_lastError = std::string(what) + ": " + api().hipGetErrorString(e);
   return static_cast<int>(e);
 }
 int failRtc(hiprtcResult r, const char* what) {
-  g_lastError = std::string(what) + ": " + hiprtcGetErrorString(r);
+  g_lastError = std::string(what) + ": " + api().hiprtcGetErrorString(r);
   return 10000 + static_cast<int>(r);
 }
-#define TCHIP_TRY(call)                 \
-  do {                                  \
-    hipError_t e_ = (call);             \
-    if (e_ != hipSuccess) {             \
-      return fail(e_, #call);           \
-    }                                   \
+#define TCHIP_TRY(call)                   \
+  do {                                    \
+    if (!hipReady()) return kNotLoaded;   \
+    hipError_t e_ = (api().call);         \
+    if (e_ != hipSuccess) {               \
+      return fail(e_, #call);             \
+    }                                     \
   } while (0)
 
 char* dupString(const std::string& s) {
@@ -34,6 +143,17 @@ char* dupString(const std::string& s) {
     std::memcpy(p, s.c_str(), s.size() + 1);
   }
   return p;
+}
+
+// device properties through the versioned entry point; a generously sized buffer guards against
+// a runtime whose struct is larger than this build's header
+int deviceProps(int device, hipDeviceProp_t* out) {
+  if (!hipReady()) return kNotLoaded;
+  std::vector<char> buf(sizeof(hipDeviceProp_t) + 4096, 0);
+  hipError_t e = api().hipGetDevicePropertiesFn(reinterpret_cast<hipDeviceProp_t*>(buf.data()), device);
+  if (e != hipSuccess) return fail(e, "hipGetDeviceProperties");
+  std::memcpy(out, buf.data(), sizeof(hipDeviceProp_t));
+  return 0;
 }
 } // namespace
 
@@ -53,14 +173,14 @@ int tchip_set_device(int device) {
 }
 int tchip_device_name(int device, char* buf, size_t n) {
   hipDeviceProp_t p;
-  TCHIP_TRY(hipGetDeviceProperties(&p, device));
+  if (int st = deviceProps(device, &p)) return st;
   std::strncpy(buf, p.name, n);
   if (n) buf[n - 1] = '\0';
   return 0;
 }
 int tchip_device_arch(int device, char* buf, size_t n) {
   hipDeviceProp_t p;
-  TCHIP_TRY(hipGetDeviceProperties(&p, device));
+  if (int st = deviceProps(device, &p)) return st;
   std::string arch = p.gcnArchName; // "gfx950:sramecc+:xnack-"
   arch = arch.substr(0, arch.find(':'));
   std::strncpy(buf, arch.c_str(), n);
@@ -69,13 +189,13 @@ int tchip_device_arch(int device, char* buf, size_t n) {
 }
 int tchip_device_lds_bytes(int device, size_t* bytes) {
   hipDeviceProp_t p;
-  TCHIP_TRY(hipGetDeviceProperties(&p, device));
+  if (int st = deviceProps(device, &p)) return st;
   *bytes = p.sharedMemPerBlock;
   return 0;
 }
 int tchip_device_compute_units(int device, int* count) {
   hipDeviceProp_t p;
-  TCHIP_TRY(hipGetDeviceProperties(&p, device));
+  if (int st = deviceProps(device, &p)) return st;
   *count = p.multiProcessorCount;
   return 0;
 }
@@ -94,8 +214,9 @@ int tchip_rtc_compile(
   *code = nullptr;
   *codeSize = 0;
   if (log) *log = nullptr;
+  if (!hipReady()) return kNotLoaded;
   hiprtcProgram prog;
-  hiprtcResult r = hiprtcCreateProgram(&prog, source, name, 0, nullptr, nullptr);
+  hiprtcResult r = api().hiprtcCreateProgram(&prog, source, name, 0, nullptr, nullptr);
   if (r != HIPRTC_SUCCESS) {
     return failRtc(r, "hiprtcCreateProgram");
   }
@@ -104,26 +225,26 @@ int tchip_rtc_compile(
   for (int i = 0; i < numFlags; ++i) {
     opts.push_back(flags[i]);
   }
-  r = hiprtcCompileProgram(prog, static_cast<int>(opts.size()), opts.data());
+  r = api().hiprtcCompileProgram(prog, static_cast<int>(opts.size()), opts.data());
   size_t logSize = 0;
-  hiprtcGetProgramLogSize(prog, &logSize);
+  api().hiprtcGetProgramLogSize(prog, &logSize);
   std::string logText(logSize, '\0');
   if (logSize) {
-    hiprtcGetProgramLog(prog, &logText[0]);
+    api().hiprtcGetProgramLog(prog, &logText[0]);
   }
   if (log) *log = dupString(logText);
   if (r != HIPRTC_SUCCESS) {
-    hiprtcDestroyProgram(&prog);
-    g_lastError = std::string("hiprtcCompileProgram: ") + hiprtcGetErrorString(r) + "\n" + logText;
+    api().hiprtcDestroyProgram(&prog);
+    g_lastError = std::string("hiprtcCompileProgram: ") + api().hiprtcGetErrorString(r) + "\n" + logText;
     return 10000 + static_cast<int>(r);
   }
   size_t n = 0;
-  r = hiprtcGetCodeSize(prog, &n);
+  r = api().hiprtcGetCodeSize(prog, &n);
   if (r == HIPRTC_SUCCESS) {
     *code = static_cast<char*>(std::malloc(n));
-    r = *code ? hiprtcGetCode(prog, *code) : HIPRTC_ERROR_OUT_OF_MEMORY;
+    r = *code ? api().hiprtcGetCode(prog, *code) : HIPRTC_ERROR_OUT_OF_MEMORY;
   }
-  hiprtcDestroyProgram(&prog);
+  api().hiprtcDestroyProgram(&prog);
   if (r != HIPRTC_SUCCESS) {
     std::free(*code);
     *code = nullptr;
@@ -185,7 +306,8 @@ int tchip_event_destroy(tchip_event_t ev) {
   return 0;
 }
 int tchip_get_last_error(void) {
-  hipError_t e = hipGetLastError();
+  if (!hipReady()) return kNotLoaded;
+  hipError_t e = api().hipGetLastError();
   if (e != hipSuccess) {
     fail(e, "hipGetLastError");
   }
