@@ -594,6 +594,54 @@ class StageCodegen {
     return affineStr(total) + extra;
   }
 
+  // Larger than what the L2 of one XCD keeps between uses.
+  static constexpr int64_t kStreamingBytes = 4 << 20;
+
+  int64_t viewBytes(const std::string& tensor) const {
+    const TensorView& v = st_.views.at(tensor);
+    int64_t n = (v.type.bits + 7) / 8;
+    for (int64_t e : v.extents) n *= e;
+    return n;
+  }
+
+  // An operand every element of which is needed by one thread only (all parallel variables that
+  // are spread over blocks, threads or sequential tile loops occur in its subscripts) and that is
+  // too large to stay in cache anyway: loads of it carry the non-temporal hint.
+  bool streamedOnce(const std::string& tensor, const std::vector<ExprRef>& subs) const {
+    if (viewBytes(tensor) < kStreamingBytes) return false;
+    std::set<std::string> used;
+    for (const auto& sub : subs) {
+      Affine a = ir::toAffine(sub);
+      if (!a.valid) return false;
+      for (const auto& c : a.coef) {
+        if (c.second != 0) used.insert(c.first);
+      }
+    }
+    for (int i = 0; i < st_.numParallel; ++i) {
+      const LoopVar& v = st_.vars[i];
+      if (v.extent == 1 || used.count(v.name)) continue;
+      if (v.numTiles == 1 && v.threadAxis < 0) continue; // repeated inside one thread only
+      return false;
+    }
+    return true;
+  }
+
+  // The stage's result when nothing later in this kernel reads it back and it is too large to be
+  // found in cache by a later kernel: stores of it carry the non-temporal hint.
+  bool streamedStore() const {
+    if (!kc_.opts.useReadOnlyCacheValue || viewBytes(st_.tensor) < kStreamingBytes) return false;
+    for (size_t j = stageIdx_ + 1; j < kc_.k.stages.size(); ++j) {
+      if (kc_.k.stages[j].views.count(st_.tensor)) return false;
+    }
+    return true;
+  }
+
+  std::string storeStmt(const std::string& cond, const std::string& value) {
+    std::string target = "p" + st_.tensor + "[" + flatIndex(st_.tensor, st_.lhsSubs, "") + "]";
+    if (streamedStore()) return "if (" + cond + ") __builtin_nontemporal_store(" + value + ", &" + target + ");";
+    return "if (" + cond + ") " + target + " = " + value + ";";
+  }
+
   std::string loadStr(const ExprRef& e, const std::string& accRef) {
     // the stage's own running value
     if (e->name == st_.tensor && !accRef.empty() && e->args.size() == st_.lhsSubs.size()) {
@@ -607,7 +655,7 @@ class StageCodegen {
       }
     }
     std::string global = "p" + e->name + "[" + flatIndex(e->name, e->args, accRef) + "]";
-    if (kc_.opts.useReadOnlyCacheValue && !st_.views.at(e->name).isOutput && ntLoads_) {
+    if (kc_.opts.useReadOnlyCacheValue && !st_.views.at(e->name).isOutput && streamedOnce(e->name, e->args)) {
       // streaming read of an input that is never written: keep it out of the way of cached data
       global = "__builtin_nontemporal_load(&" + global + ")";
     }
@@ -1025,14 +1073,26 @@ class StageCodegen {
     }
     std::string base = std::to_string(v.min);
     if (v.numTiles > 1) base += " + " + tv(v) + " * " + std::to_string(v.tile);
-    em_.line("const int p_" + v.name + " = " + p + ";");
-    em_.line("const int " + iv(v) + " = " + base + " + p_" + v.name + ";");
+    // Points outside the tile or the variable's range are folded onto the last valid point: the
+    // folded iteration repeats valid work with in-bounds accesses, so loads and arithmetic need
+    // no guard (straight-line code the compiler can vectorise and schedule freely); only the
+    // stores and the reduction updates look at the predicate, which is taken before folding.
+    bool overCover = v.threadAxis >= 0 && v.perThread * kc_.k.block[v.threadAxis] != v.tile;
     std::string pred;
-    if (v.threadAxis >= 0 && v.perThread * kc_.k.block[v.threadAxis] != v.tile) {
-      pred = "p_" + v.name + " < " + std::to_string(v.tile);
+    if (overCover) {
+      em_.line("const int u_" + v.name + " = " + p + ";");
+      em_.line("const int p_" + v.name + " = __tc::tmin(u_" + v.name + ", " + std::to_string(v.tile - 1) + ");");
+      pred = "u_" + v.name + " < " + std::to_string(v.tile);
+    } else {
+      em_.line("const int p_" + v.name + " = " + p + ";");
     }
     if (v.partial()) {
-      pred += (pred.empty() ? "" : " && ") + iv(v) + " <= " + std::to_string(v.min + v.extent - 1);
+      std::string last = std::to_string(v.min + v.extent - 1);
+      em_.line("const int w_" + v.name + " = " + base + " + " + (overCover ? "u_" : "p_") + v.name + ";");
+      em_.line("const int " + iv(v) + " = __tc::tmin(" + base + " + p_" + v.name + ", " + last + ");");
+      pred += (pred.empty() ? "" : " && ") + std::string("w_") + v.name + " <= " + last;
+    } else {
+      em_.line("const int " + iv(v) + " = " + base + " + p_" + v.name + ";");
     }
     return pred;
   }
@@ -1075,13 +1135,13 @@ class StageCodegen {
   // --- statements -----------------------------------------------------------------------------
   void emitPointwise(const StageStmt& s) {
     int n = openUnrolled();
-    em_.line("if (ok_) acc_[a_] = " + castTo(s.rhs, accType_, accValid_ ? "acc_[a_]" : "") + ";");
+    em_.line("acc_[a_] = " + castTo(s.rhs, accType_, accValid_ ? "acc_[a_]" : "") + ";");
     closeN(n);
   }
 
   void preloadAcc() {
     int n = openUnrolled();
-    em_.line("if (ok_) acc_[a_] = p" + st_.tensor + "[" + flatIndex(st_.tensor, st_.lhsSubs, "") + "];");
+    em_.line("acc_[a_] = p" + st_.tensor + "[" + flatIndex(st_.tensor, st_.lhsSubs, "") + "];");
     closeN(n);
     accValid_ = true;
   }
@@ -1174,7 +1234,9 @@ class StageCodegen {
     }
     {
       int n = openUnrolled();
-      std::string cond = rpred.empty() ? "ok_" : "ok_ && " + rpred;
+      // folded parallel points only repeat valid work and are never stored: the update is
+      // guarded by the reduction's own predicate alone
+      const std::string& cond = rpred;
       if (cached) {
         // slot of this (register-tile element, reduction iteration) in the per-thread cache
         std::string rlin = "0";
@@ -1187,14 +1249,19 @@ class StageCodegen {
         cacheSlot_ = "a_ * " + std::to_string(rcount) + " + " + rlin;
         for (const auto& c : regCaches) {
           if (c.second.producer) {
-            em_.line("if (" + cond + ") " + c.second.name + "[" + cacheSlot_ + "] = " + c.first + ";");
+            em_.line(c.second.name + "[" + cacheSlot_ + "] = " + c.first + ";");
           }
         }
         inCachedReduction_ = true;
       }
       std::string rhs = castTo(s.rhs, accType_, "acc_[a_]");
       inCachedReduction_ = false;
-      em_.line("if (" + cond + ") " + target + "[a_] = " + combine(s.op, target + "[a_]", rhs) + ";");
+      if (cond.empty()) {
+        em_.line(target + "[a_] = " + combine(s.op, target + "[a_]", rhs) + ";");
+      } else {
+        em_.line("const " + accType_.cName() + " r_ = " + rhs + ";");
+        em_.line("if (" + cond + ") " + target + "[a_] = " + combine(s.op, target + "[a_]", "r_") + ";");
+      }
       closeN(n);
     }
     closeN(ropened);
@@ -1518,7 +1585,7 @@ class StageCodegen {
           // reduction operator without reduction indices: a single combine with the old value
           if (!accValid_) preloadAcc();
           int n = openUnrolled();
-          em_.line("if (ok_) acc_[a_] = " + combine(s.op, "acc_[a_]", castTo(s.rhs, accType_, "acc_[a_]")) + ";");
+          em_.line("acc_[a_] = " + combine(s.op, "acc_[a_]", castTo(s.rhs, accType_, "acc_[a_]")) + ";");
           closeN(n);
         } else {
           if (!accValid_ && readsOwnValue(s, st_)) preloadAcc();
@@ -1534,7 +1601,7 @@ class StageCodegen {
       int n = openUnrolled();
       std::string cond = "ok_";
       if (st_.threadReduction) cond += " && threadIdx.x == 0";
-      em_.line("if (" + cond + ") p" + st_.tensor + "[" + flatIndex(st_.tensor, st_.lhsSubs, "") + "] = acc_[a_];");
+      em_.line(storeStmt(cond, "acc_[a_]"));
       closeN(n);
     }
     closeN(opened);
@@ -1558,7 +1625,6 @@ class StageCodegen {
   bool inCachedReduction_ = false;
   std::string cacheSlot_;
   int clampId_ = 0;
-  bool ntLoads_ = true;
 };
 
 // ------------------------------------------------------------------------------------------
