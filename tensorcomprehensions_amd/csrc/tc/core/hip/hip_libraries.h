@@ -14,7 +14,11 @@ namespace hip {
 constexpr const char* kDeviceTypes = R"HIP(
 typedef long long int64;
 typedef unsigned long long uint64;
-namespace __tc { typedef float floatx4 __attribute__((ext_vector_type(4))); }
+namespace __tc {
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+// same vector read through a pointer that is only element-aligned
+typedef float floatx4u __attribute__((ext_vector_type(4), aligned(4)));
+}
 )HIP";
 
 // Halide-style integer semantics for / and % in subscripts (round toward -infinity),

@@ -576,6 +576,25 @@ class StageCodegen {
     return "((" + t.cName() + ")(" + s + "))";
   }
 
+  // flattened element offset as an affine form of the stage's variables (invalid when a
+  // subscript is not affine)
+  Affine flatAffine(const std::string& tensor, const std::vector<ExprRef>& subs) const {
+    const TensorView& v = st_.views.at(tensor);
+    auto strides = makeStridesFromSizes(v.extents);
+    Affine total;
+    total.valid = true;
+    for (size_t j = 0; j < subs.size(); ++j) {
+      Affine a = ir::toAffine(subs[j]);
+      if (!a.valid) {
+        total.valid = false;
+        return total;
+      }
+      for (const auto& c : a.coef) total.coef[c.first] += c.second * strides[j];
+      total.constant += a.constant * strides[j];
+    }
+    return total;
+  }
+
   std::string flatIndex(const std::string& tensor, const std::vector<ExprRef>& subs, const std::string& accRef) {
     const TensorView& v = st_.views.at(tensor);
     auto strides = makeStridesFromSizes(v.extents);
@@ -655,6 +674,10 @@ class StageCodegen {
       }
     }
     std::string global = "p" + e->name + "[" + flatIndex(e->name, e->args, accRef) + "]";
+    {
+      auto it = hoistedLoads_.find(global);
+      if (it != hoistedLoads_.end()) return it->second;
+    }
     if (kc_.opts.useReadOnlyCacheValue && !st_.views.at(e->name).isOutput && streamedOnce(e->name, e->args)) {
       // streaming read of an input that is never written: keep it out of the way of cached data
       global = "__builtin_nontemporal_load(&" + global + ")";
@@ -769,6 +792,22 @@ class StageCodegen {
   }
 
   // Decide which read-only operands of statement `s` to stage in LDS.
+  // Matrix-core stages whose block tile holds a single 16-row group of the M side: the M-side
+  // operand of a wavefront is the same for all of its output tiles, so each lane keeps its
+  // elements (one per reduction step) in registers for the whole stage instead of re-reading them.
+  static constexpr int64_t kMaxResidentSteps = 64;
+  bool mfmaKeepsMOperandInRegisters() const {
+    if (!st_.mfma) return false;
+    int64_t MT = 1, BT = 1, KT = 1;
+    for (const auto& n : st_.mfmaM) MT *= var(n).tile;
+    for (const auto& n : st_.mfmaBatch) BT *= var(n).tile;
+    for (const auto& n : st_.mfmaK) KT *= var(n).tile;
+    for (const auto& n : st_.mfmaK) {
+      if (var(n).numTiles > 1) return false;
+    }
+    return MT <= 16 && BT == 1 && ceilDiv(KT, 4) <= kMaxResidentSteps;
+  }
+
   void planPromotions(const StageStmt& s, int64_t& ldsBudgetBytes) {
     if (!kc_.opts.useSharedMemoryValue || s.redVars.empty()) return;
     for (const auto& v : st_.vars) {
@@ -803,8 +842,12 @@ class StageCodegen {
       int64_t bytes;
     };
     std::vector<Cand> cands;
+    std::string residentOperand;
+    if (mfmaKeepsMOperandInRegisters()) {
+      residentOperand = s.rhs->args[st_.mfmaSwapOperands ? 1 : 0]->name; // read once per wavefront
+    }
     for (const auto& acc : accesses) {
-      if (bad.count(acc.first)) continue;
+      if (bad.count(acc.first) || acc.first == residentOperand) continue;
       const TensorView& view = st_.views.at(acc.first);
       if (view.isOutput) continue; // may be written by another stage of this kernel
       const auto& ref = acc.second.front();
@@ -881,8 +924,8 @@ class StageCodegen {
 
   void emitLdsDecls() {
     for (const auto& p : st_.promotions) {
-      em_.line("__shared__ " + st_.views.at(p.tensor).type.cName() + " " + p.ldsName + "[" +
-               std::to_string(p.elems) + "];");
+      em_.line("__shared__ __attribute__((aligned(16))) " + st_.views.at(p.tensor).type.cName() + " " + p.ldsName +
+               "[" + std::to_string(p.elems) + "];");
     }
   }
 
@@ -894,53 +937,109 @@ class StageCodegen {
     }
   }
 
-  int64_t copyIterations(const Promotion& p) const {
-    int64_t count = 1;
-    for (auto e : p.extents) count *= e;
-    return ceilDiv(count, kc_.NT());
-  }
-
-  // Whole-footprint variants used by the software pipeline: every thread keeps its share of the
-  // tile in `regs` between the load and the store phase.  Footprint origins must be in scope.
-  void emitCopyLoads(const Promotion& p, const std::string& regs) { emitCopyPhase(p, regs, true); }
-  void emitCopyStores(const Promotion& p, const std::string& regs) { emitCopyPhase(p, regs, false); }
-
+  // --- global -> LDS copies --------------------------------------------------------------------
+  // Copy dimensions: trailing dimensions the footprint covers completely (and that are not
+  // padded in LDS) are contiguous in both memories and fold into their outer neighbour, which
+  // removes most of the index decoding.  When the innermost copy dimension is contiguous on both
+  // sides and every row starts on a multiple of four elements, threads move 16-byte vectors.
   struct CopyDim {
     int64_t extent, tensorExtent, gStride, lStride;
     std::string lo;
+    int64_t loGcd; // every value of `lo` is a multiple of this (0: lo is always 0)
   };
-  std::vector<CopyDim> copyDims(const Promotion& p) const {
+  struct CopyPlan {
+    std::vector<CopyDim> dims;
+    int64_t count = 1;  // elements
+    int vec = 1;        // elements per thread and iteration
+    int64_t iters = 1;  // iterations per thread
+    std::string elemType, regType;
+  };
+
+  static int64_t gcd(int64_t a, int64_t b) {
+    a = std::abs(a);
+    b = std::abs(b);
+    while (b) {
+      int64_t t = a % b;
+      a = b;
+      b = t;
+    }
+    return a;
+  }
+
+  // a divisor of every value footprintLow(p, j) can take
+  int64_t footprintLowGcd(const Promotion& p, size_t j) const {
+    const Footprint& fp = footprints_.at(p.tensor);
+    int64_t g = std::abs(fp.minConst[j]);
+    for (const auto& c : fp.coefs[j].coef) {
+      const LoopVar& v = var(c.first);
+      bool fixed = (v.reduction && !p.insideReductionTiles) || v.numTiles == 1;
+      g = gcd(g, c.second * v.min);
+      if (!fixed) g = gcd(g, c.second * v.tile);
+      if (c.second < 0) g = gcd(g, c.second * (spanOf(v, p.insideReductionTiles) - 1));
+    }
+    return g;
+  }
+
+  CopyPlan copyPlan(const Promotion& p) const {
     const TensorView& view = st_.views.at(p.tensor);
     auto gStridesFull = makeStridesFromSizes(view.extents);
-    std::vector<CopyDim> dims;
+    CopyPlan plan;
+    for (auto e : p.extents) plan.count *= e;
     for (size_t j = 0; j < p.extents.size(); ++j) {
-      dims.push_back(CopyDim{p.extents[j], view.extents[j], gStridesFull[j], p.ldsStrides[j], loPrefix(p) + std::to_string(j)});
+      plan.dims.push_back(CopyDim{p.extents[j], view.extents[j], gStridesFull[j], p.ldsStrides[j],
+                                  loPrefix(p) + std::to_string(j), footprintLowGcd(p, j)});
     }
+    auto& dims = plan.dims;
     while (dims.size() >= 2) {
       CopyDim& in = dims.back();
       CopyDim& out = dims[dims.size() - 2];
       bool full = in.extent == in.tensorExtent && out.lStride == in.lStride * in.extent &&
           out.gStride == in.gStride * in.tensorExtent;
       if (!full) break;
+      // (out, in) -> one dimension of extent out*in starting at out.lo * in.extent (in.lo is 0)
       out.lo = "(" + out.lo + ") * " + std::to_string(in.extent);
+      out.loGcd *= in.extent;
       out.extent *= in.extent;
       out.tensorExtent *= in.tensorExtent;
       out.gStride = in.gStride;
       out.lStride = in.lStride;
       dims.pop_back();
     }
-    return dims;
+    plan.elemType = view.type.cName();
+    plan.regType = plan.elemType;
+    if (view.type.isFloat() && view.type.bits == 32 && !dims.empty()) {
+      const CopyDim& in = dims.back();
+      bool ok = in.gStride == 1 && in.lStride == 1 && in.extent % 4 == 0 && in.tensorExtent % 4 == 0 &&
+          in.loGcd % 4 == 0;
+      for (size_t j = 0; j + 1 < dims.size(); ++j) ok &= dims[j].gStride % 4 == 0 && dims[j].lStride % 4 == 0;
+      if (ok) {
+        plan.vec = 4;
+        plan.regType = "__tc::floatx4";
+      }
+    }
+    plan.iters = ceilDiv(plan.count / plan.vec, kc_.NT());
+    return plan;
   }
 
-  void emitCopyPhase(const Promotion& p, const std::string& regs, bool loads) {
-    int64_t count = 1;
-    for (auto e : p.extents) count *= e;
-    std::vector<CopyDim> dims = copyDims(p);
-    em_.line("#pragma unroll");
-    em_.open("for (int it_ = 0; it_ < " + std::to_string(copyIterations(p)) + "; ++it_)");
-    em_.line("const int c_ = it_ * " + std::to_string(kc_.NT()) + " + tid_;");
-    int64_t div = count;
-    std::string cond = "c_ < " + std::to_string(count), gidx, lidx;
+  int64_t copyRegisters(const Promotion& p) const {
+    CopyPlan plan = copyPlan(p);
+    return plan.iters * plan.vec;
+  }
+  std::string copyRegisterDecl(const Promotion& p, const std::string& regs) const {
+    CopyPlan plan = copyPlan(p);
+    return plan.regType + " " + regs + "[" + std::to_string(plan.iters) + "];";
+  }
+
+  // One copy iteration of every thread: the global load of its element (vector) into
+  // regs[slot], unconditional and from a clamped address so that loads issue back to back, or
+  // the LDS store of regs[slot].
+  void emitCopyStep(const Promotion& p, const CopyPlan& plan, const std::string& itExpr, const std::string& regs,
+                    const std::string& slot, bool loads) {
+    const auto& dims = plan.dims;
+    std::string unit = "(" + itExpr + ") * " + std::to_string(kc_.NT()) + " + tid_";
+    em_.line("const int c_ = " + (plan.vec > 1 ? std::to_string(plan.vec) + " * (" + unit + ")" : unit) + ";");
+    int64_t div = plan.count;
+    std::string cond = "c_ < " + std::to_string(plan.count), gidx, lidx;
     for (size_t j = 0; j < dims.size(); ++j) {
       div /= dims[j].extent;
       std::string l = "l" + std::to_string(j) + "_";
@@ -957,97 +1056,49 @@ class StageCodegen {
       lidx += (j ? " + " : "") + l + (dims[j].lStride != 1 ? " * " + std::to_string(dims[j].lStride) : "");
     }
     if (dims.empty()) gidx = lidx = "0";
+    std::string cast = plan.vec > 1 ? "*(const __tc::floatx4u*)&" : "";
+    std::string lcast = plan.vec > 1 ? "*(__tc::floatx4*)&" : "";
     if (loads) {
-      em_.line(regs + "[it_] = p" + p.tensor + "[(" + cond + ") ? (" + gidx + ") : 0];");
+      em_.line(regs + "[" + slot + "] = " + cast + "p" + p.tensor + "[(" + cond + ") ? (" + gidx + ") : 0];");
     } else {
-      em_.line("if (c_ < " + std::to_string(count) + ") " + p.ldsName + "[" + lidx + "] = " + regs + "[it_];");
+      em_.line("if (c_ < " + std::to_string(plan.count) + ") " + lcast + p.ldsName + "[" + lidx + "] = " + regs + "[" + slot + "];");
     }
+  }
+
+  // Whole-footprint variants used by the software pipeline: every thread keeps its share of the
+  // tile in `regs` between the load and the store phase.  Footprint origins must be in scope.
+  void emitCopyLoads(const Promotion& p, const std::string& regs) { emitCopyPhase(p, regs, true); }
+  void emitCopyStores(const Promotion& p, const std::string& regs) { emitCopyPhase(p, regs, false); }
+
+  void emitCopyPhase(const Promotion& p, const std::string& regs, bool loads) {
+    CopyPlan plan = copyPlan(p);
+    em_.line("#pragma unroll");
+    em_.open("for (int it_ = 0; it_ < " + std::to_string(plan.iters) + "; ++it_)");
+    emitCopyStep(p, plan, "it_", regs, "it_", loads);
     em_.close();
   }
 
   void emitCopyIn(const Promotion& p) {
-    const TensorView& view = st_.views.at(p.tensor);
-    auto gStridesFull = makeStridesFromSizes(view.extents);
-    int64_t count = 1;
-    for (auto e : p.extents) count *= e;
-    std::string loPrefix = "lo" + std::to_string(stageIdx_) + "_" + p.tensor + "_";
-    for (size_t j = 0; j < p.extents.size(); ++j) {
-      em_.line("const int " + loPrefix + std::to_string(j) + " = " + footprintLow(p, j) + ";");
-    }
-    // Copy dimensions: trailing dimensions the footprint covers completely (and that are not
-    // padded in LDS) are contiguous in both memories and fold into their outer neighbour, which
-    // removes most of the index decoding.
-    struct CopyDim {
-      int64_t extent, tensorExtent, gStride, lStride;
-      std::string lo;
-    };
-    std::vector<CopyDim> dims;
-    for (size_t j = 0; j < p.extents.size(); ++j) {
-      dims.push_back(CopyDim{p.extents[j], view.extents[j], gStridesFull[j], p.ldsStrides[j], loPrefix + std::to_string(j)});
-    }
-    while (dims.size() >= 2) {
-      CopyDim& in = dims.back();
-      CopyDim& out = dims[dims.size() - 2];
-      bool full = in.extent == in.tensorExtent && out.lStride == in.lStride * in.extent &&
-          out.gStride == in.gStride * in.tensorExtent;
-      if (!full) break;
-      // (out, in) -> one dimension of extent out*in starting at out.lo * in.extent (in.lo is 0)
-      out.lo = "(" + out.lo + ") * " + std::to_string(in.extent);
-      out.extent *= in.extent;
-      out.tensorExtent *= in.tensorExtent;
-      out.gStride = in.gStride;
-      out.lStride = in.lStride;
-      dims.pop_back();
-    }
-    // Two phases per chunk of iterations: all global loads first (unconditional, from a clamped
-    // address, so they are issued back to back and their latencies overlap), then the LDS stores.
-    int64_t iters = ceilDiv(count, kc_.NT());
-    int64_t chunk = std::min<int64_t>(iters, kc_.opts.unrollCopySharedValue ? 32 : 16);
-    std::string ty = view.type.cName();
-    auto decompose = [&](const std::string& itExpr, std::string& cond, std::string& gidx, std::string& lidx) {
-      em_.line("const int c_ = (" + itExpr + ") * " + std::to_string(kc_.NT()) + " + tid_;");
-      int64_t div = count;
-      cond.clear();
-      gidx.clear();
-      lidx.clear();
-      for (size_t j = 0; j < dims.size(); ++j) {
-        div /= dims[j].extent;
-        std::string l = "l" + std::to_string(j) + "_";
-        std::string e = "c_";
-        if (div > 1) e = "(" + e + " / " + std::to_string(div) + ")";
-        if (j > 0) e = e + " % " + std::to_string(dims[j].extent);
-        em_.line("const int " + l + " = " + e + ";");
-        std::string g = "g" + std::to_string(j) + "_";
-        em_.line("const int " + g + " = " + dims[j].lo + " + " + l + ";");
-        cond += (j ? " && " : "") + std::string("(unsigned)") + g + " < " + std::to_string(dims[j].tensorExtent) + "u";
-        gidx += (j ? " + " : "") + g + (dims[j].gStride != 1 ? " * " + std::to_string(dims[j].gStride) : "");
-        lidx += (j ? " + " : "") + l + (dims[j].lStride != 1 ? " * " + std::to_string(dims[j].lStride) : "");
-      }
-      if (dims.empty()) {
-        cond = "true";
-        gidx = lidx = "0";
-      }
-      cond = "c_ < " + std::to_string(count) + " && " + cond;
-    };
-    bool chunked = iters > chunk;
+    declareLows(p);
+    CopyPlan plan = copyPlan(p);
+    // Two phases per chunk of iterations: all global loads first, so that their latencies
+    // overlap, then the LDS stores.
+    int64_t chunk = std::min<int64_t>(plan.iters, (kc_.opts.unrollCopySharedValue ? 32 : 16) / plan.vec);
+    chunk = std::max<int64_t>(chunk, 1);
+    bool chunked = plan.iters > chunk;
     if (chunked) {
-      em_.open("for (int cb_ = 0; cb_ < " + std::to_string(iters) + "; cb_ += " + std::to_string(chunk) + ")");
+      em_.open("for (int cb_ = 0; cb_ < " + std::to_string(plan.iters) + "; cb_ += " + std::to_string(chunk) + ")");
     } else {
       em_.open("");
     }
     std::string base = chunked ? "cb_ + " : "";
-    em_.line(ty + " stage_[" + std::to_string(chunk) + "];");
-    std::string cond, gidx, lidx;
-    em_.line("#pragma unroll");
-    em_.open("for (int it_ = 0; it_ < " + std::to_string(chunk) + "; ++it_)");
-    decompose(base + "it_", cond, gidx, lidx);
-    em_.line("stage_[it_] = p" + p.tensor + "[(" + cond + ") ? (" + gidx + ") : 0];");
-    em_.close();
-    em_.line("#pragma unroll");
-    em_.open("for (int it_ = 0; it_ < " + std::to_string(chunk) + "; ++it_)");
-    decompose(base + "it_", cond, gidx, lidx);
-    em_.line("if (c_ < " + std::to_string(count) + ") " + p.ldsName + "[" + lidx + "] = stage_[it_];");
-    em_.close();
+    em_.line(plan.regType + " stage_[" + std::to_string(chunk) + "];");
+    for (bool loads : {true, false}) {
+      em_.line("#pragma unroll");
+      em_.open("for (int it_ = 0; it_ < " + std::to_string(chunk) + "; ++it_)");
+      emitCopyStep(p, plan, base + "it_", "stage_", "it_", loads);
+      em_.close();
+    }
     em_.close();
   }
 
@@ -1406,11 +1457,144 @@ class StageCodegen {
       for (const auto& n : g) exact &= !var(n).partial();
       return exact;
     };
-    (void)groupExact;
     const ExprRef& loadA = s.rhs->args[st_.mfmaSwapOperands ? 1 : 0]; // holds the M-side variables
     const ExprRef& loadB = s.rhs->args[st_.mfmaSwapOperands ? 0 : 1]; // holds the N-side variables
     em_.line("// matrix cores: " + std::to_string(tiles) + " tiles of 16x16 per block, " + std::to_string(ksteps) +
              " steps of v_mfma_f32_16x16x4_f32 each, " + std::to_string(st_.waves) + " wavefront(s)");
+    // (the register-resident operand is requested first: its latency overlaps the LDS staging)
+    em_.line("const int lm_ = threadIdx.x & 15, lj_ = threadIdx.x >> 4;");
+    // Lane group lj_ (0..3) owns a contiguous quarter of the flattened reduction and step ks_
+    // walks inside it: when a quarter is a whole number of inner-variable periods, the inner
+    // reduction indices of a step are compile-time constants after unrolling and only the
+    // outermost one depends on the lane, so operand addresses become "lane base + immediate".
+    const int64_t quarter = ceilDiv(KT, 4);
+    ksteps = quarter;
+    int64_t innerProd = 1;
+    for (size_t i = 1; i < st_.mfmaK.size(); ++i) innerProd *= var(st_.mfmaK[i]).tile;
+    const bool aligned = quarter % innerProd == 0;
+    // Opens the loop over the reduction steps of a lane, decodes the reduction indices of the
+    // step and declares kok_ when surplus steps exist; returns whether it did.
+    auto openSteps = [&]() {
+      em_.line(ksteps <= 128 ? "#pragma unroll" : "#pragma unroll 4");
+      em_.open("for (int ks_ = 0; ks_ < " + std::to_string(ksteps) + "; ++ks_)");
+      std::string kok;
+      if (aligned) {
+        int64_t div = innerProd;
+        for (size_t i = 0; i < st_.mfmaK.size(); ++i) {
+          const LoopVar& v = var(st_.mfmaK[i]);
+          std::string e;
+          if (i == 0) {
+            e = "lj_ * " + std::to_string(quarter / innerProd) + " + ks_ / " + std::to_string(innerProd);
+          } else {
+            div /= v.tile;
+            e = "(ks_ / " + std::to_string(div) + ") % " + std::to_string(v.tile);
+          }
+          // the surplus steps of the last lane group would decode past the outermost extent
+          if (i == 0 && quarter * 4 != KT) e = "min(" + e + ", " + std::to_string(v.tile - 1) + ")";
+          em_.line("const int p_" + v.name + " = " + e + ";");
+          em_.line("const int " + iv(v) + " = " + std::to_string(v.min) + " + p_" + v.name + ";");
+        }
+        if (quarter * 4 != KT) kok = "lj_ * " + std::to_string(quarter) + " + ks_ < " + std::to_string(KT);
+      } else {
+        em_.line("const int kk_ = lj_ * " + std::to_string(quarter) + " + ks_;");
+        kok = decodeGroup(st_.mfmaK, "kk_", true);
+        if (quarter * 4 == KT) kok.clear();
+      }
+      if (!kok.empty()) em_.line("const bool kok_ = " + kok + ";");
+      return !kok.empty();
+    };
+    // surplus reduction steps must contribute exact zeros
+    auto operandValue = [&](const ExprRef& load, bool masked) {
+      std::string text = loadStr(load, "");
+      return masked ? "(kok_ ? " + text + " : 0.0f)" : text;
+    };
+    const bool resident = mfmaKeepsMOperandInRegisters();
+    if (resident) {
+      em_.line("float am_[" + std::to_string(ksteps) + "];");
+      em_.open("");
+      em_.line("const int mt_ = 0, bt_ = 0;");
+      em_.line("(void)mt_; (void)bt_;");
+      if (!st_.mfmaBatch.empty()) decodeGroup(st_.mfmaBatch, "bt_", true);
+      em_.line("const int mposa_ = lm_;");
+      decodeGroup(st_.mfmaM, "mposa_", true);
+      // consecutive steps of a lane read consecutive elements when the operand's reduction
+      // subscripts are jointly contiguous: four steps are then fetched with one 16-byte load
+      bool contiguous = aligned && quarter * 4 == KT && ksteps % 4 == 0;
+      {
+        Affine fa = flatAffine(loadA->name, loadA->args);
+        contiguous &= fa.valid;
+        int64_t expect = 1;
+        for (size_t i = st_.mfmaK.size(); contiguous && i-- > 0;) {
+          const LoopVar& v = var(st_.mfmaK[i]);
+          contiguous &= fa.coefOf(v.name) == expect;
+          expect *= v.tile;
+        }
+      }
+      if (contiguous) {
+        em_.line("#pragma unroll");
+        em_.open("for (int kv_ = 0; kv_ < " + std::to_string(ksteps / 4) + "; ++kv_)");
+        em_.line("const int ks_ = 4 * kv_;");
+        int64_t div = innerProd;
+        for (size_t i = 0; i < st_.mfmaK.size(); ++i) {
+          const LoopVar& v = var(st_.mfmaK[i]);
+          std::string e;
+          if (i == 0) {
+            e = "lj_ * " + std::to_string(quarter / innerProd) + " + ks_ / " + std::to_string(innerProd);
+          } else {
+            div /= v.tile;
+            e = "(ks_ / " + std::to_string(div) + ") % " + std::to_string(v.tile);
+          }
+          em_.line("const int " + iv(v) + " = " + std::to_string(v.min) + " + " + e + ";");
+        }
+        em_.line("const __tc::floatx4 v_ = *(const __tc::floatx4u*)&p" + loadA->name + "[" +
+                 flatIndex(loadA->name, loadA->args, "") + "];");
+        em_.line("am_[ks_] = v_[0]; am_[ks_ + 1] = v_[1]; am_[ks_ + 2] = v_[2]; am_[ks_ + 3] = v_[3];");
+        em_.close();
+      } else {
+        bool masked = openSteps();
+        em_.line("am_[ks_] = " + operandValue(loadA, masked) + ";");
+        em_.close();
+      }
+      em_.close();
+    }
+    // Epilogue operands that do not depend on the column (a bias per output row, say) are the
+    // same for every tile of the wavefront: fetched once, ahead of the tile loop.
+    hoistedLoads_.clear();
+    if (resident) {
+      std::vector<std::pair<std::string, ExprRef>> invariant;
+      for (size_t i = 1; i < st_.stmts.size(); ++i) {
+        visit(st_.stmts[i].rhs, [&](const ExprRef& e) {
+          if (e->kind != Expr::Load || e->name == st_.tensor || st_.views.at(e->name).isOutput) return;
+          Affine fa = flatAffine(e->name, e->args);
+          bool ok = fa.valid;
+          for (const auto& n : st_.mfmaN) ok = ok && fa.coefOf(n) == 0;
+          if (!ok) return;
+          std::string text = "p" + e->name + "[" + flatIndex(e->name, e->args, "") + "]";
+          for (const auto& h : invariant) {
+            if (h.first == text) return;
+          }
+          invariant.emplace_back(text, e);
+        });
+      }
+      if (!invariant.empty()) {
+        for (size_t h = 0; h < invariant.size(); ++h) {
+          em_.line(st_.views.at(invariant[h].second->name).type.cName() + " eh" + std::to_string(h) + "_[4];");
+        }
+        em_.line("#pragma unroll");
+        em_.open("for (int r_ = 0; r_ < 4; ++r_)");
+        em_.line("const int bt_ = 0, mpos_ = 4 * lj_ + r_;");
+        em_.line("(void)bt_;");
+        if (!st_.mfmaBatch.empty()) decodeGroup(st_.mfmaBatch, "bt_", true);
+        decodeGroup(st_.mfmaM, "mpos_", true);
+        for (size_t h = 0; h < invariant.size(); ++h) {
+          em_.line("eh" + std::to_string(h) + "_[r_] = " + invariant[h].first + ";");
+        }
+        em_.close();
+        for (size_t h = 0; h < invariant.size(); ++h) {
+          hoistedLoads_[invariant[h].first] = "eh" + std::to_string(h) + "_[r_]";
+        }
+      }
+    }
     int opened = 0;
     if (!st_.promotions.empty()) {
       em_.open("");
@@ -1429,15 +1613,16 @@ class StageCodegen {
         em_.line("__syncthreads();");
       }
     }
-    em_.line("const int lm_ = threadIdx.x & 15, lj_ = threadIdx.x >> 4;");
-    em_.open("for (int tl_ = threadIdx.y; tl_ < " + std::to_string(tiles) + "; tl_ += " + std::to_string(st_.waves) + ")");
+    // which wavefront takes the surplus tile rotates with the block, so that the blocks sharing a
+    // compute unit load its four SIMDs evenly
+    em_.line("const int wv_ = (threadIdx.y + blockIdx.x + blockIdx.y + blockIdx.z) % " + std::to_string(st_.waves) + ";");
+    em_.open("for (int tl_ = wv_; tl_ < " + std::to_string(tiles) + "; tl_ += " + std::to_string(st_.waves) + ")");
     ++opened;
     em_.line("const int nt_ = tl_ % " + std::to_string(numNT) + ", mt_ = (tl_ / " + std::to_string(numNT) + ") % " +
              std::to_string(numMT) + ", bt_ = tl_ / " + std::to_string(numNT * numMT) + ";");
     // A row of the product depends on one row of the M-side operand only and a column on one
     // column of the N-side operand, so lanes past the end of a partial tile may load any legal
-    // element (clamped indices): their results are never stored.  Only surplus reduction steps
-    // must contribute exact zeros.
+    // element (clamped indices): their results are never stored.
     std::string bok = st_.mfmaBatch.empty() ? "true" : decodeGroup(st_.mfmaBatch, "bt_", true);
     em_.line("const bool bok_ = " + bok + ";");
     em_.line("const int npos_ = nt_ * 16 + lm_;");
@@ -1457,68 +1642,23 @@ class StageCodegen {
       em_.line("const int mposa_ = mt_ * 16 + lm_;");
       em_.line("const bool moka_ = bok_ && " + decodeGroup(st_.mfmaM, "mposa_", true) + ";");
       em_.line("(void)moka_;");
-      // Lane group lj_ (0..3) owns a contiguous quarter of the flattened reduction and step ks_
-      // walks inside it: when a quarter is a whole number of inner-variable periods, the inner
-      // reduction indices of a step are compile-time constants after unrolling and only the
-      // outermost one depends on the lane, so operand addresses become "lane base + immediate".
-      int64_t quarter = ceilDiv(KT, 4);
-      ksteps = quarter;
-      int64_t innerProd = 1;
-      for (size_t i = 1; i < st_.mfmaK.size(); ++i) innerProd *= var(st_.mfmaK[i]).tile;
-      bool aligned = quarter % innerProd == 0;
-      em_.line(ksteps <= 128 ? "#pragma unroll" : "#pragma unroll 4");
-      em_.open("for (int ks_ = 0; ks_ < " + std::to_string(ksteps) + "; ++ks_)");
-      std::string kok;
-      if (aligned) {
-        int64_t div = innerProd;
-        for (size_t i = 0; i < st_.mfmaK.size(); ++i) {
-          const LoopVar& v = var(st_.mfmaK[i]);
-          std::string e;
-          if (i == 0) {
-            e = "lj_ * " + std::to_string(quarter / innerProd) + " + ks_ / " + std::to_string(innerProd);
-          } else {
-            div /= v.tile;
-            e = "(ks_ / " + std::to_string(div) + ") % " + std::to_string(v.tile);
-          }
-          if (i == 0 && quarter * 4 != KT) e = "min(" + e + ", " + std::to_string(v.tile - 1) + ")";
-          em_.line("const int p_" + v.name + " = " + e + ";");
-          em_.line("const int " + iv(v) + " = " + std::to_string(v.min) + " + p_" + v.name + ";");
-        }
-        if (quarter * 4 != KT) kok = "lj_ * " + std::to_string(quarter) + " + ks_ < " + std::to_string(KT);
-      } else {
-        em_.line("const int kk_ = lj_ * " + std::to_string(quarter) + " + ks_;");
-        kok = decodeGroup(st_.mfmaK, "kk_", true);
-        if (quarter * 4 == KT) kok.clear();
-      }
-      auto operand = [&](const char* name, const ExprRef& load) {
-        std::string text = loadStr(load, "");
-        if (kok.empty()) {
-          em_.line(std::string("const float ") + name + " = " + text + ";");
-        } else {
-          em_.line(std::string("const float ") + name + "raw_ = " + text + ";");
-          em_.line(std::string("const float ") + name + " = kok_ ? " + name + "raw_ : 0.0f;");
-        }
-      };
-      if (!kok.empty()) em_.line("const bool kok_ = " + kok + ";");
-      if (aligned && !kok.empty()) {
-        // the surplus steps of the last lane group would decode past the outermost extent
-        const LoopVar& v0 = var(st_.mfmaK[0]);
-        em_.line("// (indices of surplus steps are clamped below)");
-        (void)v0;
-      }
-      operand("a_", loadA);
-      operand("b_", loadB);
+      bool masked = openSteps();
+      em_.line("const float a_ = " + (resident ? std::string("am_[ks_]") : operandValue(loadA, masked)) + ";");
+      em_.line("const float b_ = " + operandValue(loadB, masked) + ";");
       em_.line("c_ = __builtin_amdgcn_mfma_f32_16x16x4f32(a_, b_, c_, 0, 0, 0);");
       em_.close();
       em_.close();
     }
-    // epilogue and store: lane holds rows 4*lj_ .. 4*lj_+3 of column lm_
+    // Epilogue and store: a lane holds rows 4*lj_ .. 4*lj_+3 of column lm_.  Indices are clamped
+    // to legal points, so the epilogue's loads need no guard: the four rows are finished first
+    // (their loads issue together and, when they do not depend on the column, move out of the
+    // tile loop), then stored under one test of the column.
+    const bool mExact = groupExact(st_.mfmaM, MT, 16);
+    em_.line(accType_.cName() + " out_[4];");
     em_.line("#pragma unroll");
     em_.open("for (int r_ = 0; r_ < 4; ++r_)");
     em_.line("const int mpos_ = mt_ * 16 + 4 * lj_ + r_;");
-    // indices are clamped to legal points, so the epilogue's loads need no branch (four
-    // independent rows are then fetched together); only the store is predicated
-    em_.line("const bool okr_ = nok_ && " + decodeGroup(st_.mfmaM, "mpos_", true) + ";");
+    decodeGroup(st_.mfmaM, "mpos_", true);
     em_.line(accType_.cName() + " acc_[1];");
     em_.line("acc_[0] = c_[r_];");
     outerPred_ = "";
@@ -1527,15 +1667,24 @@ class StageCodegen {
       const StageStmt& e = st_.stmts[i];
       if (e.op != ReduceOp::None) {
         int n = openUnrolled();
-        em_.line("if (ok_) acc_[a_] = " + combine(e.op, "acc_[a_]", castTo(e.rhs, accType_, "acc_[a_]")) + ";");
+        em_.line("acc_[a_] = " + combine(e.op, "acc_[a_]", castTo(e.rhs, accType_, "acc_[a_]")) + ";");
         closeN(n);
       } else {
         emitPointwise(e);
       }
     }
-    em_.line("if (okr_) p" + st_.tensor + "[" + flatIndex(st_.tensor, st_.lhsSubs, "") + "] = acc_[0];");
+    em_.line("out_[r_] = acc_[0];");
+    em_.close();
+    em_.open("if (nok_)");
+    em_.line("#pragma unroll");
+    em_.open("for (int r_ = 0; r_ < 4; ++r_)");
+    em_.line("const int mpos_ = mt_ * 16 + 4 * lj_ + r_;");
+    std::string mok = decodeGroup(st_.mfmaM, "mpos_", true);
+    em_.line(storeStmt(mExact ? "true" : mok, "out_[r_]"));
+    em_.close();
     em_.close();
     closeN(opened);
+    hoistedLoads_.clear();
     for (const auto& p : st_.promotions) activePromotions_.erase(p.tensor);
   }
 
@@ -1622,6 +1771,7 @@ class StageCodegen {
   bool accValid_ = false;
   std::string outerPred_;
   std::set<std::string> activePromotions_;
+  std::map<std::string, std::string> hoistedLoads_; // printed global load -> register holding it
   bool inCachedReduction_ = false;
   std::string cacheSlot_;
   int clampId_ = 0;
@@ -1858,7 +2008,7 @@ void emitKernel(KernelCtx& kc, const DeviceLimits& limits, Emitter& em) {
     pipelined = true;
     for (const auto& p : gens[0].promotions()) {
       pipelined &= !p.insideReductionTiles;
-      regs += gens[0].copyIterations(p);
+      regs += gens[0].copyRegisters(p);
     }
     pipelined &= regs <= 96;
   }
@@ -1876,7 +2026,7 @@ void emitKernel(KernelCtx& kc, const DeviceLimits& limits, Emitter& em) {
     em.open("");
     ++opened;
     for (const auto& p : g.promotions()) {
-      em.line(g.promotionType(p) + " pf_" + p.tensor + "_[" + std::to_string(g.copyIterations(p)) + "];");
+      em.line(g.copyRegisterDecl(p, "pf_" + p.tensor + "_"));
     }
     em.open("");
     em.line("const int " + t + " = " + start + ";");

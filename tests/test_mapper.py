@@ -75,8 +75,8 @@ def test_lds_promotion_footprints():
     src, launches = mapped(W.BATCH_MATMUL, "batch_matmul", [(500, 26, 72), (500, 72, 26)], o)
     assert launches == [((500, 1, 1), (26, 13, 1))]
     # per block: X[1][26][72] and Y[1][72][26] (footprint = min(tile, size) per dimension)
-    assert "__shared__ float lds0_X[1872];" in src
-    assert re.search(r"__shared__ float lds0_Y\[(1872|1944)\];", src)
+    assert "float lds0_X[1872];" in src
+    assert re.search(r"float lds0_Y\[(1872|1944)\];", src)
     assert src.count("__syncthreads();") >= 2                 # before and after the copies
     # without the switch nothing is staged
     src, _ = mapped(W.BATCH_MATMUL, "batch_matmul", [(500, 26, 72), (500, 72, 26)], o.useSharedMemory(False))
@@ -90,7 +90,7 @@ def test_convolution_window_footprint_includes_the_halo():
     o = "naive;tile=1,1,16,14,14,4;mapToThreads=14,14;mapToBlocks=32,32;unroll=16;useSharedMemory=1"
     src, _ = mapped(W.GROUP_CONVOLUTION, "group_convolution", [(32, 32, 16, 16, 16), (32, 16, 16, 3, 3), (32, 16)], o)
     # input tile: 4 channels x (14+2) x (14+2)
-    assert "__shared__ float lds0_I[1024];" in src
+    assert "float lds0_I[1024];" in src
     # the weights are read at the same address by every thread of the block (f is not mapped to
     # threads here): they go through the scalar cache, not LDS
     assert "lds0_W1" not in src
@@ -99,7 +99,7 @@ def test_convolution_window_footprint_includes_the_halo():
 def test_lds_budget_is_respected():
     o = MappingOptions.naive().tile(1, 26, 26, 72).mapToThreads(26, 13).mapToBlocks(500).unroll(4).useSharedMemory(True)
     src, _ = mapped(W.BATCH_MATMUL, "batch_matmul", [(500, 26, 72), (500, 72, 26)], o.maxSharedMemory(8000))
-    assert src.count("__shared__ float") == 1                 # only one of the two 7.5 KB tiles fits
+    assert src.count("__shared__ ") == 1                      # only one of the two 7.5 KB tiles fits
 
 
 def test_fusion_strategies_decide_kernel_count():
