@@ -1,4 +1,6 @@
 // tc_autotune: C ABI of the genetic autotuner.
+#include "tc/core/mapper/sync_placement.h"
+#include <cstdio>
 #include <sstream>
 
 #include "capi/tc_capi_internal.h"
@@ -253,6 +255,27 @@ extern "C" int tc_host_query(const char* what, const char* arg, char** out) {
       result = "tile_dims=" + std::to_string(c.tilingParams.dims.size()) + ";tile=" + joinSizes(c.tilingParams.dims[0].values()) +
           ";block=" + joinSizes(c.blockParams.dims[0].values()) + ";grid=" + joinSizes(c.gridParams.dims[0].values()) +
           ";unroll=" + joinSizes(c.unrollFactor.values()) + ";genes=" + std::to_string(c.collectParameters().size());
+    } else if (w == "sync_placement") {
+      // "cyclic;n;i:k:level,i:k:level,..." -> "position:level,..." (barrier after child `position`)
+      std::stringstream ss(a);
+      std::string cyc, num, triples, item;
+      std::getline(ss, cyc, ';');
+      std::getline(ss, num, ';');
+      std::getline(ss, triples, ';');
+      int n = std::stoi(num);
+      tc::mapper::SyncNeeds need(n, std::vector<int>(n, 0));
+      std::stringstream ts(triples);
+      while (std::getline(ts, item, ',')) {
+        int i = 0, k = 0, lev = 0;
+        TC_CHECK(std::sscanf(item.c_str(), "%d:%d:%d", &i, &k, &lev) == 3) << "bad requirement '" << item << "'";
+        TC_CHECK(i >= 0 && i < n && k >= 0 && k < n && lev >= 0 && lev <= 2) << "requirement out of range";
+        need[i][k] = lev;
+      }
+      auto syncs = tc::mapper::findBestSyncs(need, cyc == "1");
+      TC_CHECK(tc::mapper::syncsAreSufficient(need, cyc == "1", syncs)) << "placement misses a requirement";
+      for (const auto& sy : syncs) {
+        result += (result.empty() ? "" : ",") + std::to_string(sy.first) + ":" + std::to_string(static_cast<int>(sy.second));
+      }
     } else if (w == "genetic_search") {
       result = runSyntheticSearch(parseSettings(a.c_str()));
     } else if (w == "options_cache_selftest") {

@@ -1,4 +1,5 @@
 #include "tc/core/mapper/mapper.h"
+#include "tc/core/mapper/sync_placement.h"
 
 #include <algorithm>
 #include <cctype>
@@ -514,6 +515,17 @@ class Emitter {
   }
 };
 
+// tensors a stage loads from (its own running value included when it re-reads it)
+std::set<std::string> tensorsRead(const StagePlan& st) {
+  std::set<std::string> r;
+  for (const auto& stmt : st.stmts) {
+    visit(stmt.rhs, [&](const ExprRef& e) {
+      if (e->kind == Expr::Load) r.insert(e->name);
+    });
+  }
+  return r;
+}
+
 struct KernelCtx {
   const ir::Function& f;
   const HipMappingOptions& opts;
@@ -650,7 +662,7 @@ class StageCodegen {
   bool streamedStore() const {
     if (!kc_.opts.useReadOnlyCacheValue || viewBytes(st_.tensor) < kStreamingBytes) return false;
     for (size_t j = stageIdx_ + 1; j < kc_.k.stages.size(); ++j) {
-      if (kc_.k.stages[j].views.count(st_.tensor)) return false;
+      if (tensorsRead(kc_.k.stages[j]).count(st_.tensor)) return false;
     }
     return true;
   }
@@ -1395,6 +1407,55 @@ class StageCodegen {
     return n;
   }
 
+  // True when this stage touches `producer`'s result only at the element the same thread wrote:
+  // both stages spread identical parallel variables over blocks and threads in the same way and
+  // every access to the tensor uses the producer's own left-hand-side subscripts.
+  bool readsPrivatelyFrom(const StagePlan& producer) const {
+    if (producer.threadReduction || producer.mfma || st_.mfma) return false;
+    if (producer.numParallel != st_.numParallel || producer.tensor == st_.tensor) return false;
+    if (tensorsRead(producer).count(st_.tensor)) return false; // it also reads what this stage overwrites
+    std::map<std::string, std::string> rename; // this stage's variable -> producer's
+    for (int i = 0; i < st_.numParallel; ++i) {
+      const LoopVar& a = producer.vars[i];
+      const LoopVar& b = st_.vars[i];
+      bool same = a.min == b.min && a.extent == b.extent && a.tile == b.tile && a.numTiles == b.numTiles &&
+          a.blockAxis == b.blockAxis && a.gridExtent == b.gridExtent && a.threadAxis == b.threadAxis &&
+          a.perThread == b.perThread && a.vectorLane == b.vectorLane;
+      if (!same) return false;
+      rename[b.name] = a.name;
+    }
+    if (producer.views.at(producer.tensor).extents != st_.views.at(producer.tensor).extents) return false;
+    std::vector<Affine> lhs;
+    for (const auto& e : producer.lhsSubs) lhs.push_back(ir::toAffine(e));
+    bool ok = true;
+    for (const auto& stmt : st_.stmts) {
+      visit(stmt.rhs, [&](const ExprRef& e) {
+        if (e->kind != Expr::Load || e->name != producer.tensor) return;
+        ok = ok && e->args.size() == lhs.size();
+        for (size_t j = 0; ok && j < lhs.size(); ++j) {
+          Affine x = ir::toAffine(e->args[j]);
+          ok = ok && x.valid && lhs[j].valid && x.constant == lhs[j].constant;
+          std::map<std::string, int64_t> renamed;
+          for (const auto& c : x.coef) {
+            if (c.second == 0) continue;
+            auto it = rename.find(c.first);
+            if (it == rename.end()) {
+              ok = false;
+              break;
+            }
+            renamed[it->second] += c.second;
+          }
+          std::map<std::string, int64_t> want;
+          for (const auto& c : lhs[j].coef) {
+            if (c.second != 0) want[c.first] = c.second;
+          }
+          ok = ok && renamed == want;
+        }
+      });
+    }
+    return ok;
+  }
+
   // --- whole stage ----------------------------------------------------------------------------
   void plan(int64_t& ldsBudgetBytes) {
     for (const auto& s : st_.stmts) {
@@ -2051,8 +2112,37 @@ void emitKernel(KernelCtx& kc, const DeviceLimits& limits, Emitter& em) {
     g.suppressCopy = true;
   }
   for (const auto& d : cacheDecls) em.line(d);
+  // Barriers between the stages: only where a later stage touches what an earlier one wrote (or
+  // overwrites what it read) through different threads, at the weakest sufficient level, placed
+  // by the exact search of sync_placement.h.  Every stage writes elements indexed by the
+  // kernel-level loop variables and reads other stages' results at the same indices, so nothing
+  // is carried from one iteration of those loops to the next.
+  std::vector<int> syncAfter(k.stages.size(), 0);
+  {
+    const int n = static_cast<int>(k.stages.size());
+    SyncNeeds need(n, std::vector<int>(n, 0));
+    const int level = static_cast<int>(kc.NT() <= limits.wavefront ? SyncLevel::Wave : SyncLevel::Block);
+    for (int i = 0; i < n; ++i) {
+      for (int j = i + 1; j < n; ++j) {
+        const StagePlan& a = k.stages[i];
+        const StagePlan& b = k.stages[j];
+        bool conflict = a.tensor == b.tensor || tensorsRead(b).count(a.tensor) || tensorsRead(a).count(b.tensor);
+        if (conflict && !gens[j].readsPrivatelyFrom(a)) need[i][j - i] = level;
+      }
+    }
+    for (const auto& sy : findBestSyncs(need, opened > 0)) syncAfter[sy.first] = static_cast<int>(sy.second);
+  }
+  auto emitSync = [&](int level) {
+    if (level == static_cast<int>(SyncLevel::Block)) {
+      em.line("__syncthreads();");
+    } else if (level == static_cast<int>(SyncLevel::Wave)) {
+      // the block is a single wavefront: order its memory operations, no hardware barrier
+      em.line("__builtin_amdgcn_fence(__ATOMIC_ACQ_REL, \"wavefront\");");
+      em.line("__builtin_amdgcn_wave_barrier();");
+    }
+  };
   for (size_t i = 0; i < k.stages.size(); ++i) {
-    if (i > 0) em.line("__syncthreads();");
+    if (i > 0) emitSync(syncAfter[i - 1]);
     if (k.stages[i].threadReduction) {
       em.open("");
       em.line(k.stages[i].views.at(k.stages[i].tensor).type.cName() + "* red_scratch_ = (" +
@@ -2070,7 +2160,7 @@ void emitKernel(KernelCtx& kc, const DeviceLimits& limits, Emitter& em) {
     for (const auto& p : g.promotions()) g.emitCopyStores(p, "pf_" + p.tensor + "_");
     em.close();
   }
-  if (k.stages.size() > 1 && opened > 0) em.line("__syncthreads();");
+  emitSync(syncAfter.back());
   for (int i = 0; i < opened; ++i) em.close();
   em.close();
 }

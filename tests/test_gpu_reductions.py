@@ -95,3 +95,22 @@ def test_moments_full_size_properties():
     Xd = X.astype(np.float64)
     assert np.abs(mean - Xd.mean(1)).max() <= W.tolerance(k, Xd.mean(1))
     assert np.abs(var - Xd.var(1)).max() <= W.tolerance(k, Xd.var(1))
+
+
+@pytest.mark.parametrize("threads,fragment", [(64, "__builtin_amdgcn_wave_barrier();"), (256, "__syncthreads();"), (32, "wave_barrier")])
+def test_moments_second_stage_sees_the_mean_across_threads(threads, fragment):
+    """The variance stage reads the mean that lane 0 stored: ordering inside one wavefront when
+    the block is a single wavefront, a block barrier otherwise."""
+    X = np.random.Generator(np.random.Philox(threads)).standard_normal((48, 2000), dtype=np.float32) + 3.0
+    ex = check(W.MOMENTS, "moments", [X], f"naive;tile=1;mapToBlocks=48;matchLibraryCalls=1;mapToThreads={threads}", 2000)
+    src = ex.compiled_source
+    assert fragment in src[src.index("// stage 0: mean"):src.index("// stage 1: var")]
+
+
+def test_point_wise_chain_needs_no_barrier():
+    chain = """def f(float(N, M) A) -> (O, P) {
+        O(i, j) = A(i, j) + 1.0
+        P(i, j) = O(i, j) * 2.0 }"""
+    A = np.random.Generator(np.random.Philox(77)).standard_normal((70, 130), dtype=np.float32)
+    ex = check(chain, "f", [A], "naive", 1)
+    assert "__syncthreads" not in ex.compiled_source and ex.num_kernels == 1

@@ -109,9 +109,38 @@ def test_fusion_strategies_decide_kernel_count():
     _, launches = mapped(W.GROUP_CONVOLUTION, "group_convolution", gc, MappingOptions.naive().scheduleFusionStrategy("Min"))
     assert len(launches) == 2
     src, launches = mapped(W.MOMENTS, "moments", [(64, 1024)], MappingOptions.naive())
-    assert len(launches) == 1 and "// stage 1: var" in src and "__syncthreads();" in src
+    # every thread owns whole rows: var re-reads the mean its own thread stored, no barrier
+    assert len(launches) == 1 and "// stage 1: var" in src
+    assert "__syncthreads" not in src and "wave_barrier" not in src
+    # reduction spread over threadIdx.x: lane 0 stores the mean the other threads read
+    rowwise = MappingOptions.naive().tile(1).mapToBlocks(64).matchLibraryCalls(True)
+    src, launches = mapped(W.MOMENTS, "moments", [(64, 1024)], rowwise.mapToThreads(64))
+    assert launches == [((64, 1, 1), (64, 1, 1))]                  # one wavefront: ordering only, no s_barrier
+    between = src[src.index("// stage 0: mean"):src.index("// stage 1: var")]
+    assert between.count("__builtin_amdgcn_wave_barrier();") == 1 and "__syncthreads" not in between
+    src, launches = mapped(W.MOMENTS, "moments", [(64, 1024)], rowwise.mapToThreads(256))
+    assert launches == [((64, 1, 1), (256, 1, 1))]
+    between = src[src.index("// stage 0: mean"):src.index("// stage 1: var")]
+    tail = between[between.rindex("pmean["):]                       # after the store of the mean
+    assert tail.count("__syncthreads();") == 1 and "wave_barrier" not in between
     _, launches = mapped(W.MOMENTS, "moments", [(64, 1024)], MappingOptions.naive().scheduleFusionStrategy("Min"))
     assert len(launches) == 2
+
+
+def test_barriers_between_stages_only_where_threads_exchange_data():
+    """Role of insertBestSyncInSeq (mapped_scop.cc:729-770) on the stage sequence of a kernel."""
+    chain = """def f(float(N, M) A) -> (O, P) {
+        O(i, j) = A(i, j) + 1.0
+        P(i, j) = O(i, j) * 2.0 }"""
+    src, launches = mapped(chain, "f", [(64, 64)], MappingOptions.naive())
+    assert len(launches) == 1 and "// stage 1: P" in src
+    assert "__syncthreads" not in src and "wave_barrier" not in src      # same thread produces and consumes
+    mirrored = """def g(float(N, M) A) -> (O, P) {
+        O(i, j) = A(i, j) + 1.0
+        P(i, j) = O(i, j) * 2.0 + O(i, M - 1 - j) }"""
+    src, launches = mapped(mirrored, "g", [(64, 64)], MappingOptions.naive().tile(32, 64).mapToThreads(64, 4))
+    if len(launches) == 1:                                             # fused: the mirrored read crosses threads
+        assert src.count("__syncthreads();") == 1
 
 
 def test_producer_consumer_matmuls_share_only_the_row_dimension():
