@@ -47,8 +47,12 @@ namespace detail {
 
 extern std::atomic<int> tunerSignal; // 0, SIGINT or SIGTERM while a tune() is running
 
-inline std::vector<size_t> inputDivisorsAndPowers2(const std::vector<const DLConstTensor*>& inputs) {
-  std::vector<size_t> sizes;
+// `extraSizes`: further extents loops of the TC run over.  The reference derives candidates from
+// the input shapes only; the output extents are added here because window-shaped accesses
+// (convolutions) loop over sizes that no input extent divides into.
+inline std::vector<size_t> inputDivisorsAndPowers2(
+    const std::vector<const DLConstTensor*>& inputs, const std::vector<size_t>& extraSizes = {}) {
+  std::vector<size_t> sizes = extraSizes;
   for (auto t : inputs) {
     for (int i = 0; i < t->ndim; ++i) sizes.push_back(static_cast<size_t>(t->shape[i]));
   }
@@ -62,9 +66,9 @@ inline std::vector<size_t> inputDivisorsAndPowers2(const std::vector<const DLCon
 // Candidate value sets derived from the input shapes (tc/autotuner/autotuner-inl.h:326-404).
 inline TuningConfiguration setupTuningParameters(
     const std::vector<const DLConstTensor*>& inputs, const std::vector<HipMappingOptions>& baseMappings,
-    size_t maxUnroll) {
+    size_t maxUnroll, const std::vector<size_t>& extraSizes = {}) {
   TC_CHECK_GE(inputs.size(), 1u);
-  std::vector<size_t> range = inputDivisorsAndPowers2(inputs);
+  std::vector<size_t> range = inputDivisorsAndPowers2(inputs, extraSizes);
   size_t maxRank = 0;
   for (auto t : inputs) maxRank = std::max<size_t>(maxRank, t->ndim);
   std::vector<size_t> tileRange = range;
@@ -146,7 +150,11 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
         canonicalTc, inputsInfo, outputsInfo, Backend::makeDeviceFilename(settings.cacheFile), settings.restoreNumber);
     bases.insert(bases.end(), restored.begin(), restored.end());
   }
-  TuningConfiguration space = detail::setupTuningParameters(firstInputs, bases, settings.maxUnroll);
+  std::vector<size_t> outputSizes;
+  for (const auto& info : outputsInfo) {
+    for (auto e : info.shape) outputSizes.push_back(static_cast<size_t>(e));
+  }
+  TuningConfiguration space = detail::setupTuningParameters(firstInputs, bases, settings.maxUnroll, outputSizes);
   space.fixParameters(fixedParams);
   std::vector<TuningConfiguration> configs;
   for (const auto& b : bases) {
