@@ -867,6 +867,9 @@ _PRELUDE = """#include <stdint.h>
 #include <math.h>
 static inline int64_t tc_floordiv(int64_t a, int64_t b) { int64_t q = a / b; return ((a % b != 0) && ((a < 0) != (b < 0))) ? q - 1 : q; }
 static inline int64_t tc_floormod(int64_t a, int64_t b) { return a - tc_floordiv(a, b) * b; }
+/* device builtins libm lacks (tc/lang/builtins.h:23-95 names them after the CUDA math library) */
+static inline float rsqrtf(float x) { return 1.0f / sqrtf(x); }
+static inline double rsqrt(double x) { return 1.0 / sqrt(x); }
 """
 
 

@@ -1,0 +1,184 @@
+"""The remaining workloads of the reference's benchmark suite and TC library (tc/benchmarks/*.h,
+tc/library/*.h) as parity cases: name -> (tc text, entry, inputs, reduction length for the
+tolerance).  An input is a shape (float32 normal values), ("int", shape, low, high) for int32
+indices, or ("scalar", value) for a 0-dimensional float parameter.  Sizes are small enough for the
+CPU oracle; the comprehensions are the reference's (transposed matmul tmm.cc:42-44, convolution
+library/convolution.h:27, fully connected + ReLU chains library/2fcrelu.h:22, look-up tables
+library/lut.h:23 and 2lut.h:23, spatial batch norm library/batchnorm.h:23, group normalisation
+benchmarks/group_normalization.h:27-58, Kronecker products benchmarks/kronecker.h:124-147,
+WaveNet layer benchmarks/wavenet.h:27-72)."""
+
+TMM = """
+def tmm(float(M, K) A, float(N, K) B) -> (C) {
+    C(m, n) +=! A(m, r_k) * B(n, r_k)
+}
+"""
+
+MATMUL = """
+def matmul(float(M, K) A, float(K, N) B) -> (O) {
+    O(m, n) +=! A(m, r_k) * B(r_k, n)
+}
+"""
+
+CONVOLUTION = """
+def convolution(float(N, C, H, W) I, float(M, C, KH, KW) W1, float(M) B) -> (O) {
+    O(n, m, h, w) +=! I(n, r_c, h + r_kh, w + r_kw) * W1(m, r_c, r_kh, r_kw)
+    O(n, m, h, w) = O(n, m, h, w) + B(m)
+}
+"""
+
+FCRELU2 = """
+def func_2fcrelu(float(B, M) I, float(N, M) W1, float(N) B1, float(O, N) W2, float(O) B2) -> (O1, O2) {
+    O1(b, n) +=! I(b, m) * W1(n, m)
+    O1(b, n) = O1(b, n) + B1(n)
+    O1(b, n) = fmax(O1(b, n), 0)
+    O2(b, o) +=! O1(b, n) * W2(o, n)
+    O2(b, o) = O2(b, o) + B2(o)
+    O2(b, o) = fmax(O2(b, o), 0)
+}
+"""
+
+LUT = """
+def lut(float(E, D) LUT, int32(B, L) I) -> (O) {
+    O(i, j) +=! LUT(I(i, k), j)
+}
+"""
+
+LUT2 = """
+def func_2lut(float(E1, D) LUT1, int32(B, L1) I1, float(E2, D) LUT2, int32(B, L2) I2) -> (O1, O2) {
+    O1(i, j) +=! LUT1(I1(i, k), j)
+    O2(i, j) +=! LUT2(I2(i, k), j)
+}
+"""
+
+BATCHNORM = """
+def spatialBatchNorm(float momentum, float eps, float(N, C, H, W) I, float(C) rMeanIn, float(C) rVarIn)
+-> (O, rMeanOut, rVarOut, mean, centered, variance, expectedVariance, normalizedOut)
+{
+    mean(c) +=! I(nn, c, hh, ww)
+    mean(c) = mean(c) / (N * H * W)
+    rMeanOut(c) = (1 - momentum) * rMeanIn(c) + momentum * mean(c)
+    centered(n, c, h, w) = I(n, c, h, w) - rMeanOut(c)
+    variance(n, c, h, w) = centered(n, c, h, w) * centered(n, c, h, w)
+    expectedVariance(c) +=! (variance(n, c, h, w) + eps) / (N * H * W)
+    rVarOut(c) = rsqrt((1 - momentum) * rVarIn(c) + momentum * expectedVariance(c))
+    O(n, c, h, w) = centered(n, c, h, w) * rVarOut(c)
+    normalizedOut(n, c, h, w) = O(n, c, h, w)
+}
+"""
+
+MOMENTS2 = """
+def moments2_2D_1D(float(N, K) I) -> (mean, var) {
+    mean(n) +=! I(n, r_k)
+    var(n) +=! I(n, r_k) * I(n, r_k)
+    mean(n) = mean(n) / (K)
+    var(n) = var(n) / (K) - mean(n) * mean(n)
+}
+"""
+
+GROUP_NORMALIZATION = """
+def group_normalization(float(N, G, D, H, W) I, float(G, D) gamma, float(G, D) beta,
+                        float(N, G) mean, float(N, G) var) -> (O) {
+    O(n, g, d, h, w) = gamma(g, d) * (I(n, g, d, h, w) - mean(n, g)) * rsqrt(var(n, g) + 1e-5) + beta(g, d)
+}
+"""
+
+GROUP_NORMALIZATION_SINGLE_KERNEL = """
+def group_normalization_single_kernel(float(N, G, D, H, W) I, float(G, D) gamma, float(G, D) beta)
+-> (O, sum, sumSquares) {
+    sum(n, g) +=! I(n, g, r_d, r_h, r_w)
+    sumSquares(n, g) +=! I(n, g, r_d, r_h, r_w) * I(n, g, r_d, r_h, r_w)
+    O(n, g, d, h, w) = gamma(g, d)
+        * (I(n, g, d, h, w) - sum(n, g) / (D * H * W))
+        * rsqrt(sumSquares(n, g) / (D * H * W) - sum(n, g) * sum(n, g) / (D * H * W) / (D * H * W) + 1e-5)
+        + beta(g, d)
+}
+"""
+
+KRONECKER3 = """
+def Kronecker3Full(float(D0, N0) W0, float(D1, N1) W1, float(D2, N2) W2, float(M, N0, N1, N2) X)
+-> (Y, XW2, XW2W1) {
+    XW2(m, n0, n1, d2) +=! X(m, n0, n1, r_n2) * W2(d2, r_n2)
+    XW2W1(m, n0, d1, d2) +=! XW2(m, n0, r_n1, d2) * W1(d1, r_n1)
+    Y(m, d0, d1, d2) +=! XW2W1(m, r_n0, d1, d2) * W0(d0, r_n0)
+}
+"""
+
+WAVENET1 = """
+def wavenet1(
+    float(B, RESIDUAL_C, RECEPTIVE_FIELD) Data,
+    float(DILATION_C, RESIDUAL_C, 2) FilterWeight,
+    float(DILATION_C) FilterBias,
+    float(DILATION_C, RESIDUAL_C, 2) GateWeight,
+    float(DILATION_C) GateBias,
+    float(RESIDUAL_C, DILATION_C) ResWeight,
+    float(RESIDUAL_C) ResBias,
+    float(SKIP_C, DILATION_C) SkipWeight,
+    float(SKIP_C) SkipBias,
+    float(DILATION_FACTOR) Dilation)
+    -> (FilterOut, GateOut, NonLin, Res, Skip)
+{
+    FilterOut(b, dilation_c, rf) = FilterBias(dilation_c)
+        where b in 0:B, dilation_c in 0:DILATION_C, rf in 0:RECEPTIVE_FIELD
+    FilterOut(b, dilation_c, rf) += Data(b, r_residual_c, rf) * FilterWeight(dilation_c, r_residual_c, 1) +
+        ((rf - DILATION_FACTOR >= 0) ?
+            Data(b, r_residual_c, rf - DILATION_FACTOR) * FilterWeight(dilation_c, r_residual_c, 0) : float(0))
+        where rf in 0:RECEPTIVE_FIELD
+    GateOut(b, dilation_c, rf) = GateBias(dilation_c)
+        where b in 0:B, dilation_c in 0:DILATION_C, rf in 0:RECEPTIVE_FIELD
+    GateOut(b, dilation_c, rf) += Data(b, r_residual_c, rf) * GateWeight(dilation_c, r_residual_c, 1) +
+        ((rf - DILATION_FACTOR >= 0) ?
+            Data(b, r_residual_c, rf - DILATION_FACTOR) * GateWeight(dilation_c, r_residual_c, 0) : float(0))
+        where rf in 0:RECEPTIVE_FIELD
+    NonLin(b, dilation_c, rf) = tanh(FilterOut(b, dilation_c, rf))
+        where rf in 0:RECEPTIVE_FIELD
+    NonLin(b, dilation_c, rf) *= 1 / (1 + exp(-GateOut(b, dilation_c, rf)))
+        where rf in 0:RECEPTIVE_FIELD
+    Res(b, residual_c, rf) = Data(b, residual_c, rf) + ResBias(residual_c)
+    Res(b, residual_c, rf) += NonLin(b, r_dilation_c, rf) * ResWeight(residual_c, r_dilation_c)
+    Skip(b, skip, rf) +=! NonLin(b, r_dilation_c, rf) * SkipWeight(skip, r_dilation_c)
+        where rf in 0:RECEPTIVE_FIELD
+    Skip(b, skip, rf) = Skip(b, skip, rf) + SkipBias(skip)
+        where rf in 0:RECEPTIVE_FIELD
+}
+"""
+
+CASES = {
+    "tmm": (TMM, "tmm", [(32, 256), (128, 256)], 256),
+    "tmm_odd": (TMM, "tmm", [(37, 70), (51, 70)], 70),
+    "matmul": (MATMUL, "matmul", [(72, 60), (60, 50)], 60),
+    "convolution": (CONVOLUTION, "convolution", [(3, 4, 12, 11), (8, 4, 3, 3), (8,)], 36),
+    "2fcrelu": (FCRELU2, "func_2fcrelu", [(20, 48), (36, 48), (36,), (24, 36), (24,)], 48),
+    "lut": (LUT, "lut", [(50, 24), ("int", (9, 7), 0, 50)], 7),
+    "2lut": (LUT2, "func_2lut", [(50, 24), ("int", (9, 7), 0, 50), (30, 24), ("int", (9, 5), 0, 30)], 7),
+    "batchnorm": (BATCHNORM, "spatialBatchNorm",
+                  [("scalar", 0.1), ("scalar", 1e-5), (4, 6, 7, 5), (6,), ("positive", (6,))], 140),
+    "moments2": (MOMENTS2, "moments2_2D_1D", [(24, 500)], 500),
+    "group_normalization": (GROUP_NORMALIZATION, "group_normalization",
+                            [(3, 4, 5, 6, 7), (4, 5), (4, 5), (3, 4), ("positive", (3, 4))], 1),
+    "group_normalization_single_kernel": (GROUP_NORMALIZATION_SINGLE_KERNEL, "group_normalization_single_kernel",
+                                          [(3, 4, 5, 6, 7), (4, 5), (4, 5)], 210),
+    "kronecker3": (KRONECKER3, "Kronecker3Full", [(6, 5), (7, 4), (8, 3), (10, 5, 4, 3)], 5),
+    "wavenet1": (WAVENET1, "wavenet1",
+                 [(1, 8, 100), (8, 8, 2), (8,), (8, 8, 2), (8,), (8, 8), (8,), (16, 8), (16,), (2,)], 16),
+}
+
+
+def make_inputs(name, seed=2024):
+    import numpy as np
+    rng = np.random.Generator(np.random.Philox(seed))
+    out = []
+    for spec in CASES[name][2]:
+        if isinstance(spec[0], str):
+            kind = spec[0]
+            if kind == "int":
+                out.append(rng.integers(spec[2], spec[3], size=spec[1]).astype(np.int32))
+            elif kind == "scalar":
+                out.append(np.array(spec[1], dtype=np.float32))
+            elif kind == "positive":
+                out.append((rng.random(spec[1], dtype=np.float32) + 0.5).astype(np.float32))
+            else:
+                raise ValueError(kind)
+        else:
+            out.append(rng.standard_normal(spec, dtype=np.float32))
+    return out

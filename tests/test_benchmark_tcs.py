@@ -1,0 +1,99 @@
+"""The other workloads of the reference's benchmark suite (tests/benchmark_tcs.py): the oracle is
+pinned against the library routines the reference's own benchmarks check with (at::mm, conv2d,
+relu(addmm), embedding sums, group norm; tc/benchmarks/*.cc), and every case must map and JIT for
+gfx950 under several mapping options (hipRTC needs no GPU)."""
+import numpy as np
+import pytest
+import torch
+
+import tensorcomprehensions_amd as tc
+from oracle import tc_oracle
+from tests import benchmark_tcs as B
+
+OPTION_SETS = {
+    "naive": "naive",
+    "tiled_lds": "naive;tile=4,16,8;mapToThreads=16,4;mapToBlocks=64,64;useSharedMemory=1;unroll=16",
+    "library_reductions": "naive;tile=1,1;mapToThreads=64;mapToBlocks=128,128;matchLibraryCalls=1;unroll=4",
+    "matrix_cores": "naive;tile=32,32,0;mapToThreads=64,4;mapToBlocks=64,64;useMfma=1;useSharedMemory=1",
+}
+
+
+def f64(a):
+    return torch.from_numpy(np.asarray(a, dtype=np.float64))
+
+
+def close(got, want, k):
+    want = want.numpy() if isinstance(want, torch.Tensor) else want
+    scale = max(1.0, float(np.abs(want).max()))
+    assert got.shape == want.shape
+    assert np.abs(got - want).max() <= 1e-5 * np.sqrt(k) * scale
+
+
+def test_oracle_matches_library_routines():
+    ins = B.make_inputs("tmm")
+    close(tc_oracle.run(B.TMM, "tmm", ins)[0], f64(ins[0]) @ f64(ins[1]).T, 256)
+    ins = B.make_inputs("matmul")
+    close(tc_oracle.run(B.MATMUL, "matmul", ins)[0], f64(ins[0]) @ f64(ins[1]), 60)
+    ins = B.make_inputs("convolution")
+    ref = torch.nn.functional.conv2d(f64(ins[0]), f64(ins[1]), f64(ins[2]))
+    close(tc_oracle.run(B.CONVOLUTION, "convolution", ins)[0], ref, 36)
+    I, W1, B1, W2, B2 = B.make_inputs("2fcrelu")
+    o1 = torch.relu(f64(I) @ f64(W1).T + f64(B1))
+    o2 = torch.relu(o1 @ f64(W2).T + f64(B2))
+    got = tc_oracle.run(B.FCRELU2, "func_2fcrelu", [I, W1, B1, W2, B2])
+    close(got[0], o1, 48)
+    close(got[1], o2, 48 * 36)
+    lut, idx = B.make_inputs("lut")
+    close(tc_oracle.run(B.LUT, "lut", [lut, idx])[0], f64(lut)[torch.from_numpy(idx).long()].sum(1), 7)
+    X, = B.make_inputs("moments2")
+    mean, var = tc_oracle.run(B.MOMENTS2, "moments2_2D_1D", [X])
+    close(mean, f64(X).mean(1), 500)
+    close(var, f64(X).var(1, unbiased=False), 500)
+    I, gamma, beta = B.make_inputs("group_normalization_single_kernel")
+    ref = torch.nn.functional.group_norm(f64(I).reshape(3, 20, 6, 7), 4, eps=1e-5).reshape(3, 4, 5, 6, 7)
+    ref = ref * f64(gamma)[None, :, :, None, None] + f64(beta)[None, :, :, None, None]
+    got = tc_oracle.run(B.GROUP_NORMALIZATION_SINGLE_KERNEL, "group_normalization_single_kernel", [I, gamma, beta])
+    close(got[0], ref, 210)
+    close(got[1], f64(I).sum((2, 3, 4)), 210)
+    W0, W1k, W2k, X = B.make_inputs("kronecker3")
+    ref = torch.einsum("mabc,xa,yb,zc->mxyz", f64(X), f64(W0), f64(W1k), f64(W2k))
+    close(tc_oracle.run(B.KRONECKER3, "Kronecker3Full", [W0, W1k, W2k, X])[0], ref, 60)
+
+
+def test_oracle_batchnorm_and_wavenet_closed_forms():
+    momentum, eps, I, rMeanIn, rVarIn = B.make_inputs("batchnorm")
+    out = dict(zip(["O", "rMeanOut", "rVarOut", "mean", "centered", "variance", "expectedVariance", "normalizedOut"],
+                   tc_oracle.run(B.BATCHNORM, "spatialBatchNorm", [momentum, eps, I, rMeanIn, rVarIn])))
+    x = f64(I)
+    mean = x.mean((0, 2, 3))
+    rmean = (1 - 0.1) * f64(rMeanIn) + float(np.float32(0.1)) * mean
+    centered = x - rmean[None, :, None, None]
+    ev = (centered * centered + float(np.float32(1e-5))).mean((0, 2, 3))
+    rvar = 1.0 / torch.sqrt((1 - 0.1) * f64(rVarIn) + float(np.float32(0.1)) * ev)
+    close(out["mean"], mean, 140)
+    close(out["rMeanOut"], rmean, 140)
+    close(out["expectedVariance"], ev, 140)
+    close(out["rVarOut"], rvar, 140)
+    close(out["O"], centered * rvar[None, :, None, None], 140)
+    assert np.array_equal(out["O"], out["normalizedOut"])
+    ins = B.make_inputs("wavenet1")
+    data, fw, fb, gw, gb, rw, rb, sw, sb, dil = [f64(a) for a in ins]
+    shifted = torch.zeros_like(data)
+    shifted[:, :, 2:] = data[:, :, :-2]                  # DILATION_FACTOR = extent of `Dilation` = 2
+    filt = fb[None, :, None] + torch.einsum("bcr,dc->bdr", data, fw[:, :, 1]) + torch.einsum("bcr,dc->bdr", shifted, fw[:, :, 0])
+    gate = gb[None, :, None] + torch.einsum("bcr,dc->bdr", data, gw[:, :, 1]) + torch.einsum("bcr,dc->bdr", shifted, gw[:, :, 0])
+    nonlin = torch.tanh(filt) * torch.sigmoid(gate)
+    res = data + rb[None, :, None] + torch.einsum("bdr,cd->bcr", nonlin, rw)
+    skip = torch.einsum("bdr,sd->bsr", nonlin, sw) + sb[None, :, None]
+    got = tc_oracle.run(B.WAVENET1, "wavenet1", ins)
+    for g, want in zip(got, [filt, gate, nonlin, res, skip]):
+        close(g, want, 16)
+
+
+@pytest.mark.parametrize("options", sorted(OPTION_SETS))
+@pytest.mark.parametrize("name", sorted(B.CASES))
+def test_every_case_maps_and_compiles_for_gfx950(name, options):
+    src, entry, _, _ = B.CASES[name]
+    shapes = [tc.ShapeOnly(a.shape, str(a.dtype)) for a in B.make_inputs(name)]
+    ex = tc.compile(src, entry, shapes, OPTION_SETS[options])
+    assert ex.num_kernels >= 1 and "__global__" in ex.compiled_source

@@ -1,0 +1,54 @@
+"""HIP backend vs the CPU oracle on the other workloads of the reference's benchmark suite
+(transposed matmul, convolution, fully connected chains, look-up tables with indirect indexing,
+batch and group normalisation, Kronecker products, a WaveNet layer), under plain, tiled + LDS,
+thread-mapped-reduction and matrix-core mapping options."""
+import numpy as np
+import pytest
+import torch
+
+import tensorcomprehensions_amd as tc
+from oracle import tc_oracle
+from tests import benchmark_tcs as B
+from tests.test_benchmark_tcs import OPTION_SETS
+
+pytestmark = pytest.mark.gpu
+
+# reductions feeding later reductions: tolerance on the product of the lengths
+CHAINED = {"2fcrelu": 48 * 36, "kronecker3": 60, "batchnorm": 140, "wavenet1": 16 * 8,
+           "group_normalization_single_kernel": 210}
+
+
+@pytest.mark.parametrize("options", sorted(OPTION_SETS))
+@pytest.mark.parametrize("name", sorted(B.CASES))
+def test_parity_with_oracle(name, options):
+    src, entry, _, k = B.CASES[name]
+    print(f"case {name} options {options}", flush=True)
+    ins_np = B.make_inputs(name)
+    ref = tc_oracle.run(src, entry, ins_np)
+    ins = [torch.from_numpy(a).cuda() for a in ins_np]
+    ex = tc.compile(src, entry, ins, OPTION_SETS[options])
+    outs = tc.prepare_outputs(src, entry, ins)
+    for o in outs:
+        o.fill_(float("nan"))
+    tc.run(ex, ins, outs)
+    torch.cuda.synchronize()
+    k = CHAINED.get(name, k)
+    for o, r in zip(outs, ref):
+        got = o.cpu().numpy()
+        assert got.shape == r.shape
+        scale = max(1.0, float(np.abs(r).max()))
+        assert np.abs(got - r).max() <= 1e-5 * np.sqrt(k) * scale, (name, options, ex.launch_bounds())
+
+
+def test_lookup_indices_are_exact():
+    """Indirect indexing with integer-valued tables: sums are exact, any wrong row shows."""
+    rng = np.random.Generator(np.random.Philox(5))
+    lut = rng.integers(-8, 9, size=(50, 24)).astype(np.float32)
+    idx = rng.integers(0, 50, size=(9, 7)).astype(np.int32)
+    ref = tc_oracle.run(B.LUT, "lut", [lut, idx])[0]
+    ins = [torch.from_numpy(lut).cuda(), torch.from_numpy(idx).cuda()]
+    for options in ("naive", OPTION_SETS["tiled_lds"], OPTION_SETS["library_reductions"]):
+        ex = tc.compile(B.LUT, "lut", ins, options)
+        (out,) = tc.prepare_outputs(B.LUT, "lut", ins)
+        tc.run(ex, ins, [out])
+        assert np.array_equal(out.cpu().numpy(), ref)

@@ -81,3 +81,17 @@ def test_matches_exhaustive_search_on_random_instances():
         assert covered(n, cyclic, need, at), (n, cyclic, need, at)
         cost = (at.count(2), at.count(1))
         assert cost == brute_force(n, cyclic, need), (n, cyclic, need, at)
+
+
+def test_dense_random_requirements_as_in_the_reference_test():
+    """Same experiment as SyncConfigInSeqOptimalityTest (test/test_cuda_mapper.cc:168-350): every
+    entry of the requirement matrix uniform in {0, 1, 2}, 2-4 children, with and without a loop."""
+    for cyclic in (False, True):
+        for n in range(2, 5):
+            for seed in range(50):
+                rng = random.Random(seed * 10 + n)
+                need = {(i, k): rng.randint(0, 2) for i in range(n) for k in range(n)}
+                need = {key: lev for key, lev in need.items() if lev}
+                at = solve(n, cyclic, need)
+                assert covered(n, cyclic, need, at), (n, cyclic, need, at)
+                assert (at.count(2), at.count(1)) == brute_force(n, cyclic, need), (n, cyclic, need, at)
