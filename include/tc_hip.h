@@ -141,6 +141,15 @@ int tc_autotune(
     const tc_dl_tensor* const* outputs, int num_outputs,
     const char* base_options, const char* settings, char** best);
 
+/* The `count` best options recorded for this TC and these input sizes in an options cache file
+ * written by a tuning run (`cache_file` setting); an empty text when the file or the entry is
+ * missing.  loadTopKFromCacheFile, tc/autotuner/options_cache-inl.h:338-356, as used by
+ * make_load_from_cache_options_factory (tensor_comprehensions/__init__.py:278-296). */
+int tc_options_cache_load(
+    const char* tc, const char* entry_point,
+    const tc_dl_tensor* const* inputs, int num_inputs,
+    const char* cache_file, int count, char** best);
+
 /* Host-side tuner logic without a device, for bindings and tests:
  *   "powers2_and_ceil_divisors", "72"  -> "1,2,3,4,5,8,9,..."   (tc/autotuner/utils.cc:42-56)
  *   "search_space", "<shape>;<shape>..." e.g. "500x26x72;500x72x26" -> candidate value sets

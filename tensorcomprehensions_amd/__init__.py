@@ -87,8 +87,21 @@ class Executor:
 
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
-        if h:
+        if h and _capi is not None:                      # module globals are gone at interpreter exit
             _capi.lib().tc_executor_destroy(h)
+
+    def __call__(self, *inputs, outputs=None, unchecked=False):
+        """Run on `inputs`; allocates the outputs unless given.  Returns one tensor or a tuple, like
+        the reference's Executor.__call__ (tensor_comprehensions/__init__.py:80-121)."""
+        if outputs is None:
+            if self._signature is None:
+                raise TcError("outputs must be passed: this executor does not know its TC")
+            outputs = prepare_outputs(self._signature[0], self._signature[1], list(inputs))
+        outputs = list(outputs) if isinstance(outputs, (list, tuple)) else [outputs]
+        (unchecked_run if unchecked else run)(self, list(inputs), outputs)
+        return outputs[0] if len(outputs) == 1 else tuple(outputs)
+
+    _signature = None
 
     @property
     def compiled_source(self):
@@ -158,7 +171,9 @@ def compile(tc, entry_point, inputs, options=None):
     handle = ctypes.c_void_p()
     _capi.check(_capi.lib().tc_compile(tc.encode(), entry_point.encode(), pack.ptr, len(pack),
                                        _opt_text(options), ctypes.byref(handle)))
-    return Executor(handle)
+    ex = Executor(handle)
+    ex._signature = (tc, entry_point)
+    return ex
 
 
 def run(executor, inputs, outputs):
@@ -235,3 +250,19 @@ def autotune(tc, entry_point, inputs, base_options=None, outputs=None, **setting
     _capi.check(_capi.lib().tc_autotune(tc.encode(), entry_point.encode(), pin.ptr, len(pin), pout.ptr, len(pout),
                                         _opt_text(base_options), text.encode(), ctypes.byref(best)))
     return [MappingOptions(line) for line in _capi.take_string(best).splitlines() if line]
+
+
+def load_from_cache(tc, entry_point, inputs, cache_file, count=1):
+    """The `count` best options a tuning run stored for this TC and these sizes in `cache_file`
+    (the reference's MappingOptionsCache.load, tensor_comprehensions/__init__.py:278-296); [] when
+    the file or the entry is missing."""
+    pack = _pack(inputs)
+    best = ctypes.c_void_p()
+    _capi.check(_capi.lib().tc_options_cache_load(tc.encode(), entry_point.encode(), pack.ptr, len(pack),
+                                                  str(cache_file).encode(), int(count), ctypes.byref(best)))
+    return [MappingOptions(line) for line in _capi.take_string(best).splitlines() if line]
+
+
+from .highlevel import (TC, TunerConfig, assert_almost_equal, autotune_and_compile, define,  # noqa: E402
+                        make_autotuned_options_factory, make_load_from_cache_options_factory,
+                        make_naive_options_factory)

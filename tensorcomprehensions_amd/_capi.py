@@ -101,6 +101,8 @@ def _declare(l):
     l.tc_host_query.argtypes = [ctypes.c_char_p, ctypes.c_char_p, P(ctypes.c_void_p)]
     l.tc_autotune.argtypes = [ctypes.c_char_p, ctypes.c_char_p, tensors, ctypes.c_int, tensors, ctypes.c_int,
                               ctypes.c_char_p, ctypes.c_char_p, P(ctypes.c_void_p)]
+    l.tc_options_cache_load.argtypes = [ctypes.c_char_p, ctypes.c_char_p, tensors, ctypes.c_int, ctypes.c_char_p,
+                                        ctypes.c_int, P(ctypes.c_void_p)]
 
 
 def check(status):

@@ -93,6 +93,32 @@ extern "C" int tc_autotune(
   }
 }
 
+extern "C" int tc_options_cache_load(
+    const char* tcText, const char* entry, const tc_dl_tensor* const* inputs, int numInputs,
+    const char* cacheFile, int count, char** best) {
+  using namespace tc;
+  try {
+    auto defs = tc::detail::parse(tcText);
+    TC_CHECK_EQ(defs.count(entry), 1u) << "attempting to access undefined function " << entry;
+    CompilerOptions quiet;
+    quiet.emitWarnings = false;
+    std::ostringstream canon;
+    canon << lang::canonicalize(lang::Sema(quiet).checkFunction(defs.at(entry)));
+    auto in = capi::constTensors(inputs, numInputs);
+    auto inputsInfo = makeTensorInfoVector(in);
+    auto outputsInfo = tc::inferOutputTensorInfo(tcText, entry, in);
+    auto found = autotune::loadTopKFromCacheFile<HipBackend>(
+        canon.str(), inputsInfo, outputsInfo, HipBackend::makeDeviceFilename(cacheFile), static_cast<size_t>(std::max(count, 0)));
+    std::string text;
+    for (const auto& o : found) text += o.toText() + "\n";
+    *best = capi::dupString(text);
+    return 0;
+  } catch (const std::exception& e) {
+    tc::capi::lastError = e.what();
+    return 1;
+  }
+}
+
 // ------------------------------------------------------------------------------------------
 // tc_host_query: tuner logic that needs no device
 // ------------------------------------------------------------------------------------------

@@ -124,3 +124,36 @@ def test_autotune_survives_unmappable_candidates():
     A, B = torch.randn(64, 64, device="cuda"), torch.randn(64, 64, device="cuda")
     best = tc.autotune(MM, "matmul", [A, B], "naive", generations=2, pop_size=6, threads=4, seed=3, top_k=2)
     assert 1 <= len(best) <= 2
+
+
+def test_define_compiles_on_demand_and_memoises():
+    defs = """
+    def add(float(N) A, float(N) B) -> (C) { C(i) = A(i) + B(i) }
+    def scale(float(N) A) -> (C) { C(i) = A(i) * 2.0 }
+    """
+    T = tc.define(defs, tc.make_naive_options_factory())
+    a, b = torch.randn(1000, device="cuda"), torch.randn(1000, device="cuda")
+    assert torch.equal(T.add(a, b), a + b)
+    assert torch.equal(T.scale(a), a * 2)
+    assert len(T._executors) == 2
+    out = torch.empty_like(a)
+    assert T.add(b, a, outputs=[out]) is out and torch.equal(out, a + b)
+    assert len(T._executors) == 2                      # same sizes: no recompilation
+    T.add(a[:10].contiguous(), b[:10].contiguous())
+    assert len(T._executors) == 3
+    tc.assert_almost_equal(T.add(a, b), a + b, a, b, operations=1)
+
+
+def test_autotune_and_compile_with_cache_round_trip(tmp_path):
+    src = "def add(float(N, M) A, float(N, M) B) -> (C) { C(i, j) = A(i, j) + B(i, j) }"
+    a, b = torch.randn(64, 300, device="cuda"), torch.randn(64, 300, device="cuda")
+    cache = str(tmp_path / "options")
+    cfg = tc.TunerConfig().generations(2).pop_size(6).threads(4).seed(3)
+    add = tc.autotune_and_compile(src, "add", a, b, starting_options="naive", tuner_config=cfg,
+                                  cache_filename=cache, store_to_cache=True)
+    assert torch.equal(add(a, b), a + b)
+    stored = tc.load_from_cache(src, "add", [a, b], cache, 3)
+    assert 1 <= len(stored) <= 3
+    T = tc.define(src, tc.make_load_from_cache_options_factory(cache))
+    assert torch.equal(T.add(a, b), a + b)
+    assert tc.load_from_cache(src, "add", [a[:8].contiguous(), b[:8].contiguous()], cache) == []   # other sizes
