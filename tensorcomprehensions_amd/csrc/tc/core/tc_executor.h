@@ -26,7 +26,8 @@ void checkSizesAndStridesAreCompliant(
     const DLT* t = actual[i];
     const TensorInfo& e = expected[i];
     TC_CHECK_EQ(static_cast<size_t>(t->ndim), e.shape.size())
-        << what << " " << i << ": expected " << e.shape.size() << " dimensions";
+        << what << " " << i << ": expected " << e.shape.size() << " dimensions but found tensor with " << t->ndim
+        << " dimensions";
     TC_CHECK(t->dtype.code == e.dtype.code && t->dtype.bits == e.dtype.bits)
         << what << " " << i << ": expected " << toString(e.dtype) << " but found " << toString(t->dtype);
     for (int d = 0; d < t->ndim; ++d) {

@@ -1,0 +1,129 @@
+"""The reference's corner cases (test/cuda/test_corner_cases.cc:82-345): short programs that must
+either fail with a recognisable message or run.  Failures are raised while compiling, so they are
+checked without a GPU; the ones that must run are GPU tests and compare values as the reference
+does."""
+import numpy as np
+import pytest
+import torch
+
+import tensorcomprehensions_amd as tc
+
+
+def F(*shape):
+    return tc.ShapeOnly(shape, "float32")
+
+
+def I(*shape):
+    return tc.ShapeOnly(shape, "int32")
+
+
+FAILS = {
+    "E1": ("expected (", " def f{} {}", []),
+    "E7": ("expected 2 inputs", "def f(float a, float c) -> (b) { b(i) = a where i in 0:10 }", [F()]),
+    "E8": ("expected type int32", "def f(int32 a) -> (b) { b(i) = a where i in 0:10 }", [F()]),
+    "E9": ("expected a tensor with 0", "def f(int32 a) -> (b) { b(i) = a where i in 0:10 }", [I(1, 2)]),
+    "E11": ("expected integral type", "def f(int32(N) a) -> (b) { b(i) = a(i + .5) }", [I(10)]),
+    "E12": ("tensor accesses cannot be used in this context",
+            "def f(int32 a, float(N) b) -> (c) { c(i) += b(i + j) where j in 0:a, i in 0:10 }", [I(), F(12)]),
+    "E13": ("tensor accesses cannot be used in this context",
+            "def f(int32 a, float(N) b) -> (c) { c(i) += b(i + j) where j in 0:a }", [I(), F(12)]),
+    "E19": ("undefined variable", "def f(float(1) a) -> (b) { b(i) = 2*foo where foo = a(i), foo in 1:2 }", [F(1)]),
+    "E20": ("Temporaries tensors", "def f(float(1) a) -> (b) { c(i) = a(i) b(i) = c(i)  }", [F(1)]),
+}
+
+
+@pytest.mark.parametrize("case", sorted(FAILS))
+def test_fails_with_the_expected_fragment(case):
+    fragment, src, inputs = FAILS[case]
+    with pytest.raises(tc.TcError) as e:
+        tc.compile(src, "f", inputs, "naive")
+    assert fragment in str(e.value), str(e.value)
+
+
+def run(src, *inputs):
+    ins = [torch.as_tensor(x).cuda() for x in inputs]
+    ex = tc.compile(src, "f", ins, "naive")
+    outs = tc.prepare_outputs(src, "f", ins)
+    tc.run(ex, ins, outs)
+    torch.cuda.synchronize()
+    return [o.cpu() for o in outs]
+
+
+@pytest.mark.gpu
+def test_degenerate_shapes_run():
+    a = torch.tensor([3.5])
+    assert run("def f(float(1) a) -> (b) { b(i) = a(i) }", a)[0].tolist() == [3.5]                      # E2
+    s = torch.tensor(2.25)
+    (b,) = run("def f(float a) -> (b) { b = a }", s)                                                      # E4
+    assert b.dim() == 0 and b.item() == 2.25
+    assert run("def f(float a) -> (b) { b(i) = a where i in 0:10 }", s)[0].tolist() == [2.25] * 10        # E6
+    (b,) = run("def f(int32 a) -> (b) { b(i) = a where i in 0:10 }", torch.tensor(7, dtype=torch.int32))  # E10
+    assert b.dtype == torch.int32 and b.tolist() == [7] * 10
+
+
+@pytest.mark.gpu
+def test_wrong_output_rank_is_refused_at_run_time():
+    src = "def f(float(1) a) -> (b) { b(i) = a(i) }"                                                     # E25
+    a = torch.ones(1).cuda()
+    ex = tc.compile(src, "f", [a], "naive")
+    with pytest.raises(tc.TcError) as e:
+        tc.run(ex, [a], [torch.ones(1, 1).cuda()])
+    assert "expected 1 dimensions but found tensor with 2 dimensions" in str(e.value)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("op", ["<=", ">=", "==", "!=", "<", ">"])
+def test_comparisons(op):                                                                                # E15
+    for x, y in ((0.25, 0.75), (0.75, 0.25), (0.5, 0.5)):
+        (c,) = run(f"def f(float a, float b) -> (c) {{ c(i) = float(a {op} b) where i in 0:1 }}", torch.tensor(x), torch.tensor(y))
+        assert c.item() == float(eval(f"{x} {op} {y}"))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("op,py", [("||", "or"), ("&&", "and")])
+def test_boolean_operators_and_precedence(op, py):                                                       # E16
+    for x in (0.25, 0.75):
+        for y in (0.25, 0.75):
+            (c,) = run(f"def f(float a, float b) -> (c) {{ c(i) = float(!(a < .5) {op} b > .5) where i in 0:1 }}",
+                       torch.tensor(x), torch.tensor(y))
+            assert c.item() == float(eval(f"(not ({x} < .5)) {py} ({y} > .5)"))
+
+
+@pytest.mark.gpu
+def test_exists_let_min_max_and_newlines():
+    a, b, c = torch.tensor([0.3]), torch.tensor([0.9]), torch.tensor([0.6])
+    assert run("def f(float(1) a) -> (b) { b(i) = 4.0 where exists a(i) }", a)[0].item() == 4.0           # E17
+    assert run("def f(float(1) a) -> (b) { b(i) = 2*foo where foo = a(i) }", a)[0].item() == pytest.approx(0.6)  # E18
+    assert run("def f(float(1) a, float(1) b) -> (c) { c(i) = max(a(i), b(i)) }", a, b)[0].item() == pytest.approx(0.9)  # E21
+    assert run("def f(float(1) a, float(1) b) -> (c) { c(i) = min(a(i), b(i)) }", a, b)[0].item() == pytest.approx(0.3)  # E22
+    src = "def f(float(1) a, float(1) b, float(1) c) -> (d) { d(i) = min(a(i), max(b(i), c(i))) }"      # E23
+    assert run(src, a, b, c)[0].item() == pytest.approx(min(0.3, max(0.9, 0.6)))
+    ragged = """
+
+def f(float(1)
+a, float(1
+) b, float
+(1) c) -> (d) { d(
+i)
+ =
+
+ min(
+a(i), max(
+b(i), c(
+i)))
+
+d(i) = d(i) + max(b(i),
+
+c(
+i))
+
+}
+"""
+    assert run(ragged, a, b, c)[0].item() == pytest.approx(min(0.3, max(0.9, 0.6)) + max(0.9, 0.6))      # E24
+
+
+@pytest.mark.gpu
+def test_integer_modulo():                                                                               # E26
+    (r,) = run("def f(int32 a, int32 b) -> (c) { c(i) = int32(a % b) where i in 0:1 }",
+               torch.tensor(17, dtype=torch.int32), torch.tensor(5, dtype=torch.int32))
+    assert r.dtype == torch.int32 and r.item() == 17 % 5
