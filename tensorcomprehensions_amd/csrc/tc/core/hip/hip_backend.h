@@ -39,6 +39,11 @@ struct HipBackend {
   using WithDevice = WithHipDevice;
   using RuntimeInformation = HipRuntimeInformation;
   using MappingOptionsAsCpp = HipMappingOptionsAsCpp;
+  using MappingOptionsCppPrinter = HipMappingOptionsCppPrinter;
+  // Cache files are written with a hand-rolled proto2 wire codec: the "proto types" are the
+  // serialized messages (tc/proto/compcache.proto:20-62 with the HIP options message as value).
+  using OptionsCacheProtoType = std::string;
+  using OptionsCacheValueProtoType = std::string;
 
   // device name; part of the tuning-cache key
   static std::string backendString() { return HipGPUInfo::GPUInfo().GetGPUName(); }

@@ -249,4 +249,20 @@ class HipMappingOptionsAsCpp {
 };
 std::ostream& operator<<(std::ostream& os, const HipMappingOptionsAsCpp& o);
 
+// Stream wrapper with the reference printer's calling convention
+// (`HipMappingOptionsCppPrinter(out, indent) << options`,
+// tc/core/cuda/cuda_mapping_options_cpp_printer.h:34-46).
+class HipMappingOptionsCppPrinter {
+ public:
+  explicit HipMappingOptionsCppPrinter(std::ostream& out, size_t ws = 0) : out_(out), ws_(ws) {}
+  friend HipMappingOptionsCppPrinter& operator<<(HipMappingOptionsCppPrinter& prn, const HipMappingOptions& options) {
+    prn.out_ << HipMappingOptionsAsCpp(options, prn.ws_);
+    return prn;
+  }
+
+ private:
+  std::ostream& out_;
+  size_t ws_;
+};
+
 } // namespace tc
