@@ -123,6 +123,34 @@ def cpu_baseline(name, budget_s=15.0):
             "sample": f"full {name} workload, median of {len(times)} runs of the sequential loop nest, {med * 1e3:.1f} ms each"}
 
 
+def aten_cpu_baseline(name, budget_s=10.0):
+    """The library routine the reference's own benchmarks compare with (at::einsum / bmm / conv2d / mean, var)
+    on the host cores with torch's default intra-op threads; None for workloads without one."""
+    import torch
+    from tests import workloads as W
+    ins = [torch.from_numpy(a) for a in W.make_inputs(name)]
+    fn = {
+        "c1_tensordot_small": lambda: torch.einsum("nachw,ncbhw->nabhw", ins[0], ins[1]),
+        "c2_tensordot": lambda: torch.einsum("nachw,ncbhw->nabhw", ins[0], ins[1]),
+        "c3_batch_matmul": lambda: torch.bmm(ins[0], ins[1]),
+        "c4_group_convolution": lambda: torch.nn.functional.conv2d(
+            ins[0].reshape(32, 512, 16, 16), ins[1].reshape(512, 16, 3, 3), ins[2].reshape(512), groups=32),
+        "c5_moments": lambda: (ins[0].mean(1), ins[0].var(1, unbiased=False)),
+    }.get(name)
+    if fn is None:
+        return None
+    fn()
+    times = []
+    t_all = time.perf_counter()
+    while len(times) < 5 and time.perf_counter() - t_all < budget_s:
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    med = sorted(times)[len(times) // 2]
+    return {"value": round(W.algorithmic_bytes(name) / med / 1e9, 3), "unit": "GB/s", "threads": torch.get_num_threads(),
+            "sample": f"ATen CPU routine on the full {name} workload, median of {len(times)} runs, {med * 1e3:.1f} ms each"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -158,6 +186,7 @@ def main():
     if not a.no_cpu:
         line["cpu_baseline"] = cpu_baseline(a.config)
         line["cpu_baseline"]["host_cores"] = os.cpu_count()
+        line["cpu_baseline"]["aten"] = aten_cpu_baseline(a.config)
     if a.all:
         others = {}
         for name in W.CONFIGS:
