@@ -1922,6 +1922,66 @@ void mapKernel(KernelCtx& kc, const DeviceLimits& limits) {
       }
     }
   }
+  // XCD-aware block order.  Consecutive linear block ids go round-robin to the 8 XCDs, each
+  // with its own L2: blocks that differ only in the x-mapped tile index end up on different XCDs.
+  // Operands that do not depend on a block-mapped variable are shared by the blocks along it, so
+  // the variable with the least shared bytes takes blockIdx.x and the one with the most the
+  // slowest axis (its blocks then meet in one L2 when the faster extents are multiples of 8).
+  {
+    const StagePlan& s0 = k.stages.front();
+    std::vector<int> positions;
+    for (int i = 0; i < s0.numParallel && i < k.sharedDepth; ++i) {
+      if (s0.vars[i].blockAxis >= 0) positions.push_back(i);
+    }
+    if (positions.size() >= 2) {
+      std::vector<double> shared(positions.size(), 0.0);
+      for (const auto& st : k.stages) {
+        std::map<std::string, std::set<std::string>> uses; // tensor -> variables in its subscripts
+        for (const auto& stmt : st.stmts) {
+          visit(stmt.rhs, [&](const ExprRef& e) {
+            if (e->kind != Expr::Load) return;
+            auto& u = uses[e->name];
+            for (const auto& a : e->args) {
+              Affine x = ir::toAffine(a);
+              if (!x.valid) {
+                for (const auto& v : st.vars) u.insert(v.name); // unknown: assume it depends on all
+                continue;
+              }
+              for (const auto& c : x.coef) {
+                if (c.second != 0) u.insert(c.first);
+              }
+            }
+          });
+        }
+        for (const auto& t : uses) {
+          const TensorView& view = st.views.at(t.first);
+          double bytes = view.type.bytes();
+          for (auto e : view.extents) bytes *= static_cast<double>(e);
+          for (int pos : positions) {
+            if (t.second.count(st.vars[pos].name)) bytes /= static_cast<double>(st.vars[pos].numTiles);
+          }
+          for (size_t r = 0; r < positions.size(); ++r) {
+            if (!t.second.count(st.vars[positions[r]].name)) shared[r] += bytes;
+          }
+        }
+      }
+      std::vector<size_t> order(positions.size());
+      for (size_t r = 0; r < order.size(); ++r) order[r] = r;
+      std::stable_sort(order.begin(), order.end(), [&](size_t a, size_t b) { return shared[a] < shared[b]; });
+      bool changes = false;
+      for (size_t r = 0; r < order.size(); ++r) changes |= order[r] != r;
+      if (changes && s0.vars[positions[order[0]]].gridExtent % 8 == 0) {
+        gridUse = {{1, 1, 1}};
+        for (auto& st : k.stages) {
+          for (size_t r = 0; r < order.size(); ++r) {
+            LoopVar& v = st.vars[positions[order[r]]];
+            v.blockAxis = static_cast<int>(r);
+            gridUse[r] = std::max(gridUse[r], v.gridExtent);
+          }
+        }
+      }
+    }
+  }
   k.block = blockUse;
   k.grid = gridUse;
   TC_CHECK_LE(k.block[0] * k.block[1] * k.block[2], limits.maxThreadsPerBlock)
