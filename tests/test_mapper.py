@@ -177,3 +177,19 @@ def test_generated_sources_compile_for_gfx950():
         ins = [ShapeOnly(s, "int32" if (src.startswith("def f(int32") and i == 0) else "float32") for i, s in enumerate(shapes)]
         ex = tc.compile(src, entry, ins, opts)
         assert ex.num_kernels >= 1 and "extern \"C\" __global__" in ex.compiled_source
+
+
+def test_block_axis_order_keeps_sharing_blocks_on_one_xcd():
+    """Blocks that share an operand must not differ in blockIdx.x (consecutive ids go to different
+    XCDs): the group convolution's weights depend on g only, so g takes x and n the slower axis; the
+    tensordot's small operand depends on n, which already is the x axis."""
+    src, launches = mapped(W.GROUP_CONVOLUTION, "group_convolution", W.CONFIGS["c4_group_convolution"][2],
+                           W.TUNED["c4_group_convolution"])
+    assert "const int t_g = blockIdx.x;" in src and "const int t_n = blockIdx.y;" in src
+    assert launches[0][0] == (32, 32, 1)
+    src, launches = mapped(W.TENSORDOT, "tensordot", W.CONFIGS["c2_tensordot"][2], W.TUNED["c2_tensordot"])
+    assert "const int t_n = blockIdx.x;" in src and launches[0][0] == (32, 64, 1)
+    # x extent not a multiple of 8: left alone
+    src, _ = mapped(W.GROUP_CONVOLUTION, "group_convolution", [(6, 5, 4, 9, 8), (5, 6, 4, 3, 3), (5, 6)],
+                    "naive;tile=1,1,8,7,6;mapToThreads=64,2;mapToBlocks=6,5")
+    assert "const int t_n = blockIdx.x;" in src
