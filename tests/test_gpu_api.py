@@ -157,3 +157,35 @@ def test_autotune_and_compile_with_cache_round_trip(tmp_path):
     T = tc.define(src, tc.make_load_from_cache_options_factory(cache))
     assert torch.equal(T.add(a, b), a + b)
     assert tc.load_from_cache(src, "add", [a[:8].contiguous(), b[:8].contiguous()], cache) == []   # other sizes
+
+
+@pytest.mark.parametrize("case", ["layernorm", "matmul_3x4x5", "matmul_72x26x72", "matmul_100x400x500"])
+def test_autotune_smoke_cases_of_the_reference(case):
+    """test/cuda/test_autotuner.cc:86-170 with its smoke-check budget (population 8, few generations):
+    the search must return options, and the best ones must compute the right values."""
+    import numpy as np
+    from oracle import tc_oracle
+    layernorm = """def layernorm(float(T, B, C) I) -> (O, mean, centered, var) {
+        mean(t, b) +=! I(t, b, c) / C
+        centered(t, b, c) = I(t, b, c) - mean(t, b)
+        var(t, b) +=! centered(t, b, c) * centered(t, b, c)
+        var(t, b) = var(t, b) / C
+        O(t, b, c) = centered(t, b, c) / rsqrt(var(t, b)) }"""
+    matmul = "def matmul(float(M, N) A, float(N, K) B) -> (output) { output(m, k) +=! A(m, r_n) * B(r_n, k) }"
+    src, entry, shapes, k = {
+        "layernorm": (layernorm, "layernorm", [(7, 32, 64)], 64),
+        "matmul_3x4x5": (matmul, "matmul", [(3, 4), (4, 5)], 4),
+        "matmul_72x26x72": (matmul, "matmul", [(72, 26), (26, 72)], 26),
+        "matmul_100x400x500": (matmul, "matmul", [(100, 400), (400, 500)], 400),
+    }[case]
+    rng = np.random.Generator(np.random.Philox(21))
+    ins_np = [rng.random(s, dtype=np.float32) for s in shapes]
+    ins = [torch.from_numpy(a).cuda() for a in ins_np]
+    best = tc.autotune(src, entry, ins, "naive", generations=2, pop_size=8, threads=8, number_elites=2, seed=5)
+    assert len(best) == 1
+    ex = tc.compile(src, entry, ins, best[0])
+    outs = tc.prepare_outputs(src, entry, ins)
+    tc.run(ex, ins, outs)
+    torch.cuda.synchronize()
+    for o, r in zip(outs, tc_oracle.run(src, entry, ins_np)):
+        assert np.abs(o.cpu().numpy() - r).max() <= 1e-5 * np.sqrt(k) * max(1.0, float(np.abs(r).max()))
