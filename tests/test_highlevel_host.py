@@ -30,3 +30,24 @@ def test_cache_lookup_of_a_missing_file_or_entry_is_empty(tmp_path):
 
 def test_naive_factory_returns_the_naive_preset():
     assert tc.make_naive_options_factory()("", "f").normalized() == tc.MappingOptions("naive").normalized()
+
+
+def test_compile_is_reentrant_across_threads():
+    """The tuner compiles candidates from several threads at once (front end, mapper and hipRTC
+    must be re-entrant): eight threads compiling different TCs and options give the same sources as
+    one thread does."""
+    import concurrent.futures
+    from tests import workloads as W
+    jobs = []
+    for name, (src, entry, shapes, _, _) in W.CONFIGS.items():
+        for options in ("naive", W.TUNED[name]):
+            jobs.append((src, entry, [tc.ShapeOnly(s) for s in shapes], options))
+
+    def build(job):
+        ex = tc.compile(*job)
+        return ex.compiled_source, [ex.launch_bounds(k) for k in range(ex.num_kernels)]
+
+    serial = [build(j) for j in jobs]
+    with concurrent.futures.ThreadPoolExecutor(max_workers=8) as pool:
+        parallel = list(pool.map(build, jobs * 3))
+    assert parallel == serial * 3
