@@ -189,3 +189,30 @@ def test_autotune_smoke_cases_of_the_reference(case):
     torch.cuda.synchronize()
     for o, r in zip(outs, tc_oracle.run(src, entry, ins_np)):
         assert np.abs(o.cpu().numpy() - r).max() <= 1e-5 * np.sqrt(k) * max(1.0, float(np.abs(r).max()))
+
+
+def test_run_can_be_captured_in_a_hip_graph_and_replayed():
+    """run() only enqueues kernel launches on the caller's stream, so a caller may capture it into
+    a HIP graph (launch-bound TCs such as the batched matmul replay without host launch cost).
+    Every replay is checked against an eager run on the same inputs."""
+    src, entry, shapes, _, k = W.CONFIGS["c3_batch_matmul"]
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    ins = [torch.randn(s, device="cuda", generator=gen) for s in shapes]
+    ex = tc.compile(src, entry, ins, W.TUNED["c3_batch_matmul"])
+    outs = tc.prepare_outputs(src, entry, ins)
+    tc.run(ex, ins, outs)                                   # loads the module outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        tc.run(ex, ins, outs)
+    eager = tc.prepare_outputs(src, entry, ins)
+    for replay in range(3):
+        for t in ins:
+            t.copy_(torch.randn(t.shape, device="cuda", generator=gen))
+        outs[0].fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        tc.run(ex, ins, eager)
+        torch.cuda.synchronize()
+        assert torch.equal(outs[0], eager[0]), replay
+        assert (outs[0] - torch.bmm(ins[0], ins[1])).abs().max().item() <= 1e-5 * 72 ** 0.5 * float(outs[0].abs().max())
