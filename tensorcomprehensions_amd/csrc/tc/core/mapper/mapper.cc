@@ -690,15 +690,15 @@ class StageCodegen {
       auto it = hoistedLoads_.find(global);
       if (it != hoistedLoads_.end()) return it->second;
     }
-    if (kc_.opts.useReadOnlyCacheValue && !st_.views.at(e->name).isOutput && streamedOnce(e->name, e->args)) {
-      // streaming read of an input that is never written: keep it out of the way of cached data
-      global = "__builtin_nontemporal_load(&" + global + ")";
-    }
     if (inCachedReduction_) {
       auto it = regCaches.find(global);
       if (it != regCaches.end()) {
         return it->second.name + "[" + cacheSlot_ + "]";
       }
+    }
+    if (kc_.opts.useReadOnlyCacheValue && !st_.views.at(e->name).isOutput && streamedOnce(e->name, e->args)) {
+      // streaming read of an input that is never written: keep it out of the way of cached data
+      global = "__builtin_nontemporal_load(&" + global + ")";
     }
     return global;
   }
@@ -1312,7 +1312,12 @@ class StageCodegen {
         cacheSlot_ = "a_ * " + std::to_string(rcount) + " + " + rlin;
         for (const auto& c : regCaches) {
           if (c.second.producer) {
-            em_.line(c.second.name + "[" + cacheSlot_ + "] = " + c.first + ";");
+            // the only read of the element from memory: streamed when the operand is large
+            std::string tensor = c.first.substr(1, c.first.find('[') - 1);
+            bool stream = kc_.opts.useReadOnlyCacheValue && !st_.views.at(tensor).isOutput &&
+                viewBytes(tensor) >= kStreamingBytes;
+            em_.line(c.second.name + "[" + cacheSlot_ + "] = " +
+                     (stream ? "__builtin_nontemporal_load(&" + c.first + ")" : c.first) + ";");
           }
         }
         inCachedReduction_ = true;
@@ -1970,7 +1975,18 @@ void mapKernel(KernelCtx& kc, const DeviceLimits& limits) {
       std::stable_sort(order.begin(), order.end(), [&](size_t a, size_t b) { return shared[a] < shared[b]; });
       bool changes = false;
       for (size_t r = 0; r < order.size(); ++r) changes |= order[r] != r;
-      if (changes && s0.vars[positions[order[0]]].gridExtent % 8 == 0) {
+      // every stage must distribute the same positions over the same extents
+      bool uniform = true;
+      for (const auto& st : k.stages) {
+        int mapped = 0;
+        for (int i = 0; i < st.numParallel; ++i) mapped += st.vars[i].blockAxis >= 0;
+        uniform &= mapped == static_cast<int>(positions.size());
+        for (int pos : positions) {
+          uniform &= pos < st.numParallel && st.vars[pos].blockAxis == s0.vars[pos].blockAxis &&
+              st.vars[pos].gridExtent == s0.vars[pos].gridExtent;
+        }
+      }
+      if (changes && uniform && s0.vars[positions[order[0]]].gridExtent % 8 == 0) {
         gridUse = {{1, 1, 1}};
         for (auto& st : k.stages) {
           for (size_t r = 0; r < order.size(); ++r) {

@@ -43,7 +43,7 @@ TUNED = {
     "c2_tensordot": "naive;tile=1,8,2,0;mapToThreads=256;mapToBlocks=32,64;unroll=128;vectorWidth=4;useReadOnlyCache=1",
     "c3_batch_matmul": "naive;tile=1,26,26;mapToThreads=64,4;mapToBlocks=500;useMfma=1;useSharedMemory=0",
     "c4_group_convolution": "naive;tile=1,1,16,14,14;mapToThreads=64,4;mapToBlocks=32,32;useMfma=1;useSharedMemory=1;useReadOnlyCache=1",
-    "c5_moments": "naive;tile=1;mapToThreads=512;mapToBlocks=1024;matchLibraryCalls=1;unroll=8;vectorWidth=4;usePrivateMemory=1",
+    "c5_moments": "naive;tile=1;mapToThreads=512;mapToBlocks=1024;matchLibraryCalls=1;unroll=8;vectorWidth=4;usePrivateMemory=1;useReadOnlyCache=1",
 }
 
 
