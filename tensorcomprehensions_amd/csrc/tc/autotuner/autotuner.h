@@ -8,7 +8,9 @@
 // SIGINT finishes the current generation and returns the best so far; SIGTERM aborts.
 #pragma once
 #include <atomic>
+#include <chrono>
 #include <condition_variable>
+#include <cstdlib>
 #include <csignal>
 #include <deque>
 #include <iostream>
@@ -21,6 +23,7 @@
 #include "tc/autotuner/utils.h"
 #include "tc/core/compiler.h"
 #include "tc/core/hip/hip.h"
+#include "tc/core/hip/hip_backend.h"
 #include "tc/core/flags.h"
 #include "tc/lang/parser.h"
 #include "tc/lang/sema.h"
@@ -41,11 +44,31 @@ struct TunerSettings {
   bool verbose = flags().debug_tuner;
   size_t restoreNumber = flags().tuner_gen_restore_number;
   std::string cacheFile; // when set: seeds the first generation from it and appends the result
+  // candidates doing more than this many times the per-thread work of the best one are not run
+  double maxSerialDepthRatio = 256.0;
 };
 
 namespace detail {
 
 extern std::atomic<int> tunerSignal; // 0, SIGINT or SIGTERM while a tune() is running
+
+// Statement instances each launched thread executes one after the other, summed over the
+// kernels of a mapped TC.
+inline double serialDepth(const tc::HipCompilationResult& r) {
+  double depth = 0;
+  for (const auto& k : r.program.kernels) {
+    double points = 0;
+    for (const auto& st : k.stages) {
+      double p = 1;
+      for (const auto& v : st.vars) p *= static_cast<double>(v.extent);
+      points += p * static_cast<double>(std::max<size_t>(1, st.stmts.size()));
+    }
+    double threads = 1;
+    for (int a = 0; a < 3; ++a) threads *= static_cast<double>(k.grid[a] * k.block[a]);
+    depth += points / std::max(1.0, threads);
+  }
+  return depth;
+}
 
 // `extraSizes`: further extents loops of the TC run over.  The reference derives candidates from
 // the input shapes only; the output extents are added here because window-shaped accesses
@@ -181,6 +204,10 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
   } restore{oldInt, oldTerm};
 
   Duration bestTime = Duration::max();
+  double bestDepth = 0; // serial depth of the candidate that holds bestTime
+  // TC_TUNER_TRACE=1: name every candidate before it is compiled and before it is run (finds the
+  // one a stalled tuning run is stuck on)
+  const bool trace = std::getenv("TC_TUNER_TRACE") != nullptr;
   for (size_t gen = 0; gen < settings.generations; ++gen) {
     auto& population = search.population;
     std::atomic<size_t> cursor{0};
@@ -198,6 +225,11 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
         try {
           MappingOptionsType options = baseMapping;
           cand->configuration.applyToHipMappingOptions(options);
+          if (trace) {
+            std::lock_guard<std::mutex> lock(mu);
+            std::cerr << "[tuner] " << std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count()
+                      << " compiling " << options.toText() << std::endl;
+          }
           ex = tc::detail::compile<Backend>(tree, firstInputs, options, quiet);
         } catch (const std::exception& e) {
           if (settings.verbose) std::cerr << "[tuner] candidate failed to compile: " << e.what() << std::endl;
@@ -234,11 +266,25 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
           continue;
         }
         ExecutorType& ex = *job.first;
+        if (trace) {
+          MappingOptionsType options = baseMapping;
+          cand->configuration.applyToHipMappingOptions(options);
+          std::cerr << "[tuner] " << std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count()
+                    << " running " << options.toText() << std::endl;
+        }
         try {
           // prune launches that cannot fill even one compute unit
           auto g = ex.grid().extractDefaultedArray();
           auto b = ex.block().extractDefaultedArray();
           if (g[0] * g[1] * g[2] * b[0] * b[1] * b[2] < settings.minLaunchTotalThreads) {
+            cand->invalid = true;
+            continue;
+          }
+          // A launch cannot be undone, so a degenerate mapping (a handful of threads walking the
+          // whole iteration space) is refused before it is run: statement instances per launched
+          // thread, summed over the kernels, against the same figure of the best candidate so far.
+          double depth = detail::serialDepth(ex.compilationResult());
+          if (bestDepth > 0 && depth > bestDepth * settings.maxSerialDepthRatio) {
             cand->invalid = true;
             continue;
           }
@@ -261,6 +307,7 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
             continue;
           }
           cand->runtime = med;
+          if (med < bestTime) bestDepth = depth;
           bestTime = std::min(bestTime, med, [](Duration a, Duration b) { return a < b; });
           generationTimes.push_back(med);
           MappingOptionsType options = baseMapping;

@@ -2016,7 +2016,9 @@ void mapKernel(KernelCtx& kc, const DeviceLimits& limits) {
     for (int i = st.numParallel - 1; i >= 0; --i) {
       LoopVar& v = st.vars[i];
       if (v.vectorLane || prod * v.perThread <= std::max<int64_t>(budget, 1) || v.perThread == 1) {
-        if (prod * v.perThread > 1024) break;
+        // bound on fully unrolled code: every accumulator of a thread-mapped reduction also
+        // unrolls one block reduction (compile time of hipRTC grows steeply beyond this)
+        if (prod * v.perThread > (st.threadReduction ? 32 : 256)) break;
         v.unrolled = true;
         prod *= v.perThread;
       } else {
