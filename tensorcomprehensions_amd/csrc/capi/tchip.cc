@@ -69,9 +69,18 @@ struct HipApi {
   }
   HipApi() {
     hipLib = openFirst({"libamdhip64.so", "libamdhip64.so.7", "libamdhip64.so.6", "/opt/rocm/lib/libamdhip64.so"});
-    rtcLib = openFirst({"libhiprtc.so", "libhiprtc.so.7", "libhiprtc.so.6", "/opt/rocm/lib/libhiprtc.so"});
+    // hipRTC is a stand-alone compiler (it shares no state with the runtime): TCHIP_HIPRTC names a
+    // specific copy, e.g. a newer ROCm's next to the runtime an older framework build brought along
+    if (const char* forced = std::getenv("TCHIP_HIPRTC")) {
+      rtcLib = dlopen(forced, RTLD_NOW | RTLD_LOCAL);
+      if (!rtcLib) loadError = std::string("cannot load TCHIP_HIPRTC=") + forced + ": " + dlerror();
+    } else {
+      rtcLib = openFirst({"libhiprtc.so", "libhiprtc.so.7", "libhiprtc.so.6", "/opt/rocm/lib/libhiprtc.so"});
+    }
     if (!hipLib) loadError = "cannot load the HIP runtime (libamdhip64.so)";
-    if (!rtcLib) loadError += std::string(loadError.empty() ? "" : "; ") + "cannot load hipRTC (libhiprtc.so)";
+    if (!rtcLib && loadError.find("TCHIP_HIPRTC") == std::string::npos) {
+      loadError += std::string(loadError.empty() ? "" : "; ") + "cannot load hipRTC (libhiprtc.so)";
+    }
     if (hipLib) {
 #define TCHIP_BIND(name) bind(hipLib, #name, name)
       TCHIP_BIND(hipGetDeviceCount);
