@@ -827,7 +827,7 @@ class StageCodegen {
     }
     bool reductionTiled = false;
     for (const auto& r : s.redVars) reductionTiled |= var(r).numTiles > 1;
-    bool inside = reductionTiled && !st_.mfma &&
+    bool inside = reductionTiled &&
         (!kc_.opts.hasSharedDepth || kc_.opts.sharedDepthValue > static_cast<uint32_t>(st_.numParallel));
     // iterations of the statement inside the promoted region
     std::set<std::string> stmtVars;
@@ -1558,7 +1558,9 @@ class StageCodegen {
           // the surplus steps of the last lane group would decode past the outermost extent
           if (i == 0 && quarter * 4 != KT) e = "min(" + e + ", " + std::to_string(v.tile - 1) + ")";
           em_.line("const int p_" + v.name + " = " + e + ";");
-          em_.line("const int " + iv(v) + " = " + std::to_string(v.min) + " + p_" + v.name + ";");
+          std::string base = std::to_string(v.min);
+          if (v.numTiles > 1) base += " + " + tv(v) + " * " + std::to_string(v.tile);
+          em_.line("const int " + iv(v) + " = " + base + " + p_" + v.name + ";");
         }
         if (quarter * 4 != KT) kok = "lj_ * " + std::to_string(quarter) + " + ks_ < " + std::to_string(KT);
       } else {
@@ -1661,49 +1663,56 @@ class StageCodegen {
         }
       }
     }
-    int opened = 0;
-    if (!st_.promotions.empty()) {
-      em_.open("");
-      ++opened;
-      if (suppressCopy) {
+    // Reduction tiling: the outermost reduction variable may run over several tiles; operands
+    // staged per reduction tile are copied inside that loop and the accumulators of all output
+    // tiles of a wavefront live in registers across it.
+    const LoopVar& k0 = var(st_.mfmaK[0]);
+    const bool kTiled = k0.numTiles > 1;
+    const int64_t tilesPerWave = ceilDiv(tiles, st_.waves);
+    auto stagePromotions = [&](bool inside) {
+      bool any = false;
+      for (const auto& p : st_.promotions) any |= p.insideReductionTiles == inside;
+      if (!any) return;
+      if (suppressCopy && !inside) {
         for (const auto& p : st_.promotions) {
+          if (p.insideReductionTiles) continue;
           declareLows(p);
           activePromotions_.insert(p.tensor);
         }
-      } else {
-        em_.line("__syncthreads();");
-        for (const auto& p : st_.promotions) {
-          emitCopyIn(p);
-          activePromotions_.insert(p.tensor);
-        }
-        em_.line("__syncthreads();");
+        return;
       }
-    }
-    // which wavefront takes the surplus tile rotates with the block, so that the blocks sharing a
-    // compute unit load its four SIMDs evenly
-    em_.line("const int wv_ = (threadIdx.y + blockIdx.x + blockIdx.y + blockIdx.z) % " + std::to_string(st_.waves) + ";");
-    em_.open("for (int tl_ = wv_; tl_ < " + std::to_string(tiles) + "; tl_ += " + std::to_string(st_.waves) + ")");
-    ++opened;
-    em_.line("const int nt_ = tl_ % " + std::to_string(numNT) + ", mt_ = (tl_ / " + std::to_string(numNT) + ") % " +
-             std::to_string(numMT) + ", bt_ = tl_ / " + std::to_string(numNT * numMT) + ";");
-    // A row of the product depends on one row of the M-side operand only and a column on one
-    // column of the N-side operand, so lanes past the end of a partial tile may load any legal
-    // element (clamped indices): their results are never stored.
-    std::string bok = st_.mfmaBatch.empty() ? "true" : decodeGroup(st_.mfmaBatch, "bt_", true);
-    em_.line("const bool bok_ = " + bok + ";");
-    em_.line("const int npos_ = nt_ * 16 + lm_;");
-    em_.line("const bool nok_ = bok_ && " + decodeGroup(st_.mfmaN, "npos_", true) + ";");
-    em_.line("__tc::floatx4 c_ = {0.0f, 0.0f, 0.0f, 0.0f};");
-    if (!s.init) {
-      // accumulate into the existing output values
+      em_.line("__syncthreads();");
+      for (const auto& p : st_.promotions) {
+        if (p.insideReductionTiles != inside) continue;
+        emitCopyIn(p);
+        activePromotions_.insert(p.tensor);
+      }
+      em_.line("__syncthreads();");
+    };
+    // decodes the output tile tl_ of this wavefront: batch and column indices, nok_
+    auto decodeTile = [&]() {
+      em_.line("const int nt_ = tl_ % " + std::to_string(numNT) + ", mt_ = (tl_ / " + std::to_string(numNT) + ") % " +
+               std::to_string(numMT) + ", bt_ = tl_ / " + std::to_string(numNT * numMT) + ";");
+      // A row of the product depends on one row of the M-side operand only and a column on one
+      // column of the N-side operand, so lanes past the end of a partial tile may load any legal
+      // element (clamped indices): their results are never stored.
+      std::string bok = st_.mfmaBatch.empty() ? "true" : decodeGroup(st_.mfmaBatch, "bt_", true);
+      em_.line("const bool bok_ = " + bok + ";");
+      em_.line("const int npos_ = nt_ * 16 + lm_;");
+      em_.line("const bool nok_ = bok_ && " + decodeGroup(st_.mfmaN, "npos_", true) + ";");
+      em_.line("(void)nok_;");
+    };
+    // existing output values when the statement accumulates into them
+    auto loadExisting = [&](const std::string& acc) {
       em_.line("#pragma unroll");
       em_.open("for (int r_ = 0; r_ < 4; ++r_)");
       em_.line("const int mpos_ = mt_ * 16 + 4 * lj_ + r_;");
       em_.line("const bool mok_ = " + decodeGroup(st_.mfmaM, "mpos_") + ";");
-      em_.line("if (nok_ && mok_) c_[r_] = p" + st_.tensor + "[" + flatIndex(st_.tensor, st_.lhsSubs, "") + "];");
+      em_.line("if (nok_ && mok_) " + acc + "[r_] = p" + st_.tensor + "[" + flatIndex(st_.tensor, st_.lhsSubs, "") + "];");
       em_.close();
-    }
-    {
+    };
+    // the reduction steps of the current reduction tile into accumulator `acc`
+    auto multiply = [&](const std::string& acc) {
       em_.open("");
       em_.line("const int mposa_ = mt_ * 16 + lm_;");
       em_.line("const bool moka_ = bok_ && " + decodeGroup(st_.mfmaM, "mposa_", true) + ";");
@@ -1711,44 +1720,97 @@ class StageCodegen {
       bool masked = openSteps();
       em_.line("const float a_ = " + (resident ? std::string("am_[ks_]") : operandValue(loadA, masked)) + ";");
       em_.line("const float b_ = " + operandValue(loadB, masked) + ";");
-      em_.line("c_ = __builtin_amdgcn_mfma_f32_16x16x4f32(a_, b_, c_, 0, 0, 0);");
+      em_.line(acc + " = __builtin_amdgcn_mfma_f32_16x16x4f32(a_, b_, " + acc + ", 0, 0, 0);");
       em_.close();
       em_.close();
-    }
+    };
     // Epilogue and store: a lane holds rows 4*lj_ .. 4*lj_+3 of column lm_.  Indices are clamped
     // to legal points, so the epilogue's loads need no guard: the four rows are finished first
     // (their loads issue together and, when they do not depend on the column, move out of the
     // tile loop), then stored under one test of the column.
-    const bool mExact = groupExact(st_.mfmaM, MT, 16);
-    em_.line(accType_.cName() + " out_[4];");
-    em_.line("#pragma unroll");
-    em_.open("for (int r_ = 0; r_ < 4; ++r_)");
-    em_.line("const int mpos_ = mt_ * 16 + 4 * lj_ + r_;");
-    decodeGroup(st_.mfmaM, "mpos_", true);
-    em_.line(accType_.cName() + " acc_[1];");
-    em_.line("acc_[0] = c_[r_];");
-    outerPred_ = "";
-    accValid_ = true;
-    for (size_t i = 1; i < st_.stmts.size(); ++i) {
-      const StageStmt& e = st_.stmts[i];
-      if (e.op != ReduceOp::None) {
-        int n = openUnrolled();
-        em_.line("acc_[a_] = " + combine(e.op, "acc_[a_]", castTo(e.rhs, accType_, "acc_[a_]")) + ";");
-        closeN(n);
-      } else {
-        emitPointwise(e);
+    auto finish = [&](const std::string& acc) {
+      const bool mExact = groupExact(st_.mfmaM, MT, 16);
+      em_.line(accType_.cName() + " out_[4];");
+      em_.line("#pragma unroll");
+      em_.open("for (int r_ = 0; r_ < 4; ++r_)");
+      em_.line("const int mpos_ = mt_ * 16 + 4 * lj_ + r_;");
+      decodeGroup(st_.mfmaM, "mpos_", true);
+      em_.line(accType_.cName() + " acc_[1];");
+      em_.line("acc_[0] = " + acc + "[r_];");
+      outerPred_ = "";
+      accValid_ = true;
+      for (size_t i = 1; i < st_.stmts.size(); ++i) {
+        const StageStmt& e = st_.stmts[i];
+        if (e.op != ReduceOp::None) {
+          int n = openUnrolled();
+          em_.line("acc_[a_] = " + combine(e.op, "acc_[a_]", castTo(e.rhs, accType_, "acc_[a_]")) + ";");
+          closeN(n);
+        } else {
+          emitPointwise(e);
+        }
       }
+      em_.line("out_[r_] = acc_[0];");
+      em_.close();
+      em_.open("if (nok_)");
+      em_.line("#pragma unroll");
+      em_.open("for (int r_ = 0; r_ < 4; ++r_)");
+      em_.line("const int mpos_ = mt_ * 16 + 4 * lj_ + r_;");
+      std::string mok = decodeGroup(st_.mfmaM, "mpos_", true);
+      em_.line(storeStmt(mExact ? "true" : mok, "out_[r_]"));
+      em_.close();
+      em_.close();
+    };
+    // which wavefront takes the surplus tile rotates with the block, so that the blocks sharing a
+    // compute unit load its four SIMDs evenly
+    const std::string waveRotation =
+        "const int wv_ = (threadIdx.y + blockIdx.x + blockIdx.y + blockIdx.z) % " + std::to_string(st_.waves) + ";";
+    int opened = 0;
+    em_.open("");
+    ++opened;
+    stagePromotions(false);
+    if (!kTiled) {
+      em_.line(waveRotation);
+      em_.open("for (int tl_ = wv_; tl_ < " + std::to_string(tiles) + "; tl_ += " + std::to_string(st_.waves) + ")");
+      ++opened;
+      decodeTile();
+      em_.line("__tc::floatx4 c_ = {0.0f, 0.0f, 0.0f, 0.0f};");
+      if (!s.init) loadExisting("c_");
+      multiply("c_");
+      finish("c_");
+    } else {
+      em_.line(waveRotation);
+      em_.line("__tc::floatx4 cacc_[" + std::to_string(tilesPerWave) + "];");
+      em_.line("#pragma unroll");
+      em_.open("for (int j_ = 0; j_ < " + std::to_string(tilesPerWave) + "; ++j_)");
+      em_.line("cacc_[j_] = __tc::floatx4{0.0f, 0.0f, 0.0f, 0.0f};");
+      if (!s.init) {
+        em_.line("const int tl_ = wv_ + j_ * " + std::to_string(st_.waves) + ";");
+        em_.open("if (tl_ < " + std::to_string(tiles) + ")");
+        decodeTile();
+        loadExisting("cacc_[j_]");
+        em_.close();
+      }
+      em_.close();
+      em_.open("for (int " + tv(k0) + " = 0; " + tv(k0) + " < " + std::to_string(k0.numTiles) + "; ++" + tv(k0) + ")");
+      stagePromotions(true);
+      em_.line("#pragma unroll");
+      em_.open("for (int j_ = 0; j_ < " + std::to_string(tilesPerWave) + "; ++j_)");
+      em_.line("const int tl_ = wv_ + j_ * " + std::to_string(st_.waves) + ";");
+      em_.open("if (tl_ < " + std::to_string(tiles) + ")");
+      decodeTile();
+      multiply("cacc_[j_]");
+      em_.close();
+      em_.close();
+      em_.close();
+      em_.line("#pragma unroll");
+      em_.open("for (int j_ = 0; j_ < " + std::to_string(tilesPerWave) + "; ++j_)");
+      ++opened;
+      em_.line("const int tl_ = wv_ + j_ * " + std::to_string(st_.waves) + ";");
+      em_.open("if (tl_ < " + std::to_string(tiles) + ")");
+      ++opened;
+      decodeTile();
+      finish("cacc_[j_]");
     }
-    em_.line("out_[r_] = acc_[0];");
-    em_.close();
-    em_.open("if (nok_)");
-    em_.line("#pragma unroll");
-    em_.open("for (int r_ = 0; r_ < 4; ++r_)");
-    em_.line("const int mpos_ = mt_ * 16 + 4 * lj_ + r_;");
-    std::string mok = decodeGroup(st_.mfmaM, "mpos_", true);
-    em_.line(storeStmt(mExact ? "true" : mok, "out_[r_]"));
-    em_.close();
-    em_.close();
     closeN(opened);
     hoistedLoads_.clear();
     for (const auto& p : st_.promotions) activePromotions_.erase(p.tensor);
@@ -1888,9 +1950,15 @@ void mapKernel(KernelCtx& kc, const DeviceLimits& limits) {
     }
     if (st.mfma) {
       // one wavefront per 16x16 output tile; the block holds as many wavefronts as the block
-      // option has threads; the reduction is consumed whole (no reduction tiling)
+      // option has threads.  Only the outermost reduction variable may be tiled (its tile must
+      // divide the extent): operands are then staged in LDS one reduction tile at a time while the
+      // accumulators of a wavefront's output tiles stay in registers.
+      bool firstReduction = true;
       for (auto& v : st.vars) {
-        if (v.reduction) {
+        if (!v.reduction) continue;
+        bool keep = firstReduction && v.numTiles > 1 && v.extent % v.tile == 0;
+        firstReduction = false;
+        if (!keep) {
           v.tile = v.extent;
           v.numTiles = 1;
         }

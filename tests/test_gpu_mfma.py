@@ -131,3 +131,35 @@ def test_prefetched_lds_staging_on_the_vector_path():
     tc.run(ex, ins, [Z])
     torch.cuda.synchronize()
     assert np.array_equal(Z.cpu().numpy(), np.einsum("bnm,bmk->bnk", X, Y))
+
+
+@pytest.mark.parametrize("opts", [
+    "naive;tile=64,64,32;mapToThreads=64,4;mapToBlocks=256,256;useMfma=1;useSharedMemory=1",
+    "naive;tile=32,48,16;mapToThreads=64,8;mapToBlocks=256,256;useMfma=1;useSharedMemory=1",
+    "naive;tile=64,32,24;mapToThreads=64,2;mapToBlocks=256,256;useMfma=1;useSharedMemory=0",
+    "naive;tile=16,16,7;mapToThreads=64,4;mapToBlocks=256,256;useMfma=1;useSharedMemory=1",   # 7 does not divide 192: untiled
+])
+def test_reduction_tiling_stages_operands_per_tile(opts):
+    """The outermost reduction index may be tiled: operands are staged in LDS once per reduction
+    tile and the accumulators of a wavefront's output tiles stay in registers across the loop."""
+    src = "def mm(float(M, K) A, float(K, N) B) -> (C) { C(m, n) +=! A(m, r_k) * B(r_k, n) }"
+    rng = np.random.Generator(np.random.Philox(41))
+    A = rng.integers(-3, 4, size=(200, 192)).astype(np.float32)
+    B = rng.integers(-3, 4, size=(192, 150)).astype(np.float32)
+    ins = [torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()]
+    ex = tc.compile(src, "mm", ins, opts)
+    (C,) = tc.prepare_outputs(src, "mm", ins)
+    C.fill_(float("nan"))
+    tc.run(ex, ins, [C])
+    torch.cuda.synchronize()
+    assert np.array_equal(C.cpu().numpy(), A @ B)                 # small integers: exact in fp32
+    tiled = "for (int t_r_k" in ex.compiled_source
+    assert tiled == (",7;" not in opts)
+    # accumulate into an existing output across reduction tiles
+    acc = "def mm(float(M, K) A, float(K, N) B) -> (C) { C(m, n) += A(m, r_k) * B(r_k, n) }"
+    ex = tc.compile(acc, "mm", ins, opts)
+    C0 = rng.integers(-5, 6, size=(200, 150)).astype(np.float32)
+    C = torch.from_numpy(C0.copy()).cuda()
+    tc.run(ex, ins, [C])
+    torch.cuda.synchronize()
+    assert np.array_equal(C.cpu().numpy(), C0 + A @ B)
