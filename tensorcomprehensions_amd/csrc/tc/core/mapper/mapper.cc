@@ -808,6 +808,7 @@ class StageCodegen {
   // operand of a wavefront is the same for all of its output tiles, so each lane keeps its
   // elements (one per reduction step) in registers for the whole stage instead of re-reading them.
   static constexpr int64_t kMaxResidentSteps = 64;
+  static constexpr int64_t kMfmaPad = 4;
   bool mfmaKeepsMOperandInRegisters() const {
     if (!st_.mfma) return false;
     int64_t MT = 1, BT = 1, KT = 1;
@@ -901,6 +902,20 @@ class StageCodegen {
       std::vector<int64_t> padded = c.p.extents;
       if (!padded.empty() && padded.back() > 1 && padded.back() % 2 == 0 && lanesWalkOuterDim(ref)) {
         padded.back() += 1;
+      }
+      // Matrix-core operands: the 16 lanes of a group walk the M- (or N-) side variable.  When that
+      // variable is not in the last subscript, consecutive lanes are a whole row apart and a row
+      // length that is a multiple of 8 elements piles them onto few LDS banks: four elements of
+      // padding spread 16 rows over 8 banks groups while rows stay 16-byte aligned for the copies.
+      if (st_.mfma && ref.size() >= 2 && padded.back() % 8 == 0 && kMfmaPad > 0) {
+        bool isA = acc.first == s.rhs->args[st_.mfmaSwapOperands ? 1 : 0]->name;
+        const auto& side = isA ? st_.mfmaM : st_.mfmaN;
+        bool inLast = false, elsewhere = false;
+        for (const auto& n : side) {
+          inLast |= ref.back().coefOf(n) != 0;
+          for (size_t j = 0; j + 1 < ref.size(); ++j) elsewhere |= ref[j].coefOf(n) != 0;
+        }
+        if (elsewhere && !inLast) padded.back() += kMfmaPad;
       }
       c.p.ldsStrides = makeStridesFromSizes(padded);
       c.p.elems = 1;
