@@ -73,6 +73,19 @@ void visit(const ExprRef& e, const std::function<void(const ExprRef&)>& fn) {
   }
 }
 
+// Visits only what every evaluation of `e` evaluates: not the branches of a select and not the
+// right-hand side of a short-circuit operator.  A load found this way may be issued ahead of the
+// expression; one guarded by a condition may address outside its tensor when the guard is false.
+void visitUnconditional(const ExprRef& e, const std::function<void(const ExprRef&)>& fn) {
+  fn(e);
+  size_t n = e->args.size();
+  if (e->kind == Expr::Select) n = 1;
+  if (e->kind == Expr::Binary && (e->name == "&&" || e->name == "||")) n = 1;
+  for (size_t i = 0; i < n; ++i) {
+    visitUnconditional(e->args[i], fn);
+  }
+}
+
 bool sameExpr(const ExprRef& a, const ExprRef& b) {
   if (a->kind != b->kind || a->name != b->name || a->ival != b->ival || a->fval != b->fval ||
       a->args.size() != b->args.size() || a->type != b->type) {
@@ -1393,11 +1406,17 @@ class StageCodegen {
       if (!mine) return "";
       if (v.reduction && v.numTiles != 1) return "";
       if (!v.reduction && !v.unrolled && v.perThread > 1) return "";
+      // the cache holds one tile: a tile loop that each stage runs by itself would reuse the
+      // elements of its last iteration; loops opened around all stages are fine
+      if (!v.reduction && !v.vectorLane && v.numTiles != 1 && static_cast<int>(i) >= kc_.k.sharedDepth &&
+          !(v.blockAxis >= 0 && v.gridExtent == v.numTiles)) {
+        return "";
+      }
       canon[v.name] = "v" + std::to_string(i);
       sig << v.min << "," << v.extent << "," << v.tile << "," << v.numTiles << "," << v.blockAxis << ","
           << v.threadAxis << "," << v.perThread << "," << v.unrolled << "," << v.vectorLane << "," << v.reduction << ";";
     }
-    visit(s->rhs, [&](const ExprRef& e) {
+    visitUnconditional(s->rhs, [&](const ExprRef& e) {
       if (e->kind != Expr::Load) return;
       const TensorView& view = st_.views.at(e->name);
       if (view.isOutput) return;
@@ -1646,7 +1665,7 @@ class StageCodegen {
     if (resident) {
       std::vector<std::pair<std::string, ExprRef>> invariant;
       for (size_t i = 1; i < st_.stmts.size(); ++i) {
-        visit(st_.stmts[i].rhs, [&](const ExprRef& e) {
+        visitUnconditional(st_.stmts[i].rhs, [&](const ExprRef& e) {
           if (e->kind != Expr::Load || e->name == st_.tensor || st_.views.at(e->name).isOutput) return;
           Affine fa = flatAffine(e->name, e->args);
           bool ok = fa.valid;
@@ -1932,6 +1951,19 @@ void mapKernel(KernelCtx& kc, const DeviceLimits& limits) {
     TC_CHECK_GT(o.block[a], 0u) << "NYI: mapping to 0 threads";
   }
   std::array<int64_t, 3> blockUse{{1, 1, 1}}, gridUse{{1, 1, 1}};
+  // Threads the stages may spread over.  A matrix-core stage addresses its lanes as
+  // (threadIdx.x = lane of a wavefront, threadIdx.y = wavefront), so a kernel that holds one runs
+  // 64 x waves threads and its other stages map onto that shape.
+  std::array<int64_t, 3> blk{{static_cast<int64_t>(o.block[0]), static_cast<int64_t>(o.block[1]),
+                              static_cast<int64_t>(o.block[2])}};
+  int nb = static_cast<int>(o.block.size());
+  int64_t waves = std::max<int64_t>(1, std::min<int64_t>(16, blk[0] * blk[1] * blk[2] / 64));
+  for (const auto& st : k.stages) {
+    if (st.mfma) {
+      blk = {{64, waves, 1}};
+      nb = 2;
+    }
+  }
   for (auto& st : k.stages) {
     // tile sizes by band position (lanes do not take a position)
     int pos = 0;
@@ -1978,8 +2010,7 @@ void mapKernel(KernelCtx& kc, const DeviceLimits& limits) {
           v.numTiles = 1;
         }
       }
-      int64_t threads = static_cast<int64_t>(o.block[0] * o.block[1] * o.block[2]);
-      st.waves = std::max<int64_t>(1, std::min<int64_t>(16, threads / 64));
+      st.waves = waves;
       blockUse[0] = std::max<int64_t>(blockUse[0], 64);
       blockUse[1] = std::max<int64_t>(blockUse[1], st.waves);
       continue;
@@ -1987,9 +2018,8 @@ void mapKernel(KernelCtx& kc, const DeviceLimits& limits) {
     // threads: innermost variables, x first
     bool hasReduction = false;
     for (const auto& s : st.stmts) hasReduction |= !s.redVars.empty();
-    st.threadReduction = o.generic.matchLibraryCallsValue && hasReduction && o.block[0] > 1;
+    st.threadReduction = o.generic.matchLibraryCallsValue && hasReduction && blk[0] > 1 && o.block[0] > 1;
     int taxis = 0;
-    int nb = static_cast<int>(o.block.size());
     if (st.threadReduction) {
       for (int i = static_cast<int>(st.vars.size()) - 1; i >= st.numParallel; --i) {
         if (!st.vars[i].vectorLane) {
@@ -2006,7 +2036,7 @@ void mapKernel(KernelCtx& kc, const DeviceLimits& limits) {
     for (auto& v : st.vars) {
       if (v.threadAxis >= 0) {
         blockUse[v.threadAxis] =
-            std::max(blockUse[v.threadAxis], std::min<int64_t>(static_cast<int64_t>(o.block[v.threadAxis]), v.tile));
+            std::max(blockUse[v.threadAxis], std::min<int64_t>(blk[v.threadAxis], v.tile));
       }
     }
   }

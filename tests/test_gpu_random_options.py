@@ -1,5 +1,7 @@
 """Seeded random mapping options (the space the genetic search draws from) on small shapes of the
-four workload families: whatever the tuner can pick must compute the right values, not only the
+four workload families and on multi-statement comprehensions of the reference's benchmark suite
+(chained matmuls with epilogues, batch normalisation, Kronecker products, the WaveNet layer with
+its guarded accesses): whatever the tuner can pick must compute the right values, not only the
 hand-picked presets.  Options the mapper refuses (TcError at compile time) are skipped; the
 number of accepted sets is asserted so that the test cannot pass vacuously."""
 import random
@@ -10,6 +12,7 @@ import torch
 
 import tensorcomprehensions_amd as tc
 from oracle import tc_oracle
+from tests import benchmark_tcs as B
 from tests import workloads as W
 
 pytestmark = pytest.mark.gpu
@@ -20,6 +23,7 @@ SHAPES = {
     "group_convolution": (W.GROUP_CONVOLUTION, "group_convolution", [(2, 3, 4, 10, 9), (3, 6, 4, 3, 3), (3, 6)], 36, 5),
     "moments": (W.MOMENTS, "moments", [(11, 700)], 700, 2),
 }
+SUITE = ["2fcrelu", "batchnorm", "kronecker3", "wavenet1"]
 SIZES = [1, 2, 3, 4, 5, 7, 8, 13, 16, 32, 64, 128]
 
 
@@ -42,11 +46,17 @@ def random_options(rng, band):
     return ";".join(parts)
 
 
-@pytest.mark.parametrize("name", sorted(SHAPES))
+@pytest.mark.parametrize("name", sorted(SHAPES) + SUITE)
 def test_random_option_sets_compute_the_oracle_values(name):
-    src, entry, shapes, k, band = SHAPES[name]
-    data = np.random.Generator(np.random.Philox(31))
-    ins_np = [data.standard_normal(s, dtype=np.float32) for s in shapes]
+    if name in SHAPES:
+        src, entry, shapes, k, band = SHAPES[name]
+        data = np.random.Generator(np.random.Philox(31))
+        ins_np = [data.standard_normal(s, dtype=np.float32) for s in shapes]
+    else:
+        from tests.test_gpu_benchmark_tcs import CHAINED
+        src, entry, _, k = B.CASES[name]
+        k, band = CHAINED.get(name, k), 4
+        ins_np = B.make_inputs(name)
     ref = tc_oracle.run(src, entry, ins_np)
     ins = [torch.from_numpy(a).cuda() for a in ins_np]
     rng = random.Random(sum(map(ord, name)) + 17)
@@ -66,5 +76,7 @@ def test_random_option_sets_compute_the_oracle_values(name):
         torch.cuda.synchronize()
         for o, r in zip(outs, ref):
             err = np.abs(o.cpu().numpy() - r).max()
-            assert err <= W.tolerance(k, r), (name, trial, options, ex.launch_bounds(), err)
+            # chained reductions: intermediate results may be smaller than their operands
+            bound = W.tolerance(k, r) if name in SHAPES else 1e-5 * np.sqrt(k) * max(1.0, float(np.abs(r).max()))
+            assert err <= bound, (name, trial, options, ex.launch_bounds(), err)
     assert accepted >= 30

@@ -193,3 +193,32 @@ def test_block_axis_order_keeps_sharing_blocks_on_one_xcd():
     src, _ = mapped(W.GROUP_CONVOLUTION, "group_convolution", [(6, 5, 4, 9, 8), (5, 6, 4, 3, 3), (5, 6)],
                     "naive;tile=1,1,8,7,6;mapToThreads=64,2;mapToBlocks=6,5")
     assert "const int t_n = blockIdx.x;" in src
+
+
+def wavenet_source(options):
+    from tests import benchmark_tcs as B
+    src, entry, shapes, _ = B.CASES["wavenet1"]
+    return mapped(src, entry, shapes, options)
+
+
+def test_register_cache_holds_only_what_every_stage_loop_shares():
+    """The cache of an operand read by several stages holds one tile: with tile loops that each
+    stage runs by itself (maximal fusion, no block mapping of rf) nothing is cached; with the loops
+    opened around all stages the unconditional read of Data is, and the read that the
+    comprehension guards with `rf - DILATION_FACTOR >= 0` never moves ahead of its guard."""
+    common = "naive;tile=1,16,4;mapToThreads=2,3,3;mapToBlocks=64,3;unroll=8;useSharedMemory=0;usePrivateMemory=1"
+    src, _ = wavenet_source(common + ";outerScheduleFusionStrategy=Max")
+    assert "for (int t_rf = 0; t_rf < 25; ++t_rf)" in src and "rcache" not in src
+    src, _ = wavenet_source(common)
+    assert "rcache0_[a_ * 8 + (0) * 8 + q_r_residual_c] = pData[800 * i_b + 100 * i_r_residual_c + i_rf];" in src
+    assert "rcache1_" not in src
+    assert "? (pData[800 * i_b + 100 * i_r_residual_c + i_rf - 2] *" in src
+
+
+def test_kernel_with_a_matrix_core_stage_runs_whole_wavefronts():
+    """A matrix-core stage reads threadIdx.x as the lane and threadIdx.y as the wavefront: the
+    other stages of its kernel are mapped onto that 64 x waves block instead of widening it."""
+    src, launches = wavenet_source("naive;tile=2;mapToThreads=128;mapToBlocks=16;matchLibraryCalls=1;useMfma=1;"
+                                   "useSharedMemory=0;outerScheduleFusionStrategy=Max")
+    assert launches == [((1, 1, 1), (64, 2, 1))]
+    assert "v_mfma_f32_16x16x4_f32" in src and "blockAllReduceX<__tc::OpSum<float>, 64, 2, 1>" in src
