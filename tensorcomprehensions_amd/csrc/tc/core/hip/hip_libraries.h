@@ -91,6 +91,17 @@ __host__ __device__ constexpr int reduceScratchElems(int bx, int by, int bz) {
   return ((bx & (bx - 1)) == 0 && bx <= 64) ? 1 : (bx % 64 == 0 ? (bx / 64) * by * bz : bx * by * bz);
 }
 
+// Completes the value here: the combine chain of one reduction is finished before the next
+// barrier instead of being deferred, which bounds the values in flight when many reductions are
+// unrolled back to back (hundreds of deferred LDS reads otherwise end up spilled).
+template <typename T> __device__ __forceinline__ void settle(T&) {}
+__device__ __forceinline__ void settle(float& v) { asm volatile("" : "+v"(v)); }
+__device__ __forceinline__ void settle(double& v) { asm volatile("" : "+v"(v)); }
+__device__ __forceinline__ void settle(int& v) { asm volatile("" : "+v"(v)); }
+__device__ __forceinline__ void settle(unsigned& v) { asm volatile("" : "+v"(v)); }
+__device__ __forceinline__ void settle(long long& v) { asm volatile("" : "+v"(v)); }
+__device__ __forceinline__ void settle(unsigned long long& v) { asm volatile("" : "+v"(v)); }
+
 template <typename Op, int BX, int BY, int BZ, typename T>
 __device__ __forceinline__ T blockAllReduceX(T v, T* scratch) {
   if (BX == 1) {
@@ -112,6 +123,7 @@ __device__ __forceinline__ T blockAllReduceX(T v, T* scratch) {
     T r = scratch[row * W];
 #pragma unroll
     for (int w = 1; w < W; ++w) r = Op::apply(r, scratch[row * W + w]);
+    settle(r);
     return r;
   }
   // any other row width: rows straddle wavefronts, go through LDS
@@ -119,7 +131,9 @@ __device__ __forceinline__ T blockAllReduceX(T v, T* scratch) {
   scratch[row * BX + threadIdx.x] = v;
   __syncthreads();
   T r = scratch[row * BX];
+#pragma unroll 8
   for (int x = 1; x < BX; ++x) r = Op::apply(r, scratch[row * BX + x]);
+  settle(r);
   return r;
 }
 } // namespace __tc

@@ -2035,8 +2035,18 @@ void mapKernel(KernelCtx& kc, const DeviceLimits& limits) {
     }
     for (auto& v : st.vars) {
       if (v.threadAxis >= 0) {
-        blockUse[v.threadAxis] =
-            std::max(blockUse[v.threadAxis], std::min<int64_t>(blk[v.threadAxis], v.tile));
+        int64_t want = v.tile;
+        if (st.threadReduction && v.reduction) {
+          // the reduction library is fastest on rows that are lane groups of a wavefront or
+          // whole wavefronts: tighten to the next such width when the option allows it
+          if (want <= 64) {
+            while (want & (want - 1)) ++want;
+          } else {
+            want = ceilDiv(want, 64) * 64;
+          }
+          if (want > blk[v.threadAxis]) want = v.tile;
+        }
+        blockUse[v.threadAxis] = std::max(blockUse[v.threadAxis], std::min<int64_t>(blk[v.threadAxis], want));
       }
     }
   }

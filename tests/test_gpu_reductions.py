@@ -114,3 +114,21 @@ def test_point_wise_chain_needs_no_barrier():
     A = np.random.Generator(np.random.Philox(77)).standard_normal((70, 130), dtype=np.float32)
     ex = check(chain, "f", [A], "naive", 1)
     assert "__syncthreads" not in ex.compiled_source and ex.num_kernels == 1
+
+
+@pytest.mark.parametrize("threads,block", [("512,2", (64, 2, 1)), ("33,2", (33, 2, 1)), ("40,2", (33, 2, 1))])
+def test_many_unrolled_reductions_on_odd_rows(threads, block):
+    """17 block reductions unrolled back to back on rows of 33 threads: with one-hot columns every
+    row sum is exactly 1, so a partial that goes missing or counts twice shows by position.  A row
+    width the option leaves room for is widened to whole lane groups (33 -> 64)."""
+    src = "def f(float(N, N) A) -> (O) { O(i) +=! fmax(A(i, j), 0) }"
+    A = torch.zeros(33, 33, device="cuda")
+    ex = tc.compile(src, "f", [A], f"naive;tile=64,0,2;mapToThreads={threads};mapToBlocks=64;unroll=128;matchLibraryCalls=1")
+    assert ex.launch_bounds() == ((1, 1, 1), block)
+    (out,) = tc.prepare_outputs(src, "f", [A])
+    for c in range(33):
+        A.zero_()
+        A[:, c] = 1
+        out.fill_(float("nan"))
+        tc.run(ex, [A], [out])
+        assert torch.all(out == 1.0), (c, out.cpu().numpy())
