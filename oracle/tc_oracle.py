@@ -415,6 +415,15 @@ class Analysis:
         for o in self.outputs:
             if o not in self.tensors:
                 raise TcError(f"undefined variable {o} used here.")
+        # a tensor has one bound, that of its last definition, applied to all its stages
+        # (tc2halide.cc:676-693, :808-870): an earlier statement inferred over a larger range
+        # writes only inside it
+        for s in d.stmts:
+            t = self.tensors[s.lhs]
+            for dim, v in enumerate(s.indices):
+                lo, hi = s.ranges[v]
+                lo, hi = max(lo, t.mins[dim]), min(hi, t.mins[dim] + t.extents[dim] - 1)
+                s.ranges[v] = (lo, hi)
 
     # -- typing ---------------------------------------------------------------------------
     def _type(self, e: Expr, s: Stmt, index_env: Dict[str, None], lets: Dict[str, Expr], allow_access=True) -> Expr:

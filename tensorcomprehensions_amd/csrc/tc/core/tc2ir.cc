@@ -575,6 +575,20 @@ ir::Function translate(
       throw lang::errorAt(checked) << "output " << o.name << " is never written";
     }
   }
+  // A tensor has one bound, that of its last definition, applied to all its stages
+  // (tc2halide.cc:676-693, :808-870): an earlier statement inferred over a larger range writes
+  // only inside it.
+  for (auto& s : f.statements) {
+    const ir::Tensor* out = nullptr;
+    for (const auto& t : f.outputs) {
+      if (t.name == s.tensor) out = &t;
+    }
+    for (size_t d = 0; d < s.lhsVars.size() && d < out->extents.size(); ++d) {
+      ir::Range& r = s.ranges[s.lhsVars[d]];
+      r.min = std::max(r.min, out->mins[d]);
+      r.max = std::min(r.max, out->mins[d] + out->extents[d] - 1);
+    }
+  }
   return f;
 }
 

@@ -127,3 +127,24 @@ def test_integer_modulo():                                                      
     (r,) = run("def f(int32 a, int32 b) -> (c) { c(i) = int32(a % b) where i in 0:1 }",
                torch.tensor(17, dtype=torch.int32), torch.tensor(5, dtype=torch.int32))
     assert r.dtype == torch.int32 and r.item() == 17 % 5
+
+
+SHRINKING = """def f(float(K, P, M, P) A) -> (O) {
+    O(i) = float(i + 3) where i in 0:16
+    O(i) min= A(i, j, i, i)
+}"""
+
+
+def test_a_tensor_takes_the_bounds_of_its_last_definition_in_every_statement():
+    """tc2halide.cc:676-693 clobbers a tensor's bounds with those of its last definition and applies
+    them to all its stages: `O` is inferred as 16 elements by the first statement and as one by the
+    second (`i` also indexes a dimension of size 1), so it has one element and the first statement
+    writes one element, not sixteen."""
+    from oracle import tc_oracle
+    assert [s for _, s, _ in tc.infer_output_tensor_info(SHRINKING, "f", [F(16, 70, 1, 70)])] == [(1,)]
+    assert tc_oracle.infer_output_shapes(SHRINKING, "f", [(16, 70, 1, 70)]) == [("O", "float", [1])]
+    src, launches = tc.map_only(SHRINKING, "f", [F(16, 70, 1, 70)], "naive;outerScheduleFusionStrategy=Min")
+    assert all(block == (1, 1, 1) for _, block in launches)
+    A = np.full((16, 70, 1, 70), 7.0, np.float32)
+    (o,) = tc_oracle.run(SHRINKING, "f", [A])
+    assert o.tolist() == [3.0]
