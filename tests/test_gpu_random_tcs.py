@@ -1,0 +1,40 @@
+"""Random comprehensions under random mapping options against the oracle: multi-statement
+definitions with shared and intersecting index ranges, windows, selects, `where` ranges, explicit
+initialisations and reductions, in float and double.  Bound: 2e-4 * scale, scale being the largest
+magnitude among the results (every intermediate is an output here).  That is tighter than the
+acceptance rule's 1e-5 * sqrt(K) * scale at the generator's largest reduction length (K = 2e5 gives
+4.5e-3) and small enough that one partial dropped from a 33-term sum shows."""
+import random
+
+import numpy as np
+import pytest
+import torch
+
+import tensorcomprehensions_amd as tc
+from tests import random_tcs
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("seed", [201, 202, 203])
+def test_random_definitions_match_the_oracle(seed):
+    rng = random.Random(seed)
+    runs = 0
+    for src, entry, ins_np, ref in random_tcs.cases(seed=seed, count=50):
+        ins = [torch.from_numpy(a).cuda() for a in ins_np]
+        scale = max(1.0, max(float(np.abs(r).max()) for r in ref if r.size))
+        for options in ("naive", random_tcs.random_options(rng), random_tcs.random_options(rng)):
+            print(src, options, flush=True)
+            ex = tc.compile(src, entry, ins, options)
+            outs = tc.prepare_outputs(src, entry, ins)
+            for o in outs:
+                o.fill_(float("nan"))
+            tc.run(ex, ins, outs)
+            torch.cuda.synchronize()
+            for o, r in zip(outs, ref):
+                got = o.cpu().numpy()
+                assert got.dtype == r.dtype and got.shape == r.shape
+                err = np.abs(got.astype(np.float64) - r).max() if r.size else 0.0
+                assert err <= 2e-4 * scale, (src, options, ex.launch_bounds(), err)
+            runs += 1
+    assert runs == 150
