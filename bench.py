@@ -4,7 +4,8 @@
 One "step" = one launch of the compiled TC over one batch of synthetic, seeded inputs that are
 already resident in HBM.  The headline workload is the HBM-bound tensordot
 O(n,c1,c3,h,w) +=! I0(n,c1,r_c2,h,w) * I1(n,r_c2,c3,h,w) at N=32, C1=512, C2=8, C3=2, H=W=28;
-`--config` selects another of the five workloads, `--all` appends their figures under "others".
+`--config` selects another of the five workloads, `--all` appends their figures under "others",
+`--suite` appends the reference's other benchmark programs at their default sizes under "suite".
 Prints ONE JSON line.
 """
 import argparse
@@ -151,6 +152,63 @@ def aten_cpu_baseline(name, budget_s=10.0):
             "sample": f"ATen CPU routine on the full {name} workload, median of {len(times)} runs, {med * 1e3:.1f} ms each"}
 
 
+def suite_library_routines():
+    """What the reference's benchmark programs time next to each TC: the ATen routine(s), here on
+    the same GPU through PyTorch (eager, one launch per operator)."""
+    import torch
+    import torch.nn.functional as F
+    return {
+        "tmm": lambda a, b: a @ b.t(),
+        "matmul": lambda a, b: a @ b,
+        "convolution": lambda i, w, b: F.conv2d(i, w, b),
+        "2fcrelu": lambda i, w1, b1, w2, b2: F.relu(F.linear(F.relu(F.linear(i, w1, b1)), w2, b2)),
+        "lut": lambda t, i: t[i.long()].sum(1),
+        "moments2": lambda x: (x.mean(1), x.var(1, unbiased=False)),
+        "group_normalization_single_kernel": lambda i, g, b: F.group_norm(
+            i.reshape(i.shape[0], -1, i.shape[3], i.shape[4]), i.shape[1], g.reshape(-1), b.reshape(-1), 1e-5),
+        "kronecker3": lambda w0, w1, w2, x: torch.einsum("mabc,ia,jb,kc->mijk", x, w0, w1, w2),
+    }
+
+
+def measure_suite(steps, warmup):
+    """Kernel time of every comprehension of tests/benchmark_tcs.py:REFERENCE_SIZES under its tuned
+    options (sum over its kernels, HIP events around `steps` back-to-back runs), the bytes of all
+    its inputs and outputs counted once (look-up tables: the gathered rows), and the library time."""
+    import torch
+    import tensorcomprehensions_amd as tc
+    from tests import benchmark_tcs as B
+    routines = suite_library_routines()
+    out = {}
+    for name, options in B.TUNED_AT_REFERENCE_SIZES.items():
+        src, entry, _, _ = B.CASES[name]
+        ins = [torch.from_numpy(a).cuda() for a in B.make_inputs(name, reference_sizes=True)]
+        ex = tc.compile(src, entry, ins, options)
+        outs = tc.prepare_outputs(src, entry, ins)
+        for _ in range(warmup):
+            tc.unchecked_run(ex, ins, outs)
+        us = tc.profile_repeated(ex, ins, outs, steps) / steps
+        nbytes = sum(t.numel() * t.element_size() for t in ins + outs)
+        if name == "lut":
+            nbytes += (ins[1].numel() * ins[0].shape[1] - ins[0].numel()) * 4
+        entry_out = {"kernel_us": round(us, 2), "kernels": ex.num_kernels, "bytes": nbytes,
+                     "gb_per_s": round(nbytes / us / 1e3, 1),
+                     "launch": [ex.launch_bounds(k) for k in range(ex.num_kernels)]}
+        fn = routines.get(name)
+        if fn is not None:
+            for _ in range(warmup):
+                fn(*ins)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(steps):
+                fn(*ins)
+            e1.record()
+            torch.cuda.synchronize()
+            entry_out["library_us"] = round(e0.elapsed_time(e1) * 1e3 / steps, 2)
+        out[name] = entry_out
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -159,6 +217,8 @@ def main():
     ap.add_argument("--config", default="c2_tensordot")
     ap.add_argument("--options", default=None)
     ap.add_argument("--all", action="store_true")
+    ap.add_argument("--suite", action="store_true",
+                    help="also time the reference's other benchmark comprehensions at their default sizes")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain copy kernel of known size (reference point for HBM byte counters)")
@@ -196,6 +256,8 @@ def main():
             others[name] = {"kernel_us": round(o["kernel_ms"] * 1e3, 3), "roofline": roofline(o),
                             "gflops": round(o["flops"] / (o["kernel_ms"] * 1e-3) / 1e9, 1), "launch": o["launch"]}
         line["others"] = others
+    if a.suite:
+        line["suite"] = measure_suite(a.steps, a.warmup)
     print(json.dumps(line))
 
 

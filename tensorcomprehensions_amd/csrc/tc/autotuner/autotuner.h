@@ -207,7 +207,8 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
   double bestDepth = 0; // serial depth of the candidate that holds bestTime
   // TC_TUNER_TRACE=1: name every candidate before it is compiled and before it is run (finds the
   // one a stalled tuning run is stuck on)
-  const bool trace = std::getenv("TC_TUNER_TRACE") != nullptr;
+  const char* traceEnv = std::getenv("TC_TUNER_TRACE");
+  const bool trace = traceEnv != nullptr && traceEnv[0] != '\0' && traceEnv[0] != '0';
   for (size_t gen = 0; gen < settings.generations; ++gen) {
     auto& population = search.population;
     std::atomic<size_t> cursor{0};

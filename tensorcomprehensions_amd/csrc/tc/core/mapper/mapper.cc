@@ -338,12 +338,22 @@ struct StageBuilder {
     return a.valid && a.constant == 0 && a.coef.size() == 1 && a.coefOf(v) == 1;
   }
 
-  // Merge adjacent parallel variables a,b when every access that mentions them has `a` alone in
-  // some dimension j and `b` alone in dimension j+1 spanning that whole dimension: the pair then
-  // walks memory exactly like one variable of extent |a|*|b| over the merged dimension.
+  // Merge adjacent variables a,b (two parallel ones, or two consecutive reduction variables of
+  // one statement) when every access that mentions them has `a` alone in some dimension j and `b`
+  // alone in dimension j+1 spanning that whole dimension: the pair then walks memory exactly
+  // like one variable of extent |a|*|b| over the merged dimension, in the same order.
   bool tryCollapse(size_t k) {
     LoopVar &a = st.vars[k], &b = st.vars[k + 1];
-    if (a.min != 0 || b.min != 0) return false;
+    if (a.min != 0 || b.min != 0 || a.reduction != b.reduction) return false;
+    StageStmt* owner = nullptr;
+    if (a.reduction) {
+      for (auto& s : st.stmts) {
+        for (size_t i = 0; i + 1 < s.redVars.size(); ++i) {
+          if (s.redVars[i] == a.name && s.redVars[i + 1] == b.name) owner = &s;
+        }
+      }
+      if (!owner) return false;
+    }
     auto loose = looseVars();
     if (loose.count(a.name) || loose.count(b.name)) return false;
     std::map<std::string, std::set<size_t>> mergeAt; // tensor -> dims j to merge with j+1
@@ -401,15 +411,22 @@ struct StageBuilder {
       ext[j] *= ext[j + 1];
       ext.erase(ext.begin() + j + 1);
     }
+    if (owner) {
+      auto it = std::find(owner->redVars.begin(), owner->redVars.end(), a.name);
+      *it = merged;
+      owner->redVars.erase(it + 1);
+    } else {
+      st.numParallel -= 1;
+    }
     a.name = merged;
     a.extent *= eb;
     st.vars.erase(st.vars.begin() + k + 1);
-    st.numParallel -= 1;
     return true;
   }
 
-  void collapse() {
-    for (size_t k = 0; k + 1 < static_cast<size_t>(st.numParallel);) {
+  // Variables before `first` are shared with the other stages of the kernel and keep their shape.
+  void collapse(size_t first = 0) {
+    for (size_t k = first; k + 1 < st.vars.size();) {
       if (!tryCollapse(k)) ++k;
     }
   }
@@ -2449,7 +2466,7 @@ MappedProgram mapToHip(
     for (size_t si : groups[gi].stages) {
       StageBuilder b(f);
       b.init(raw[si]);
-      if (single && options.collapseContiguousValue) b.collapse();
+      if (options.collapseContiguousValue) b.collapse(single ? 0 : static_cast<size_t>(groups[gi].depth));
       k.stages.push_back(std::move(b.st));
     }
     k.sharedDepth = single ? k.stages[0].numParallel : groups[gi].depth;

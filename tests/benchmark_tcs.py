@@ -164,11 +164,53 @@ CASES = {
 }
 
 
-def make_inputs(name, seed=2024):
+# The same comprehensions at the default sizes of the reference's benchmark programs
+# (tc/benchmarks/tmm.cc:42-44, MLP_model.cc:43-59 for the 1000x1024 matmul, the fc-relu chain and
+# the look-up table, convolution.cc:40-46, moments.cc:42-43, group_normalization.cc:42-46,
+# kronecker.cc:41-47, wavenet.cc:42-60), and the mapping options the autotuner found for them on an
+# MI355X (a few generations from the naive options; written relative to the naive options).
+REFERENCE_SIZES = {
+    "tmm": [(32, 256), (128, 256)],
+    "matmul": [(128, 1000), (1000, 1024)],
+    "convolution": [(32, 4, 56, 56), (4, 4, 3, 3), (4,)],
+    "2fcrelu": [(128, 2000), (128, 2000), (128,), (64, 128), (64,)],
+    "lut": [(100000, 64), ("int", (128, 50), 0, 100000)],
+    "moments2": [(1024, 36864)],
+    "group_normalization_single_kernel": [(32, 32, 16, 48, 48), (32, 16), (32, 16)],
+    "kronecker3": [(32, 16), (32, 16), (32, 16), (256, 16, 16, 16)],
+    "wavenet1": [(1, 32, 4000), (32, 32, 2), (32,), (32, 32, 2), (32,), (32, 32), (32,), (32, 32), (32,), (1,)],
+}
+TUNED_AT_REFERENCE_SIZES = {
+    "tmm": "naive;tile=64,2;unroll=2;matchLibraryCalls=1;mapToThreads=128,1;mapToBlocks=256,1;usePrivateMemory=1;"
+           "unrollCopyShared=1;useReadOnlyCache=1;vectorWidth=2;collapseContiguous=0;useMfma=1;prefetchShared=1",
+    "matmul": "naive;intraTileScheduleFusionStrategy=Max;tile=16,32;unroll=256;matchLibraryCalls=1;mapToThreads=512,2;"
+              "mapToBlocks=125,1000;unrollCopyShared=1;useReadOnlyCache=1;useMfma=1;prefetchShared=1",
+    "convolution": "naive;intraTileScheduleFusionStrategy=Min;fixParametersBeforeScheduling=1;tile=2,27,1,56;unroll=256;"
+                   "tileImperfectlyNested=1;mapToThreads=128,7;mapToBlocks=256,64;useSharedMemory=1;useReadOnlyCache=1;"
+                   "collapseContiguous=0",
+    "2fcrelu": "naive;outerScheduleFusionStrategy=Max;intraTileScheduleFusionStrategy=Max;fixParametersBeforeScheduling=1;"
+               "tile=4;unroll=32;mapToThreads=8,128;mapToBlocks=1024;useSharedMemory=1;unrollCopyShared=1;useReadOnlyCache=1;"
+               "vectorWidth=4;useMfma=1",
+    "lut": "naive;outerScheduleFusionStrategy=Min;tile=4,32,32;unroll=64;usePrivateMemory=1;unrollCopyShared=1;"
+           "collapseContiguous=0",
+    "moments2": "naive;outerScheduleFusionStrategy=Max;fixParametersBeforeScheduling=1;tile=1;unroll=64;tileImperfectlyNested=1;"
+                "matchLibraryCalls=1;mapToThreads=1024;mapToBlocks=1152;usePrivateMemory=1;unrollCopyShared=1;"
+                "useReadOnlyCache=1;vectorWidth=2;collapseContiguous=0;useMfma=1",
+    "group_normalization_single_kernel": "naive;outerScheduleFusionStrategy=Max;intraTileScheduleFusionStrategy=Min;tile=1,1;"
+                                         "unroll=64;matchLibraryCalls=1;mapToThreads=1024;mapToBlocks=32,8;usePrivateMemory=1;"
+                                         "vectorWidth=4;prefetchShared=1",
+    "kronecker3": "naive;outerScheduleFusionStrategy=Min;tile=1,32,0,128;unroll=8;tileImperfectlyNested=1;mapToThreads=128,8;"
+                  "mapToBlocks=256;unrollCopyShared=1;collapseContiguous=0;useMfma=1",
+    "wavenet1": "naive;intraTileScheduleFusionStrategy=Max;fixParametersBeforeScheduling=1;tile=2,8,16;unroll=64;"
+                "mapToThreads=32,4;mapToBlocks=2000,256;usePrivateMemory=1;collapseContiguous=0",
+}
+
+
+def make_inputs(name, seed=2024, reference_sizes=False):
     import numpy as np
     rng = np.random.Generator(np.random.Philox(seed))
     out = []
-    for spec in CASES[name][2]:
+    for spec in (REFERENCE_SIZES if reference_sizes else {name: CASES[name][2]})[name]:
         if isinstance(spec[0], str):
             kind = spec[0]
             if kind == "int":

@@ -40,6 +40,29 @@ def test_parity_with_oracle(name, options):
         assert np.abs(got - r).max() <= 1e-5 * np.sqrt(k) * scale, (name, options, ex.launch_bounds())
 
 
+@pytest.mark.parametrize("name", sorted(B.TUNED_AT_REFERENCE_SIZES))
+def test_parity_at_the_reference_sizes_with_the_tuned_options(name):
+    src, entry, _, k = B.CASES[name]
+    print(f"case {name} at the reference's default size", flush=True)
+    ins_np = B.make_inputs(name, reference_sizes=True)
+    ref = tc_oracle.run(src, entry, ins_np)
+    ins = [torch.from_numpy(a).cuda() for a in ins_np]
+    ex = tc.compile(src, entry, ins, B.TUNED_AT_REFERENCE_SIZES[name])
+    outs = tc.prepare_outputs(src, entry, ins)
+    for o in outs:
+        o.fill_(float("nan"))
+    tc.run(ex, ins, outs)
+    torch.cuda.synchronize()
+    # reduction lengths at these sizes (chains: the product of the lengths)
+    k = {"tmm": 256, "matmul": 1000, "convolution": 36, "2fcrelu": 2000 * 128, "lut": 50, "moments2": 36864,
+         "group_normalization_single_kernel": 36864, "kronecker3": 16 ** 3, "wavenet1": 32 * 64}[name]
+    for o, r in zip(outs, ref):
+        got = o.cpu().numpy()
+        assert got.shape == r.shape
+        scale = max(1.0, float(np.abs(r).max()))
+        assert np.abs(got - r).max() <= 1e-5 * np.sqrt(k) * scale, (name, ex.launch_bounds())
+
+
 def test_lookup_indices_are_exact():
     """Indirect indexing with integer-valued tables: sums are exact, any wrong row shows."""
     rng = np.random.Generator(np.random.Philox(5))
