@@ -1243,7 +1243,10 @@ class StageCodegen {
   // --- statements -----------------------------------------------------------------------------
   void emitPointwise(const StageStmt& s) {
     int n = openUnrolled();
+    inCachedReduction_ = cachedPointwise_;
+    cacheSlot_ = "a_";
     em_.line("acc_[a_] = " + castTo(s.rhs, accType_, accValid_ ? "acc_[a_]" : "") + ";");
+    inCachedReduction_ = false;
     closeN(n);
   }
 
@@ -1462,6 +1465,77 @@ class StageCodegen {
     for (const auto& r : s->redVars) n *= var(r).perThread;
     return n;
   }
+
+  // A load's flat element offset as a function of what tells threads and iterations apart: block
+  // ids / kernel-level tile loops, thread ids, and the fully unrolled per-thread loop counters
+  // named by their stride in the register-cache slot.  Two stages whose forms of an operand agree
+  // make every thread touch the same element at the same slot, whatever their loop structure
+  // (a reduction over one merged variable and a pointwise stage over (d, h*w), say).  Invalid
+  // when a variable involved is clamped, folded, tiled inside the stage or loops without being
+  // unrolled: the slot would then not name one element.
+  struct AddressForm {
+    bool valid = false;
+    std::string tensor;
+    int64_t constant = 0;
+    int64_t slots = 1;
+    std::map<std::string, int64_t> coef;
+    bool operator==(const AddressForm& o) const {
+      return valid && o.valid && tensor == o.tensor && constant == o.constant && slots == o.slots && coef == o.coef;
+    }
+  };
+  AddressForm addressForm(const ExprRef& load, const StageStmt* reduction) const {
+    AddressForm form;
+    const TensorView& view = st_.views.at(load->name);
+    if (view.isOutput) return form;
+    Affine flat = flatAffine(load->name, load->args);
+    if (!flat.valid) return form;
+    // slot layout: unrolled parallel variables, then the statement's reduction variables
+    std::vector<const LoopVar*> slotVars;
+    for (int i = 0; i < st_.numParallel; ++i) {
+      const LoopVar& v = st_.vars[i];
+      if (v.perThread > 1 && !v.unrolled) return form;
+      if (v.perThread > 1) slotVars.push_back(&v);
+    }
+    if (reduction) {
+      for (const auto& r : reduction->redVars) {
+        if (var(r).perThread > 1) slotVars.push_back(&var(r));
+      }
+    }
+    std::map<std::string, int64_t> stride;
+    for (size_t i = slotVars.size(); i-- > 0;) {
+      stride[slotVars[i]->name] = form.slots;
+      form.slots *= slotVars[i]->perThread;
+    }
+    for (const auto* sv : slotVars) {
+      if (flat.coefOf(sv->name) == 0) return form; // a slot that does not move the address
+    }
+    form.tensor = load->name;
+    form.constant = flat.constant;
+    for (size_t i = 0; i < st_.vars.size(); ++i) {
+      const LoopVar& v = st_.vars[i];
+      int64_t c = flat.coefOf(v.name);
+      if (c == 0) continue;
+      bool mine = !v.reduction ||
+          (reduction && std::find(reduction->redVars.begin(), reduction->redVars.end(), v.name) != reduction->redVars.end());
+      if (!mine || v.partial()) return form;
+      if (v.threadAxis >= 0 && v.perThread * kc_.k.block[v.threadAxis] != v.tile) return form;
+      form.constant += c * v.min;
+      if (v.numTiles > 1) {
+        if (v.reduction || static_cast<int>(i) >= kc_.k.sharedDepth) return form;
+        bool blockId = v.blockAxis >= 0 && v.gridExtent == v.numTiles;
+        form.coef[blockId ? std::string("block.") + axisName(v.blockAxis) : "t_" + v.name] += c * v.tile;
+      }
+      if (v.threadAxis >= 0) form.coef[std::string("thread.") + axisName(v.threadAxis)] += c;
+      if (v.perThread > 1) {
+        form.coef["q." + std::to_string(stride.at(v.name))] += c * (v.threadAxis >= 0 ? kc_.k.block[v.threadAxis] : 1);
+      }
+    }
+    form.valid = true;
+    return form;
+  }
+
+  // Pointwise statements of this stage read the operands in `regCaches` from the register cache.
+  bool cachedPointwise_ = false;
 
   // True when this stage touches `producer`'s result only at the element the same thread wrote:
   // both stages spread identical parallel variables over blocks and threads in the same way and
@@ -2244,6 +2318,50 @@ void emitKernel(KernelCtx& kc, const DeviceLimits& limits, Emitter& em) {
         }
         gens[i].regCaches[l.second] = StageCodegen::RegCache{it->second, producer};
         gens[i].cachedStmt_ = gens[i].firstReduction();
+      }
+    }
+  }
+
+  // The same for a pointwise stage after a reduction over the same elements (normalise after
+  // moments, say): when an operand's address forms agree, the reduction's single read of each
+  // element fills the cache and the pointwise stage finds it there.
+  if (kc.opts.usePrivateMemoryValue && gens.size() >= 2) {
+    for (size_t j = 1; j < gens.size(); ++j) {
+      const StagePlan& cs = k.stages[j];
+      bool pointwise = !cs.mfma && !cs.threadReduction && gens[j].firstReduction() == nullptr;
+      if (!pointwise) continue;
+      for (const auto& stmt : cs.stmts) {
+        if (stmt.op != ReduceOp::None) continue;
+        visitUnconditional(stmt.rhs, [&](const ExprRef& e) {
+          if (e->kind != Expr::Load) return;
+          StageCodegen::AddressForm want = gens[j].addressForm(e, nullptr);
+          if (!want.valid || want.slots > 256) return;
+          std::string mine = "p" + e->name + "[" + gens[j].flatIndex(e->name, e->args, "") + "]";
+          if (gens[j].regCaches.count(mine)) return;
+          for (size_t i = 0; i < j; ++i) {
+            const StageStmt* red = gens[i].firstReduction();
+            if (!red || k.stages[i].mfma) continue;
+            if (gens[i].cachedStmt_ && gens[i].cachedStmt_ != red) continue;
+            std::string found;
+            visitUnconditional(red->rhs, [&](const ExprRef& m) {
+              if (m->kind != Expr::Load || !found.empty()) return;
+              if (gens[i].addressForm(m, red) == want) {
+                found = "p" + m->name + "[" + gens[i].flatIndex(m->name, m->args, "") + "]";
+              }
+            });
+            if (found.empty()) continue;
+            auto it = gens[i].regCaches.find(found);
+            if (it == gens[i].regCaches.end()) {
+              std::string name = "rcache" + std::to_string(cacheDecls.size()) + "_";
+              cacheDecls.push_back(cs.views.at(e->name).type.cName() + " " + name + "[" + std::to_string(want.slots) + "];");
+              it = gens[i].regCaches.emplace(found, StageCodegen::RegCache{name, true}).first;
+              gens[i].cachedStmt_ = red;
+            }
+            gens[j].regCaches[mine] = StageCodegen::RegCache{it->second.name, false};
+            gens[j].cachedPointwise_ = true;
+            break;
+          }
+        });
       }
     }
   }

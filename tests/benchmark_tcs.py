@@ -196,9 +196,10 @@ TUNED_AT_REFERENCE_SIZES = {
     "moments2": "naive;outerScheduleFusionStrategy=Max;fixParametersBeforeScheduling=1;tile=1;unroll=64;tileImperfectlyNested=1;"
                 "matchLibraryCalls=1;mapToThreads=1024;mapToBlocks=1152;usePrivateMemory=1;unrollCopyShared=1;"
                 "useReadOnlyCache=1;vectorWidth=2;collapseContiguous=0;useMfma=1",
-    "group_normalization_single_kernel": "naive;outerScheduleFusionStrategy=Max;intraTileScheduleFusionStrategy=Min;tile=1,1;"
-                                         "unroll=64;matchLibraryCalls=1;mapToThreads=1024;mapToBlocks=32,8;usePrivateMemory=1;"
-                                         "vectorWidth=4;prefetchShared=1",
+    # 576 threads x float4 = one 48x48 plane per pass: the normalising stage then finds every
+    # element in the register cache the two reductions filled (one read of the input)
+    "group_normalization_single_kernel": "naive;outerScheduleFusionStrategy=Max;tile=1,1;unroll=64;matchLibraryCalls=1;"
+                                         "mapToThreads=576;mapToBlocks=32,32;usePrivateMemory=1;vectorWidth=4",
     "kronecker3": "naive;outerScheduleFusionStrategy=Min;tile=1,32,0,128;unroll=8;tileImperfectlyNested=1;mapToThreads=128,8;"
                   "mapToBlocks=256;unrollCopyShared=1;collapseContiguous=0;useMfma=1",
     "wavenet1": "naive;intraTileScheduleFusionStrategy=Max;fixParametersBeforeScheduling=1;tile=2,8,16;unroll=64;"

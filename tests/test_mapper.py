@@ -222,3 +222,21 @@ def test_kernel_with_a_matrix_core_stage_runs_whole_wavefronts():
                                    "useSharedMemory=0;outerScheduleFusionStrategy=Max")
     assert launches == [((1, 1, 1), (64, 2, 1))]
     assert "v_mfma_f32_16x16x4_f32" in src and "blockAllReduceX<__tc::OpSum<float>, 64, 2, 1>" in src
+
+
+def test_pointwise_stage_reads_the_reductions_register_cache():
+    """Normalise-after-moments in one kernel: the reductions run over one merged variable
+    (r_d, r_h, r_w collapse), the normalising stage over (d, h*w); with 576 threads x 4 lanes every
+    thread meets the same element at the same slot in all three stages, so the input is read
+    once.  With 512 threads the forms differ and the last stage reads memory again."""
+    from tests import benchmark_tcs as B
+    src, entry, _, _ = B.CASES["group_normalization_single_kernel"]
+    shapes = B.REFERENCE_SIZES["group_normalization_single_kernel"]
+    common = ("naive;tile=1,1;mapToBlocks=32,32;matchLibraryCalls=1;vectorWidth=4;unroll=64;usePrivateMemory=1;"
+              "outerScheduleFusionStrategy=Max;mapToThreads=")
+    text, launches = mapped(src, entry, shapes, common + "576")
+    assert launches == [((32, 32, 1), (576, 1, 1))]
+    assert text.count("pI[") == 1 and "float rcache0_[64];" in text
+    assert "(rcache0_[a_] - (psum[" in text
+    text, _ = mapped(src, entry, shapes, common + "512")
+    assert text.count("pI[") == 2
