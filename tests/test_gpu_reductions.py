@@ -132,3 +132,24 @@ def test_many_unrolled_reductions_on_odd_rows(threads, block):
         out.fill_(float("nan"))
         tc.run(ex, [A], [out])
         assert torch.all(out == 1.0), (c, out.cpu().numpy())
+
+
+SOFTMAX = """
+def softmax(float(N, D) I) -> (O, maxVal, expSum) {
+    maxVal(n) max=! I(n, d)
+    expSum(n) +=! exp(I(n, d) - maxVal(n))
+    O(n, d) = exp(I(n, d) - maxVal(n)) / expSum(n)
+}
+"""
+
+
+@pytest.mark.parametrize("d,threads,reads", [(1024, 64, 1), (1024, 256, 1), (1000, 64, 2), (777, 128, 2)])
+def test_softmax_row_stays_in_registers_between_the_stages(d, threads, reads):
+    """Two reductions and a pointwise stage over the same row in one kernel: where the threads
+    cover the row exactly, all three take it from one read (register cache); where they do not
+    (folded points), the pointwise stage reads memory again.  Values against the oracle either way."""
+    print(f"softmax d={d} threads={threads}", flush=True)
+    A = np.random.Generator(np.random.Philox(d)).standard_normal((37, d), dtype=np.float32)
+    ex = check(SOFTMAX, "softmax", [A], f"naive;tile=1;mapToThreads={threads};mapToBlocks=64;matchLibraryCalls=1;"
+               f"vectorWidth=4;unroll=64;usePrivateMemory=1;outerScheduleFusionStrategy=Max", d)
+    assert ex.num_kernels == 1 and ex.compiled_source.count("pI[") == reads
