@@ -1517,18 +1517,26 @@ class StageCodegen {
       if (c == 0) continue;
       bool mine = !v.reduction ||
           (reduction && std::find(reduction->redVars.begin(), reduction->redVars.end(), v.name) != reduction->redVars.end());
-      if (!mine || v.partial()) return form;
-      if (v.threadAxis >= 0 && v.perThread * kc_.k.block[v.threadAxis] != v.tile) return form;
+      if (!mine) return form;
+      if (v.numTiles > 1 && (v.reduction || static_cast<int>(i) >= kc_.k.sharedDepth)) return form;
+      bool blockId = v.blockAxis >= 0 && v.gridExtent == v.numTiles;
+      std::string tileSym = blockId ? std::string("block.") + axisName(v.blockAxis) : "t_" + v.name;
+      int64_t B = v.threadAxis >= 0 ? kc_.k.block[v.threadAxis] : 1;
+      bool folded = v.partial() || (v.threadAxis >= 0 && v.perThread * B != v.tile);
+      if (folded) {
+        // the index is a clamped function of the same symbols: comparable only as a whole, between
+        // variables that are tiled, spread and clamped alike
+        std::ostringstream d;
+        d << "folded(" << v.min << "," << v.extent << "," << v.tile << "," << v.numTiles << ","
+          << (v.numTiles > 1 ? tileSym : std::string("-")) << "," << v.threadAxis << "," << B << "," << v.perThread << ","
+          << (v.perThread > 1 ? stride.at(v.name) : 0) << ")";
+        form.coef[d.str()] += c;
+        continue;
+      }
       form.constant += c * v.min;
-      if (v.numTiles > 1) {
-        if (v.reduction || static_cast<int>(i) >= kc_.k.sharedDepth) return form;
-        bool blockId = v.blockAxis >= 0 && v.gridExtent == v.numTiles;
-        form.coef[blockId ? std::string("block.") + axisName(v.blockAxis) : "t_" + v.name] += c * v.tile;
-      }
+      if (v.numTiles > 1) form.coef[tileSym] += c * v.tile;
       if (v.threadAxis >= 0) form.coef[std::string("thread.") + axisName(v.threadAxis)] += c;
-      if (v.perThread > 1) {
-        form.coef["q." + std::to_string(stride.at(v.name))] += c * (v.threadAxis >= 0 ? kc_.k.block[v.threadAxis] : 1);
-      }
+      if (v.perThread > 1) form.coef["q." + std::to_string(stride.at(v.name))] += c * B;
     }
     form.valid = true;
     return form;
