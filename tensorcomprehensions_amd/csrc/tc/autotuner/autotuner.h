@@ -46,6 +46,9 @@ struct TunerSettings {
   std::string cacheFile; // when set: seeds the first generation from it and appends the result
   // candidates doing more than this many times the per-thread work of the best one are not run
   double maxSerialDepthRatio = 256.0;
+  // generation 0 also holds a few structured variants of the first base mapping (streaming,
+  // row-reduction and matrix-core shapes); the search then starts from more than one basin
+  bool seedHeuristics = true;
 };
 
 namespace detail {
@@ -86,6 +89,75 @@ inline std::vector<size_t> inputDivisorsAndPowers2(
   return mergeVectors(std::move(out), powers2andCeilDivisors(256));
 }
 
+// Thread counts that cover merged trailing dimensions exactly, whole or in lanes of 2 or 4
+// elements (784 = 28*28 -> 196 threads x float4): contiguous dimensions collapse in the mapper, and
+// a block that covers the merged extent has no folded points.
+inline std::vector<size_t> mergedDimensionThreadCounts(const std::vector<const DLConstTensor*>& inputs) {
+  std::vector<size_t> merged;
+  for (auto t : inputs) {
+    size_t product = 1;
+    for (int i = t->ndim - 1; i >= 0 && product <= 4096; --i) {
+      product *= static_cast<size_t>(t->shape[i]);
+      for (size_t lanes : {1, 2, 4}) {
+        if (i < t->ndim - 1 && product % lanes == 0 && product / lanes >= 64 && product / lanes <= 1024) {
+          merged.push_back(product / lanes);
+        }
+      }
+    }
+  }
+  std::sort(merged.begin(), merged.end());
+  merged.erase(std::unique(merged.begin(), merged.end()), merged.end());
+  return merged;
+}
+
+// Structured starting points next to the caller's base mapping.  The genetic search from one
+// point tends to settle in that point's basin (small blocks of scalar accesses for the naive
+// options); these cover the three kernel shapes the mapper is built around.  Every value used is
+// a member of the search space (0, powers of two up to 256, merged-dimension thread counts).
+inline std::vector<HipMappingOptions> heuristicSeeds(
+    const HipMappingOptions& base, const std::vector<const DLConstTensor*>& inputs) {
+  std::vector<HipMappingOptions> seeds;
+  std::vector<uint64_t> threadCounts{256};
+  for (size_t m : mergedDimensionThreadCounts(inputs)) {
+    if (threadCounts.size() < 3) threadCounts.push_back(m);
+  }
+  for (uint64_t threads : threadCounts) {
+    // streaming: outer dimensions over blocks, a short unrolled dimension, the merged innermost
+    // dimension over the threads in lanes of four
+    for (uint64_t inner : {1, 4, 8}) {
+      HipMappingOptions o = base;
+      o.generic.tile(std::vector<uint64_t>{1, inner, 0, 0});
+      o.generic.unroll(128);
+      o.mapToThreads(threads).mapToBlocks(256, 256).useReadOnlyCache(true);
+      o.vectorWidthValue = 4;
+      o.collapseContiguousValue = true;
+      seeds.push_back(o);
+    }
+    // row reductions: one row per block, the reduction over the threads, later stages of the
+    // kernel from the register cache
+    for (uint64_t unroll : {8, 64}) {
+      HipMappingOptions o = base;
+      o.generic.tile(std::vector<uint64_t>{1, 1});
+      o.generic.unroll(unroll);
+      o.generic.matchLibraryCallsValue = true;
+      o.generic.outerScheduleOptions.fusionStrategy = FusionStrategy::Max;
+      o.mapToThreads(threads).mapToBlocks(256, 256).useReadOnlyCache(true).usePrivateMemory(true);
+      o.vectorWidthValue = 4;
+      o.collapseContiguousValue = true;
+      seeds.push_back(o);
+    }
+  }
+  // dense contractions: one batch element and a 32x32 output tile per block on the matrix cores
+  for (bool lds : {false, true}) {
+    HipMappingOptions o = base;
+    o.generic.tile(std::vector<uint64_t>{1, 32, 32});
+    o.mapToThreads(64, 4).mapToBlocks(256, 256).useSharedMemory(lds).useReadOnlyCache(true);
+    o.useMfmaValue = true;
+    seeds.push_back(o);
+  }
+  return seeds;
+}
+
 // Candidate value sets derived from the input shapes (tc/autotuner/autotuner-inl.h:326-404).
 inline TuningConfiguration setupTuningParameters(
     const std::vector<const DLConstTensor*>& inputs, const std::vector<HipMappingOptions>& baseMappings,
@@ -97,6 +169,8 @@ inline TuningConfiguration setupTuningParameters(
   std::vector<size_t> tileRange = range;
   tileRange.push_back(0); // 0 = do not tile this dimension
   std::vector<size_t> blockRange = range, gridRange = range;
+  // Deviation: thread counts that cover merged trailing dimensions exactly.
+  blockRange = mergeVectors(std::move(blockRange), mergedDimensionThreadCounts(inputs));
   size_t tileDims = maxRank + 1;
   for (const auto& b : baseMappings) {
     blockRange = mergeVectors(std::move(blockRange), std::vector<size_t>(b.block.extractVector().begin(), b.block.extractVector().end()));
@@ -168,6 +242,11 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
 
   // search space and starting points
   std::vector<MappingOptionsType> bases = baseMappings;
+  if (settings.seedHeuristics) {
+    for (auto& seed : detail::heuristicSeeds(baseMappings.front(), firstInputs)) {
+      if (std::find(bases.begin(), bases.end(), seed) == bases.end()) bases.push_back(std::move(seed));
+    }
+  }
   if (!settings.cacheFile.empty()) {
     auto restored = loadTopKFromCacheFile<Backend>(
         canonicalTc, inputsInfo, outputsInfo, Backend::makeDeviceFilename(settings.cacheFile), settings.restoreNumber);

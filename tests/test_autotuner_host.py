@@ -34,7 +34,10 @@ def test_search_space_from_shapes():
     for v in (26, 72, 500, 13, 36, 250, 256, 64):           # divisors of the dims, and of 256
         assert v in tile and v in block
     assert fields["unroll"] == "1,2,4,8,16,32,64,128,256"
-    assert fields["block"] == fields["grid"]                # naive's 64,4 / 256,256 are already members
+    grid = [int(x) for x in fields["grid"].split(",")]      # naive's 64,4 / 256,256 are already members
+    # blocks add the thread counts that cover merged trailing dimensions exactly, whole or in lanes
+    # of 2 or 4: 26*72 = 1872 -> 936, 468 (72*26 likewise)
+    assert sorted(set(block) - set(grid)) == [468, 936] and set(grid) <= set(block)
 
 
 def test_base_mapping_outside_the_space_is_refused():
