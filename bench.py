@@ -217,6 +217,8 @@ def main():
     ap.add_argument("--config", default="c2_tensordot")
     ap.add_argument("--options", default=None)
     ap.add_argument("--all", action="store_true")
+    ap.add_argument("--tune", default=None, metavar="GENERATIONSxPOPULATION",
+                    help="autotune the workload from the naive options first (e.g. 5x40) and measure the best")
     ap.add_argument("--suite", action="store_true",
                     help="also time the reference's other benchmark comprehensions at their default sizes")
     ap.add_argument("--no-cpu", action="store_true")
@@ -231,6 +233,19 @@ def main():
 
     if a.calibrate:
         calibrate_copy(a.steps)
+    tuned_in = None
+    if a.tune:
+        import tensorcomprehensions_amd as tc
+        gens, pop = (int(x) for x in a.tune.lower().split("x"))
+        src, entry = W.CONFIGS[a.config][0], W.CONFIGS[a.config][1]
+        ins = [torch.from_numpy(x).cuda() for x in W.make_inputs(a.config)]
+        t0 = time.perf_counter()
+        best = tc.autotune(src, entry, ins, "naive", generations=gens, pop_size=pop, threads=16, seed=1, top_k=1)
+        tuned_in = time.perf_counter() - t0
+        if not best:
+            sys.exit("the autotuner found no runnable candidate")
+        a.options = best[0].to_text()
+        del ins
     m = measure(a.config, a.steps, a.warmup, a.options)
     value = m["bytes"] * a.steps / m["wall_s"] / 1e9
     line = {
@@ -243,6 +258,8 @@ def main():
         "roofline": roofline(m),
         "device": torch.cuda.get_device_name(0),
     }
+    if tuned_in is not None:
+        line["config"]["options_from"] = f"autotuned from the naive options, {a.tune} candidates, {tuned_in:.0f} s"
     if not a.no_cpu:
         line["cpu_baseline"] = cpu_baseline(a.config)
         line["cpu_baseline"]["host_cores"] = os.cpu_count()
