@@ -1924,8 +1924,59 @@ class StageCodegen {
         em_.close();
       }
       em_.close();
-      em_.open("for (int " + tv(k0) + " = 0; " + tv(k0) + " < " + std::to_string(k0.numTiles) + "; ++" + tv(k0) + ")");
-      stagePromotions(true);
+      // Software pipeline over the reduction tiles (prefetchShared): the global loads of the next
+      // tile's operands are issued before the current tile is multiplied and land in registers;
+      // they go to LDS after the multiplication, between two barriers.
+      bool pipelineK = kc_.opts.prefetchSharedValue;
+      int64_t stagingRegs = 0;
+      bool anyInside = false;
+      for (const auto& p : st_.promotions) {
+        if (!p.insideReductionTiles) continue;
+        anyInside = true;
+        stagingRegs += copyRegisters(p);
+      }
+      pipelineK = pipelineK && anyInside && stagingRegs <= 64;
+      const std::string tk = tv(k0);
+      if (pipelineK) {
+        em_.open("");
+        ++opened;
+        for (const auto& p : st_.promotions) {
+          if (p.insideReductionTiles) em_.line(copyRegisterDecl(p, "pk_" + p.tensor + "_"));
+        }
+        em_.open("");
+        em_.line("const int " + tk + " = 0;");
+        for (const auto& p : st_.promotions) {
+          if (!p.insideReductionTiles) continue;
+          declareLows(p);
+          emitCopyLoads(p, "pk_" + p.tensor + "_");
+        }
+        em_.line("__syncthreads();");
+        for (const auto& p : st_.promotions) {
+          if (p.insideReductionTiles) emitCopyStores(p, "pk_" + p.tensor + "_");
+        }
+        em_.close();
+      }
+      em_.open("for (int " + tk + " = 0; " + tk + " < " + std::to_string(k0.numTiles) + "; ++" + tk + ")");
+      if (pipelineK) {
+        em_.line("__syncthreads();");
+        em_.line("const bool more_ = " + tk + " + 1 < " + std::to_string(k0.numTiles) + ";");
+        em_.open("if (more_)");
+        tileOverride[k0.name] = "(" + tk + " + 1)";
+        for (const auto& p : st_.promotions) {
+          if (!p.insideReductionTiles) continue;
+          declareLows(p);
+          emitCopyLoads(p, "pk_" + p.tensor + "_");
+        }
+        tileOverride.clear();
+        em_.close();
+        for (const auto& p : st_.promotions) {
+          if (!p.insideReductionTiles) continue;
+          declareLows(p);
+          activePromotions_.insert(p.tensor);
+        }
+      } else {
+        stagePromotions(true);
+      }
       em_.line("#pragma unroll");
       em_.open("for (int j_ = 0; j_ < " + std::to_string(tilesPerWave) + "; ++j_)");
       em_.line("const int tl_ = wv_ + j_ * " + std::to_string(st_.waves) + ";");
@@ -1934,6 +1985,14 @@ class StageCodegen {
       multiply("cacc_[j_]");
       em_.close();
       em_.close();
+      if (pipelineK) {
+        em_.line("__syncthreads();");
+        em_.open("if (more_)");
+        for (const auto& p : st_.promotions) {
+          if (p.insideReductionTiles) emitCopyStores(p, "pk_" + p.tensor + "_");
+        }
+        em_.close();
+      }
       em_.close();
       em_.line("#pragma unroll");
       em_.open("for (int j_ = 0; j_ < " + std::to_string(tilesPerWave) + "; ++j_)");

@@ -138,6 +138,9 @@ def test_prefetched_lds_staging_on_the_vector_path():
     "naive;tile=32,48,16;mapToThreads=64,8;mapToBlocks=256,256;useMfma=1;useSharedMemory=1",
     "naive;tile=64,32,24;mapToThreads=64,2;mapToBlocks=256,256;useMfma=1;useSharedMemory=0",
     "naive;tile=16,16,7;mapToThreads=64,4;mapToBlocks=256,256;useMfma=1;useSharedMemory=1",   # 7 does not divide 192: untiled
+    # software pipeline over the reduction tiles: the next tile's operands load while this one multiplies
+    "naive;tile=64,64,32;mapToThreads=64,4;mapToBlocks=256,256;useMfma=1;useSharedMemory=1;prefetchShared=1",
+    "naive;tile=32,48,16;mapToThreads=64,8;mapToBlocks=3,2;useMfma=1;useSharedMemory=1;prefetchShared=1",
 ])
 def test_reduction_tiling_stages_operands_per_tile(opts):
     """The outermost reduction index may be tiled: operands are staged in LDS once per reduction
@@ -155,6 +158,7 @@ def test_reduction_tiling_stages_operands_per_tile(opts):
     assert np.array_equal(C.cpu().numpy(), A @ B)                 # small integers: exact in fp32
     tiled = "for (int t_r_k" in ex.compiled_source
     assert tiled == (",7;" not in opts)
+    assert ("pk_A_" in ex.compiled_source) == ("prefetchShared=1" in opts)
     # accumulate into an existing output across reduction tiles
     acc = "def mm(float(M, K) A, float(K, N) B) -> (C) { C(m, n) += A(m, r_k) * B(r_k, n) }"
     ex = tc.compile(acc, "mm", ins, opts)
