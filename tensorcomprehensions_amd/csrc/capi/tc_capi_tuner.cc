@@ -283,6 +283,42 @@ extern "C" int tc_host_query(const char* what, const char* arg, char** out) {
       result = "tile_dims=" + std::to_string(c.tilingParams.dims.size()) + ";tile=" + joinSizes(c.tilingParams.dims[0].values()) +
           ";block=" + joinSizes(c.blockParams.dims[0].values()) + ";grid=" + joinSizes(c.gridParams.dims[0].values()) +
           ";unroll=" + joinSizes(c.unrollFactor.values()) + ";genes=" + std::to_string(c.collectParameters().size());
+    } else if (w == "tuner_seeds") {
+      // "rank:shapes": smallest output rank, then shapes as for search_space -> the structured
+      // starting points the search space accepts (one option text per line), as generation 0
+      // would hold them next to the naive options
+      std::vector<std::vector<int64_t>> shapes;
+      size_t colon = a.find(':');
+      TC_CHECK(colon != std::string::npos) << "expected <smallest output rank>:<shapes>";
+      size_t smallestOutputRank = std::stoul(a.substr(0, colon));
+      std::stringstream ss(a.substr(colon + 1));
+      std::string sh;
+      while (std::getline(ss, sh, ';')) {
+        std::vector<int64_t> dims;
+        std::stringstream ds(sh);
+        std::string d;
+        while (std::getline(ds, d, 'x')) dims.push_back(std::stoll(d));
+        shapes.push_back(dims);
+      }
+      std::vector<DLConstTensor> ts(shapes.size());
+      std::vector<const DLConstTensor*> ptrs;
+      for (size_t i = 0; i < shapes.size(); ++i) {
+        ts[i] = DLConstTensor{nullptr, {kDLROCM, 0}, static_cast<int>(shapes[i].size()), {2, 32, 1}, shapes[i].data(), nullptr, 0};
+        ptrs.push_back(&ts[i]);
+      }
+      HipMappingOptions naive = HipMappingOptions::makeNaiveMappingOptions();
+      TuningConfiguration space = tc::autotune::detail::setupTuningParameters(ptrs, {naive}, 256);
+      for (const auto& seed : tc::autotune::detail::heuristicSeeds(naive, ptrs, smallestOutputRank)) {
+        try {
+          TuningConfiguration c = space;
+          c.fromHipMappingOptions(seed);
+          if (!c.isValid()) continue;
+          HipMappingOptions applied = naive;
+          c.applyToHipMappingOptions(applied);
+          result += (result.empty() ? "" : "\n") + applied.toText();
+        } catch (const std::invalid_argument&) {
+        }
+      }
     } else if (w == "sync_placement") {
       // "cyclic;n;i:k:level,i:k:level,..." -> "position:level,..." (barrier after child `position`)
       std::stringstream ss(a);

@@ -115,8 +115,14 @@ inline std::vector<size_t> mergedDimensionThreadCounts(const std::vector<const D
 // options); these cover the three kernel shapes the mapper is built around.  Every value used is
 // a member of the search space (0, powers of two up to 256, merged-dimension thread counts).
 inline std::vector<HipMappingOptions> heuristicSeeds(
-    const HipMappingOptions& base, const std::vector<const DLConstTensor*>& inputs) {
+    const HipMappingOptions& base, const std::vector<const DLConstTensor*>& inputs, size_t smallestOutputRank) {
   std::vector<HipMappingOptions> seeds;
+  size_t maxRank = 0;
+  uint64_t largest = 256; // largest extent: a grid limit that never forces a block to loop over tiles
+  for (auto t : inputs) {
+    maxRank = std::max<size_t>(maxRank, t->ndim);
+    for (int i = 0; i < t->ndim; ++i) largest = std::max<uint64_t>(largest, static_cast<uint64_t>(t->shape[i]));
+  }
   std::vector<uint64_t> threadCounts{256};
   for (size_t m : mergedDimensionThreadCounts(inputs)) {
     if (threadCounts.size() < 3) threadCounts.push_back(m);
@@ -126,9 +132,11 @@ inline std::vector<HipMappingOptions> heuristicSeeds(
     // dimension over the threads in lanes of four
     for (uint64_t inner : {1, 4, 8}) {
       HipMappingOptions o = base;
-      o.generic.tile(std::vector<uint64_t>{1, inner, 0, 0});
+      std::vector<uint64_t> tile{1, inner};
+      while (tile.size() < maxRank) tile.push_back(0);
+      o.generic.tile(tile);
       o.generic.unroll(128);
-      o.mapToThreads(threads).mapToBlocks(256, 256).useReadOnlyCache(true);
+      o.mapToThreads(threads).mapToBlocks(largest, 256).useReadOnlyCache(true);
       o.vectorWidthValue = 4;
       o.collapseContiguousValue = true;
       seeds.push_back(o);
@@ -137,11 +145,15 @@ inline std::vector<HipMappingOptions> heuristicSeeds(
     // kernel from the register cache
     for (uint64_t unroll : {8, 64}) {
       HipMappingOptions o = base;
-      o.generic.tile(std::vector<uint64_t>{1, 1});
+      // the output of lowest rank is what the reductions produce: its dimensions are the rows
+      // (tile 1 each: one row per block); the reduction dimensions after them stay whole
+      std::vector<uint64_t> rows(std::max<size_t>(1, smallestOutputRank), 1);
+      rows.push_back(0);
+      o.generic.tile(rows);
       o.generic.unroll(unroll);
       o.generic.matchLibraryCallsValue = true;
       o.generic.outerScheduleOptions.fusionStrategy = FusionStrategy::Max;
-      o.mapToThreads(threads).mapToBlocks(256, 256).useReadOnlyCache(true).usePrivateMemory(true);
+      o.mapToThreads(threads).mapToBlocks(largest, 256).useReadOnlyCache(true).usePrivateMemory(true);
       o.vectorWidthValue = 4;
       o.collapseContiguousValue = true;
       seeds.push_back(o);
@@ -151,7 +163,7 @@ inline std::vector<HipMappingOptions> heuristicSeeds(
   for (bool lds : {false, true}) {
     HipMappingOptions o = base;
     o.generic.tile(std::vector<uint64_t>{1, 32, 32});
-    o.mapToThreads(64, 4).mapToBlocks(256, 256).useSharedMemory(lds).useReadOnlyCache(true);
+    o.mapToThreads(64, 4).mapToBlocks(largest, 256).useSharedMemory(lds).useReadOnlyCache(true);
     o.useMfmaValue = true;
     seeds.push_back(o);
   }
@@ -242,11 +254,6 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
 
   // search space and starting points
   std::vector<MappingOptionsType> bases = baseMappings;
-  if (settings.seedHeuristics) {
-    for (auto& seed : detail::heuristicSeeds(baseMappings.front(), firstInputs)) {
-      if (std::find(bases.begin(), bases.end(), seed) == bases.end()) bases.push_back(std::move(seed));
-    }
-  }
   if (!settings.cacheFile.empty()) {
     auto restored = loadTopKFromCacheFile<Backend>(
         canonicalTc, inputsInfo, outputsInfo, Backend::makeDeviceFilename(settings.cacheFile), settings.restoreNumber);
@@ -263,6 +270,21 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
     TuningConfiguration c = space;
     c.fromHipMappingOptions(b); // throws std::invalid_argument for values outside the space
     configs.push_back(c);
+  }
+  if (settings.seedHeuristics) {
+    // after the caller's own starting points; a seed the (possibly restricted) space cannot
+    // express is left out
+    size_t smallestOutputRank = outputsInfo.empty() ? 1 : outputsInfo.front().shape.size();
+    for (const auto& info : outputsInfo) smallestOutputRank = std::min(smallestOutputRank, info.shape.size());
+    for (const auto& seed : detail::heuristicSeeds(baseMappings.front(), firstInputs, smallestOutputRank)) {
+      if (std::find(bases.begin(), bases.end(), seed) != bases.end()) continue;
+      try {
+        TuningConfiguration c = space;
+        c.fromHipMappingOptions(seed);
+        if (c.isValid()) configs.push_back(c);
+      } catch (const std::invalid_argument&) {
+      }
+    }
   }
   SearchStrategy search(
       configs, settings.generations, settings.populationSize, settings.crossOverRate, settings.mutationRate,
