@@ -161,6 +161,8 @@ def suite_library_routines():
         "tmm": lambda a, b: a @ b.t(),
         "matmul": lambda a, b: a @ b,
         "convolution": lambda i, w, b: F.conv2d(i, w, b),
+        "group_convolution": lambda i, w, b: F.conv2d(
+            i.reshape(i.shape[0], -1, i.shape[3], i.shape[4]), w.reshape(-1, *w.shape[2:]), b.reshape(-1), groups=i.shape[1]),
         "2fcrelu": lambda i, w1, b1, w2, b2: F.relu(F.linear(F.relu(F.linear(i, w1, b1)), w2, b2)),
         "lut": lambda t, i: t[i.long()].sum(1),
         "moments2": lambda x: (x.mean(1), x.var(1, unbiased=False)),

@@ -143,7 +143,15 @@ def wavenet1(
 }
 """
 
+GROUP_CONVOLUTION = """
+def group_convolution(float(N, G, C, H, W) I, float(G, F, C, KH, KW) W1, float(G, F) B) -> (O) {
+    O(n, g, o, h, w) +=! I(n, g, r_i, h + r_kh, w + r_kw) * W1(g, o, r_i, r_kh, r_kw)
+    O(n, g, o, h, w) = O(n, g, o, h, w) + B(g, o)
+}
+"""
+
 CASES = {
+    "group_convolution": (GROUP_CONVOLUTION, "group_convolution", [(2, 3, 4, 10, 9), (3, 5, 4, 3, 3), (3, 5)], 36),
     "tmm": (TMM, "tmm", [(32, 256), (128, 256)], 256),
     "tmm_odd": (TMM, "tmm", [(37, 70), (51, 70)], 70),
     "matmul": (MATMUL, "matmul", [(72, 60), (60, 50)], 60),
@@ -166,10 +174,11 @@ CASES = {
 
 # The same comprehensions at the default sizes of the reference's benchmark programs
 # (tc/benchmarks/tmm.cc:42-44, MLP_model.cc:43-59 for the 1000x1024 matmul, the fc-relu chain and
-# the look-up table, convolution.cc:40-46, moments.cc:42-43, group_normalization.cc:42-46,
+# the look-up table, convolution.cc:40-46, group_convolution.cc:42-49, moments.cc:42-43, group_normalization.cc:42-46,
 # kronecker.cc:41-47, wavenet.cc:42-60), and the mapping options the autotuner found for them on an
 # MI355X (a few generations from the naive options; written relative to the naive options).
 REFERENCE_SIZES = {
+    "group_convolution": [(32, 32, 4, 56, 56), (32, 4, 4, 3, 3), (32, 4)],
     "tmm": [(32, 256), (128, 256)],
     "matmul": [(128, 1000), (1000, 1024)],
     "convolution": [(32, 4, 56, 56), (4, 4, 3, 3), (4,)],
@@ -181,12 +190,16 @@ REFERENCE_SIZES = {
     "wavenet1": [(1, 32, 4000), (32, 32, 2), (32,), (32, 32, 2), (32,), (32, 32), (32,), (32, 32), (32,), (1,)],
 }
 TUNED_AT_REFERENCE_SIZES = {
+    # one (n, g) image per block and half its rows per block in z, the 4x56x56 input window in LDS,
+    # 54 threads along w; hand-set: the search's thread counts do not contain 54 x 9
+    "group_convolution": "naive;tile=1,1,4,27,0;mapToThreads=54,9;mapToBlocks=32,32,8;useSharedMemory=1;unroll=16;"
+                         "useReadOnlyCache=1",
     "tmm": "naive;tile=64,2;unroll=2;matchLibraryCalls=1;mapToThreads=128,1;mapToBlocks=256,1;usePrivateMemory=1;"
            "unrollCopyShared=1;useReadOnlyCache=1;vectorWidth=2;collapseContiguous=0;useMfma=1;prefetchShared=1",
     "matmul": "naive;intraTileScheduleFusionStrategy=Max;tile=16,32;unroll=256;matchLibraryCalls=1;mapToThreads=512,2;"
               "mapToBlocks=125,1000;unrollCopyShared=1;useReadOnlyCache=1;useMfma=1;prefetchShared=1",
-    "convolution": "naive;intraTileScheduleFusionStrategy=Min;fixParametersBeforeScheduling=1;tile=2,27,1,56;unroll=256;"
-                   "tileImperfectlyNested=1;mapToThreads=128,7;mapToBlocks=256,64;useSharedMemory=1;useReadOnlyCache=1;"
+    "convolution": "naive;intraTileScheduleFusionStrategy=Min;fixParametersBeforeScheduling=1;tile=1,27,1,0;unroll=128;"
+                   "tileImperfectlyNested=1;mapToThreads=256,1;mapToBlocks=256,64,1;useSharedMemory=1;useReadOnlyCache=1;"
                    "collapseContiguous=0",
     "2fcrelu": "naive;outerScheduleFusionStrategy=Max;intraTileScheduleFusionStrategy=Max;fixParametersBeforeScheduling=1;"
                "tile=4;unroll=32;mapToThreads=8,128;mapToBlocks=1024;useSharedMemory=1;unrollCopyShared=1;useReadOnlyCache=1;"
@@ -200,10 +213,11 @@ TUNED_AT_REFERENCE_SIZES = {
     # element in the register cache the two reductions filled (one read of the input)
     "group_normalization_single_kernel": "naive;outerScheduleFusionStrategy=Max;tile=1,1;unroll=64;matchLibraryCalls=1;"
                                          "mapToThreads=576;mapToBlocks=32,32;usePrivateMemory=1;vectorWidth=4",
-    "kronecker3": "naive;outerScheduleFusionStrategy=Min;tile=1,32,0,128;unroll=8;tileImperfectlyNested=1;mapToThreads=128,8;"
-                  "mapToBlocks=256;unrollCopyShared=1;collapseContiguous=0;useMfma=1",
-    "wavenet1": "naive;intraTileScheduleFusionStrategy=Max;fixParametersBeforeScheduling=1;tile=2,8,16;unroll=64;"
-                "mapToThreads=32,4;mapToBlocks=2000,256;usePrivateMemory=1;collapseContiguous=0",
+    "kronecker3": "naive;outerScheduleFusionStrategy=Max;intraTileScheduleFusionStrategy=Min;tile=1,32;unroll=256;"
+                  "mapToThreads=128,4;mapToBlocks=256,32;unrollCopyShared=1;useReadOnlyCache=1;collapseContiguous=0;useMfma=1",
+    "wavenet1": "naive;intraTileScheduleFusionStrategy=Max;fixParametersBeforeScheduling=1;tile=2,2000,16,1;mapToThreads=16,64;"
+                "mapToBlocks=2000,256;useSharedMemory=1;usePrivateMemory=1;privateDepth=8;sharedDepth=3;vectorWidth=4;"
+                "collapseContiguous=0;prefetchShared=1",
 }
 
 

@@ -37,6 +37,9 @@ def test_oracle_matches_library_routines():
     ins = B.make_inputs("convolution")
     ref = torch.nn.functional.conv2d(f64(ins[0]), f64(ins[1]), f64(ins[2]))
     close(tc_oracle.run(B.CONVOLUTION, "convolution", ins)[0], ref, 36)
+    I, Wg, Bg = B.make_inputs("group_convolution")
+    ref = torch.nn.functional.conv2d(f64(I).reshape(2, 12, 10, 9), f64(Wg).reshape(15, 4, 3, 3), f64(Bg).reshape(15), groups=3)
+    close(tc_oracle.run(B.GROUP_CONVOLUTION, "group_convolution", [I, Wg, Bg])[0], ref.reshape(2, 3, 5, 8, 7), 36)
     I, W1, B1, W2, B2 = B.make_inputs("2fcrelu")
     o1 = torch.relu(f64(I) @ f64(W1).T + f64(B1))
     o2 = torch.relu(o1 @ f64(W2).T + f64(B2))

@@ -54,7 +54,7 @@ def test_parity_at_the_reference_sizes_with_the_tuned_options(name):
     tc.run(ex, ins, outs)
     torch.cuda.synchronize()
     # reduction lengths at these sizes (chains: the product of the lengths)
-    k = {"tmm": 256, "matmul": 1000, "convolution": 36, "2fcrelu": 2000 * 128, "lut": 50, "moments2": 36864,
+    k = {"tmm": 256, "matmul": 1000, "convolution": 36, "group_convolution": 36, "2fcrelu": 2000 * 128, "lut": 50, "moments2": 36864,
          "group_normalization_single_kernel": 36864, "kronecker3": 16 ** 3, "wavenet1": 32 * 64}[name]
     for o, r in zip(outs, ref):
         got = o.cpu().numpy()
