@@ -87,8 +87,10 @@ int sharedPrefix(const RawStage& A, const RawStage& B) {
   };
   // RAW / WAW: B touches what A wrote
   limitBy(B, a0.tensor, a0.lhsVars.size());
-  if (a0.tensor == b0.tensor) {
-    return -1; // same tensor, different box: keep apart
+  if (a0.tensor == b0.tensor && a0.lhsVars.size() > d) {
+    // a later stage of another shape rewrites the tensor: they share a kernel only when every
+    // subscript of the tensor is a shared variable (each iteration then touches its own element)
+    return -1;
   }
   // WAR: A read what B writes
   limitBy(A, b0.tensor, b0.lhsVars.size());

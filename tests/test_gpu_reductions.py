@@ -153,3 +153,27 @@ def test_softmax_row_stays_in_registers_between_the_stages(d, threads, reads):
     ex = check(SOFTMAX, "softmax", [A], f"naive;tile=1;mapToThreads={threads};mapToBlocks=64;matchLibraryCalls=1;"
                f"vectorWidth=4;unroll=64;usePrivateMemory=1;outerScheduleFusionStrategy=Max", d)
     assert ex.num_kernels == 1 and ex.compiled_source.count("pI[") == reads
+
+
+ROW_NORMALISE = """
+def f(float(N, M) A) -> (S, T) {
+    S(n, m) = A(n, m) + 2
+    T(n) +=! A(n, m) * A(n, m)
+    S(n, m) = S(n, m) / (T(n) + 1)
+}
+"""
+
+
+@pytest.mark.parametrize("options", [
+    "naive;tile=1;mapToThreads=128;mapToBlocks=64;outerScheduleFusionStrategy=Max",
+    "naive;tile=1;mapToThreads=128;mapToBlocks=64;outerScheduleFusionStrategy=Max;matchLibraryCalls=1;vectorWidth=4;usePrivateMemory=1",
+    "naive;tile=2,64;mapToThreads=32,2;mapToBlocks=8;outerScheduleFusionStrategy=Max;unroll=4",
+    "naive;outerScheduleFusionStrategy=Min",
+])
+def test_tensor_rewritten_by_a_later_stage_of_the_same_kernel(options):
+    """S is written, a reduction over the same rows follows, then S is rewritten from itself and
+    the reduction's result: one kernel under maximal fusion (the rewrite waits behind a barrier
+    for the reduction), three kernels under minimal fusion; same values."""
+    A = np.random.Generator(np.random.Philox(9)).standard_normal((50, 384), dtype=np.float32)
+    ex = check(ROW_NORMALISE, "f", [A], options, 384)
+    assert ex.num_kernels == (3 if "Min" in options else 1)

@@ -240,3 +240,26 @@ def test_pointwise_stage_reads_the_reductions_register_cache():
     assert "(rcache0_[a_] - (psum[" in text
     text, _ = mapped(src, entry, shapes, common + "512")
     assert text.count("pI[") == 2
+
+
+def test_a_later_rewrite_of_a_tensor_joins_the_kernel_of_its_producer():
+    """One-pass moments: mean and var are reduced, then rescaled by two pointwise statements that
+    do not follow their reductions directly.  Every subscript of both tensors is the shared row
+    variable, so all four stages form one kernel."""
+    from tests import benchmark_tcs as B
+    text, launches = mapped(B.MOMENTS2, "moments2_2D_1D", [(64, 512)],
+                            "naive;tile=1;mapToThreads=128;mapToBlocks=64;matchLibraryCalls=1;outerScheduleFusionStrategy=Max")
+    assert launches == [((64, 1, 1), (128, 1, 1))]
+    assert [ln.strip() for ln in text.split("\n") if ln.strip().startswith("// stage")] == [
+        "// stage 0: mean", "// stage 1: var", "// stage 2: mean", "// stage 3: var"]
+    # a rewrite over a variable the stages do not share stays in the kernel too, behind a barrier:
+    # other threads wrote the elements it reads
+    rows = """def f(float(N, M) A) -> (S, T) {
+        S(n, m) = A(n, m)
+        T(n) +=! A(n, m)
+        S(n, m) = S(n, m) / T(n)
+    }"""
+    text, launches = mapped(rows, "f", [(64, 512)], "naive;tile=1;mapToThreads=128;mapToBlocks=64;outerScheduleFusionStrategy=Max")
+    assert len(launches) == 1
+    body = text[text.index("// stage 1: T"):text.index("// stage 2: S")]
+    assert "__syncthreads();" in body
