@@ -115,7 +115,8 @@ inline std::vector<size_t> mergedDimensionThreadCounts(const std::vector<const D
 // options); these cover the three kernel shapes the mapper is built around.  Every value used is
 // a member of the search space (0, powers of two up to 256, merged-dimension thread counts).
 inline std::vector<HipMappingOptions> heuristicSeeds(
-    const HipMappingOptions& base, const std::vector<const DLConstTensor*>& inputs, size_t smallestOutputRank) {
+    const HipMappingOptions& base, const std::vector<const DLConstTensor*>& inputs, size_t smallestOutputRank,
+    size_t innermostOutputExtent = 0) {
   std::vector<HipMappingOptions> seeds;
   size_t maxRank = 0;
   uint64_t largest = 256; // largest extent: a grid limit that never forces a block to loop over tiles
@@ -156,6 +157,20 @@ inline std::vector<HipMappingOptions> heuristicSeeds(
       o.mapToThreads(threads).mapToBlocks(largest, 256).useReadOnlyCache(true).usePrivateMemory(true);
       o.vectorWidthValue = 4;
       o.collapseContiguousValue = true;
+      seeds.push_back(o);
+    }
+  }
+  // windows (convolutions with few channels): one image per block with its input window in LDS,
+  // the innermost output dimension along threadIdx.x and as many rows as fit along threadIdx.y
+  if (innermostOutputExtent >= 8 && innermostOutputExtent <= 256 && smallestOutputRank >= 3) {
+    uint64_t rows = 1;
+    while (rows * 2 * innermostOutputExtent <= 1024 && rows < 16) rows *= 2;
+    for (uint64_t unroll : {4, 16}) {
+      HipMappingOptions o = base;
+      o.generic.tile(std::vector<uint64_t>{1, 1, 0, 0, 0});
+      o.generic.unroll(unroll);
+      o.mapToThreads(innermostOutputExtent, rows).mapToBlocks(largest, 256).useSharedMemory(true).useReadOnlyCache(true);
+      o.collapseContiguousValue = false;
       seeds.push_back(o);
     }
   }
@@ -275,8 +290,13 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
     // after the caller's own starting points; a seed the (possibly restricted) space cannot
     // express is left out
     size_t smallestOutputRank = outputsInfo.empty() ? 1 : outputsInfo.front().shape.size();
-    for (const auto& info : outputsInfo) smallestOutputRank = std::min(smallestOutputRank, info.shape.size());
-    for (const auto& seed : detail::heuristicSeeds(baseMappings.front(), firstInputs, smallestOutputRank)) {
+    size_t innermostOutputExtent = 0;
+    for (const auto& info : outputsInfo) {
+      smallestOutputRank = std::min(smallestOutputRank, info.shape.size());
+      if (!info.shape.empty()) innermostOutputExtent = std::max<size_t>(innermostOutputExtent, info.shape.back());
+    }
+    for (const auto& seed :
+         detail::heuristicSeeds(baseMappings.front(), firstInputs, smallestOutputRank, innermostOutputExtent)) {
       if (std::find(bases.begin(), bases.end(), seed) != bases.end()) continue;
       try {
         TuningConfiguration c = space;
