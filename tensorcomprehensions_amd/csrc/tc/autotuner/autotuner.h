@@ -49,6 +49,9 @@ struct TunerSettings {
   // generation 0 also holds a few structured variants of the first base mapping (streaming,
   // row-reduction and matrix-core shapes); the search then starts from more than one basin
   bool seedHeuristics = true;
+  // after the last generation: rounds of one-gene steps around the best candidate (every gene
+  // moved to its neighbouring values, one at a time); a round that finds nothing better ends it
+  size_t refinementRounds = 2;
 };
 
 namespace detail {
@@ -330,8 +333,10 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
   // one a stalled tuning run is stuck on)
   const char* traceEnv = std::getenv("TC_TUNER_TRACE");
   const bool trace = traceEnv != nullptr && traceEnv[0] != '\0' && traceEnv[0] != '0';
-  for (size_t gen = 0; gen < settings.generations; ++gen) {
-    auto& population = search.population;
+  using Population = std::vector<std::unique_ptr<CandidateConfiguration>>;
+  // compiles (worker threads) and measures (this device) every candidate of `population`;
+  // returns the runtimes of the valid ones
+  auto evaluatePopulation = [&](Population& population) {
     std::atomic<size_t> cursor{0};
     std::mutex mu;
     std::condition_variable cv;
@@ -454,9 +459,12 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
     if (detail::tunerSignal == SIGTERM) {
       throw std::runtime_error("Abort requested");
     }
+    return generationTimes;
+  };
+  auto report = [&](const std::string& what, std::vector<Duration> generationTimes, size_t size) {
     if (settings.verbose || flags().tuner_gen_log_generations) {
       std::sort(generationTimes.begin(), generationTimes.end());
-      std::cerr << "[tuner] generation " << gen << ": " << generationTimes.size() << "/" << population.size()
+      std::cerr << "[tuner] " << what << ": " << generationTimes.size() << "/" << size
                 << " valid";
       if (!generationTimes.empty()) {
         std::cerr << " (best/median/worst) " << generationTimes.front().toMicroSecondsF() << "/"
@@ -465,8 +473,47 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
       }
       std::cerr << std::endl;
     }
+  };
+  for (size_t gen = 0; gen < settings.generations; ++gen) {
+    report("generation " + std::to_string(gen), evaluatePopulation(search.population), search.population.size());
     if (detail::tunerSignal == SIGINT) break;
     if (gen + 1 < settings.generations) search.updateParameters();
+  }
+  // Refinement (deviation): the genetic search recombines whole candidates; the last few percent
+  // are usually one gene away from its best one.
+  {
+    const CandidateConfiguration* best = nullptr;
+    for (const auto& c : search.population) {
+      if (!c->invalid && c->runtime != Duration::zero() && (!best || c->runtime < best->runtime)) best = c.get();
+    }
+    std::unique_ptr<CandidateConfiguration> center;
+    if (best) center.reset(new CandidateConfiguration(*best));
+    for (size_t round = 0; center && round < settings.refinementRounds && detail::tunerSignal == 0; ++round) {
+      Population neighbours;
+      size_t genes = center->configuration.collectParameters().size();
+      for (size_t g = 0; g < genes; ++g) {
+        for (int step : {-1, 1}) {
+          TuningConfiguration c = center->configuration;
+          RangeParameter* p = c.collectParameters()[g];
+          if (p->isForced()) continue;
+          long idx = static_cast<long>(p->selectedIndex()) + step;
+          if (idx < 0 || idx >= static_cast<long>(p->numberOptions())) continue;
+          p->selectOption(static_cast<size_t>(idx));
+          if (c.isValid()) neighbours.emplace_back(new CandidateConfiguration(c));
+        }
+      }
+      if (neighbours.empty()) break;
+      report("refinement " + std::to_string(round), evaluatePopulation(neighbours), neighbours.size());
+      const CandidateConfiguration* better = nullptr;
+      for (const auto& c : neighbours) {
+        if (!c->invalid && c->runtime != Duration::zero() && c->runtime < center->runtime &&
+            (!better || c->runtime < better->runtime)) {
+          better = c.get();
+        }
+      }
+      if (!better) break;
+      center.reset(new CandidateConfiguration(*better));
+    }
   }
   if (!settings.cacheFile.empty()) {
     appendTopKToCacheFile<Backend>(*optionsCache, Backend::makeDeviceFilename(settings.cacheFile), std::max<size_t>(topK, 10));

@@ -39,6 +39,7 @@ class RangeParameter {
   }
   bool isForced() const { return fixed_; }
   size_t value() const { return fixed_ ? fixedValue_ : values_.at(selected_); }
+  size_t selectedIndex() const { return selected_; }
   const std::vector<size_t>& values() const { return values_; }
   std::string name;
 
