@@ -201,9 +201,8 @@ TUNED_AT_REFERENCE_SIZES = {
     "convolution": "naive;intraTileScheduleFusionStrategy=Min;fixParametersBeforeScheduling=1;tile=1,27,1,0;unroll=128;"
                    "tileImperfectlyNested=1;mapToThreads=256,1;mapToBlocks=256,64,1;useSharedMemory=1;useReadOnlyCache=1;"
                    "collapseContiguous=0",
-    "2fcrelu": "naive;outerScheduleFusionStrategy=Max;intraTileScheduleFusionStrategy=Max;fixParametersBeforeScheduling=1;"
-               "tile=4;unroll=32;mapToThreads=8,128;mapToBlocks=1024;useSharedMemory=1;unrollCopyShared=1;useReadOnlyCache=1;"
-               "vectorWidth=4;useMfma=1",
+    "2fcrelu": "naive;outerScheduleFusionStrategy=Min;fixParametersBeforeScheduling=1;tile=1,32;unroll=256;mapToThreads=64;"
+               "mapToBlocks=2000,256;useSharedMemory=1;useReadOnlyCache=1;sharedDepth=1",
     "lut": "naive;outerScheduleFusionStrategy=Min;tile=4,32,32;unroll=64;usePrivateMemory=1;unrollCopyShared=1;"
            "collapseContiguous=0",
     "moments2": "naive;outerScheduleFusionStrategy=Max;fixParametersBeforeScheduling=1;tile=1;unroll=64;tileImperfectlyNested=1;"
@@ -213,8 +212,9 @@ TUNED_AT_REFERENCE_SIZES = {
     # element in the register cache the two reductions filled (one read of the input)
     "group_normalization_single_kernel": "naive;outerScheduleFusionStrategy=Max;tile=1,1;unroll=64;matchLibraryCalls=1;"
                                          "mapToThreads=576;mapToBlocks=32,32;usePrivateMemory=1;vectorWidth=4",
-    "kronecker3": "naive;outerScheduleFusionStrategy=Max;intraTileScheduleFusionStrategy=Min;tile=1,32;unroll=256;"
-                  "mapToThreads=128,4;mapToBlocks=256,32;unrollCopyShared=1;useReadOnlyCache=1;collapseContiguous=0;useMfma=1",
+    "kronecker3": "naive;outerScheduleFusionStrategy=Max;intraTileScheduleFusionStrategy=Max;tile=1,16,256;unroll=8;"
+                  "tileImperfectlyNested=1;mapToThreads=32,32;mapToBlocks=256,32;useSharedMemory=1;useReadOnlyCache=1;"
+                  "privateDepth=5;collapseContiguous=0;useMfma=1;prefetchShared=1",
     "wavenet1": "naive;intraTileScheduleFusionStrategy=Max;fixParametersBeforeScheduling=1;tile=2,2000,16,1;mapToThreads=16,64;"
                 "mapToBlocks=2000,256;useSharedMemory=1;usePrivateMemory=1;privateDepth=8;sharedDepth=3;vectorWidth=4;"
                 "collapseContiguous=0;prefetchShared=1",
