@@ -39,7 +39,7 @@ CONFIGS = {
 
 # Hand-picked mapping options per config (starting points of the tuner, also used by the benchmark).
 TUNED = {
-    "c1_tensordot_small": "naive;tile=1,1,2,0;mapToThreads=256;mapToBlocks=16,8;unroll=64;vectorWidth=1",
+    "c1_tensordot_small": "naive;tile=1,1,0,0,0;mapToThreads=425;mapToBlocks=256,256;unroll=128;vectorWidth=4;useReadOnlyCache=1",
     "c2_tensordot": "naive;tile=1,8,2,0;mapToThreads=256;mapToBlocks=32,64;unroll=128;vectorWidth=4;useReadOnlyCache=1",
     "c3_batch_matmul": "naive;tile=1,26,26;mapToThreads=64,4;mapToBlocks=500;useMfma=1;useSharedMemory=0",
     "c4_group_convolution": "naive;tile=1,1,16,14,14;mapToThreads=64,4;mapToBlocks=32,32;useMfma=1;useSharedMemory=1;useReadOnlyCache=1",
