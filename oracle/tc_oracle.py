@@ -602,6 +602,13 @@ class Analysis:
             if len(ann.dims) != len(s.indices):
                 raise TcError(f" tensor defined with {len(s.indices)} dimensions but declared as an output with {len(ann.dims)} dimensions.")
             scalar = _canon(ann.scalar)
+        if s.lhs in self.tensors and s.lhs not in self.inputs:
+            # a later statement keeps the type of the tensor's first definition; Halide refuses an
+            # update definition of another type (tc2halide.cc builds one Func per tensor), so a
+            # value that would lose precision is an error as it is for annotated outputs
+            have = self.tensors[s.lhs].scalar
+            if _canon(have) != match_types(scalar, have):
+                raise TcError(f" attempting to assign type {scalar} to narrower type {have} without an explicit cast")
         if s.assign in ("+=", "*=", "min=", "max=") and s.lhs not in self.tensors:
             self.warnings.append(f"Reduction without initialization. If {s.lhs} is not pre-initialized ...")
         if s.lhs not in self.outputs:

@@ -489,6 +489,18 @@ struct Lowering {
       if (t.name == s.tensor) out = &t;
     }
     TC_CHECK(out) << s.tensor << " is not an output";
+    if (!(out->argNames.empty() && out->extents.empty())) {
+      // a later statement of a tensor keeps the type of its first definition; Halide refuses an
+      // update definition of another type, so a value that would lose precision is an error
+      // here as it is for outputs annotated with a type (sema.h:531-551)
+      const ScalarType &have = out->type, &got = s.type;
+      bool narrows = (got.code == ScalarType::Float && have.code != ScalarType::Float) ||
+          (got.code == have.code && got.bits > have.bits);
+      if (narrows) {
+        throw lang::errorAt(stmtTree) << " attempting to assign type " << got.cName() << " to narrower type "
+                                      << have.cName() << " without an explicit cast";
+      }
+    }
     if (out->argNames.empty() && out->extents.empty()) {
       out->argNames = s.lhsVars;
       out->type = s.type;

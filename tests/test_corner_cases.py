@@ -148,3 +148,22 @@ def test_a_tensor_takes_the_bounds_of_its_last_definition_in_every_statement():
     A = np.full((16, 70, 1, 70), 7.0, np.float32)
     (o,) = tc_oracle.run(SHRINKING, "f", [A])
     assert o.tolist() == [3.0]
+
+
+def test_later_statement_cannot_narrow_into_the_tensors_first_type():
+    """`O` is int32 by its first definition; accumulating floats into it would be an update
+    definition of another type, which the reference's Halide lowering refuses.  The front end and
+    the oracle say so in the words used for annotated outputs; with an explicit cast, or a float
+    initial value, the program is accepted."""
+    from oracle import tc_oracle
+    bad = "def f(float(N) A) -> (O) { O(i) = 0 where i in 0:4\n O(i) += A(i) * 1.5 }"
+    with pytest.raises(tc.TcError) as e:
+        tc.map_only(bad, "f", [F(4)], "naive")
+    assert "to narrower type" in str(e.value)
+    with pytest.raises(tc_oracle.TcError) as e:
+        tc_oracle.infer_output_shapes(bad, "f", [(4,)])
+    assert "to narrower type" in str(e.value)
+    for good in ("def f(float(N) A) -> (O) { O(i) = 0 where i in 0:4\n O(i) += int32(A(i) * 1.5) }",
+                 "def f(float(N) A) -> (O) { O(i) = 0.0 where i in 0:4\n O(i) += A(i) * 1.5 }"):
+        tc.map_only(good, "f", [F(4)], "naive")
+        tc_oracle.infer_output_shapes(good, "f", [(4,)])
