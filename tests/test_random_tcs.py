@@ -23,3 +23,35 @@ def test_front_end_and_mapper_accept_what_the_oracle_accepts():
             tc.compile(src, entry, shapes, options)     # hipRTC accepts the generated source
             compiled += 1
     assert compiled == 6
+
+
+def test_front_end_rejects_what_the_oracle_rejects():
+    """Draws the oracle's range inference refuses (unsolved or empty ranges, mostly) are refused by
+    the C++ front end as well: acceptance agrees in both directions."""
+    from oracle import tc_oracle
+    rejected = []
+    original = tc_oracle.infer_output_shapes
+
+    def spy(src, name, shapes):
+        try:
+            return original(src, name, shapes)
+        except tc_oracle.TcError:
+            rejected.append((src, name, shapes))
+            raise
+
+    random_tcs.tc_oracle.infer_output_shapes = spy
+    try:
+        rng = random.Random(13)
+        n = 0
+        while len(rejected) < 150:
+            n += 1
+            random_tcs.generate(rng, f"g{n}")
+    finally:
+        random_tcs.tc_oracle.infer_output_shapes = original
+    for src, name, shapes in rejected:
+        dtype = "float64" if "double(" in src else "float32"
+        try:
+            tc.infer_output_tensor_info(src, name, [tc.ShapeOnly(s, dtype) for s in shapes])
+        except tc.TcError:
+            continue
+        raise AssertionError("accepted although the oracle refuses it:\n" + src)
