@@ -157,7 +157,7 @@ int tc_options_cache_load(
  *   "genetic_search", "seed=..;generations=..;pop_size=.." -> best synthetic cost per generation
  *   "options_cache_selftest", "<scratch file>" -> "ok" or the first failed expectation
  *   "median", "3,1,2,10" -> "2"                                  (tc/core/utils/math.h:23-37)
- *   "tuner_seeds", "<lowest output rank>:<shape>;<shape>..." -> the structured starting points
+ *   "tuner_seeds", "<lowest output rank>[,<innermost output extent>]:<shape>;<shape>..." -> the structured starting points
  *       generation 0 holds next to the base mapping, one option text per line
  *   "sync_placement", "<cyclic 0|1>;<stages>;i:k:level,..." -> "position:level,..." (barriers the
  *       exact placement puts after stage `position` for the given stage-to-stage requirements) */

@@ -285,13 +285,16 @@ extern "C" int tc_host_query(const char* what, const char* arg, char** out) {
           ";block=" + joinSizes(c.blockParams.dims[0].values()) + ";grid=" + joinSizes(c.gridParams.dims[0].values()) +
           ";unroll=" + joinSizes(c.unrollFactor.values()) + ";genes=" + std::to_string(c.collectParameters().size());
     } else if (w == "tuner_seeds") {
-      // "rank:shapes": smallest output rank, then shapes as for search_space -> the structured
+      // "rank[,innermost output extent]:shapes", shapes as for search_space -> the structured
       // starting points the search space accepts (one option text per line), as generation 0
       // would hold them next to the naive options
       std::vector<std::vector<int64_t>> shapes;
       size_t colon = a.find(':');
       TC_CHECK(colon != std::string::npos) << "expected <smallest output rank>:<shapes>";
-      size_t smallestOutputRank = std::stoul(a.substr(0, colon));
+      std::string head = a.substr(0, colon);
+      size_t comma = head.find(',');
+      size_t smallestOutputRank = std::stoul(head.substr(0, comma));
+      size_t innermostOutputExtent = comma == std::string::npos ? 0 : std::stoul(head.substr(comma + 1));
       std::stringstream ss(a.substr(colon + 1));
       std::string sh;
       while (std::getline(ss, sh, ';')) {
@@ -308,8 +311,10 @@ extern "C" int tc_host_query(const char* what, const char* arg, char** out) {
         ptrs.push_back(&ts[i]);
       }
       HipMappingOptions naive = HipMappingOptions::makeNaiveMappingOptions();
-      TuningConfiguration space = tc::autotune::detail::setupTuningParameters(ptrs, {naive}, 256);
-      for (const auto& seed : tc::autotune::detail::heuristicSeeds(naive, ptrs, smallestOutputRank)) {
+      std::vector<size_t> outputSizes;
+      if (innermostOutputExtent > 0) outputSizes.push_back(innermostOutputExtent);
+      TuningConfiguration space = tc::autotune::detail::setupTuningParameters(ptrs, {naive}, 256, outputSizes);
+      for (const auto& seed : tc::autotune::detail::heuristicSeeds(naive, ptrs, smallestOutputRank, innermostOutputExtent)) {
         try {
           TuningConfiguration c = space;
           c.fromHipMappingOptions(seed);

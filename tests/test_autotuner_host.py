@@ -82,3 +82,14 @@ def test_structured_seeds_are_members_of_the_search_space():
     # row reductions: one row per block (tile 1 on each dimension of the lowest-rank output), the
     # reduction dimension whole, a grid limit that covers all rows
     assert sum(";tile=1,0;" in r and "matchLibraryCalls=1" in r and "mapToBlocks=32768,256" in r for r in rows) == 2
+
+
+def test_window_seeds_for_convolutions():
+    """Outputs of rank three or more with an innermost extent of 8..256 also get the window seeds:
+    one image per block, input window in LDS, the innermost output extent along threadIdx.x and a
+    power of two of rows along threadIdx.y (group convolution at the benchmark's size: 54 x 16)."""
+    seeds = tc.host_query("tuner_seeds", "5,54:32x32x4x56x56;32x4x4x3x3;32x4").split("\n")
+    windows = [s for s in seeds if "mapToThreads=54,16" in s]
+    assert len(windows) == 2
+    assert all(";tile=1,1,0,0,0;" in s and "useSharedMemory=1" in s and "collapseContiguous=0" in s for s in windows)
+    assert not any("mapToThreads=54" in s for s in tc.host_query("tuner_seeds", "1,54:1024x54").split("\n"))
