@@ -100,3 +100,16 @@ def test_every_case_maps_and_compiles_for_gfx950(name, options):
     shapes = [tc.ShapeOnly(a.shape, str(a.dtype)) for a in B.make_inputs(name)]
     ex = tc.compile(src, entry, shapes, OPTION_SETS[options])
     assert ex.num_kernels >= 1 and "__global__" in ex.compiled_source
+
+
+@pytest.mark.parametrize("name", sorted(B.TUNED_AT_REFERENCE_SIZES))
+def test_tuned_options_compile_at_the_reference_sizes(name):
+    """The stored options map and compile (hipRTC, gfx950) at the reference's default sizes: the
+    thread block fits the device, LDS stays within 160 KB, every kernel has a launch."""
+    src, entry, _, _ = B.CASES[name]
+    shapes = [tc.ShapeOnly(s[1], "int32") if isinstance(s[0], str) else tc.ShapeOnly(s) for s in B.REFERENCE_SIZES[name]]
+    ex = tc.compile(src, entry, shapes, B.TUNED_AT_REFERENCE_SIZES[name])
+    assert ex.num_kernels >= 1 and ex.lds_bytes() <= 160 * 1024
+    for k in range(ex.num_kernels):
+        grid, block = ex.launch_bounds(k)
+        assert 1 <= block[0] * block[1] * block[2] <= 1024 and min(grid) >= 1

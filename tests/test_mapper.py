@@ -263,3 +263,19 @@ def test_a_later_rewrite_of_a_tensor_joins_the_kernel_of_its_producer():
     assert len(launches) == 1
     body = text[text.index("// stage 1: T"):text.index("// stage 2: S")]
     assert "__syncthreads();" in body
+
+
+def test_tuned_options_of_the_five_workloads_compile_with_the_expected_launches():
+    """The options bench.py uses (tests/workloads.py:TUNED) map to the launch shapes the
+    measurements quote, and hipRTC compiles them for gfx950 without a GPU."""
+    expected = {
+        "c1_tensordot_small": [((16, 8, 1), (425, 1, 1))],
+        "c2_tensordot": [((32, 64, 1), (196, 1, 1))],
+        "c3_batch_matmul": [((500, 1, 1), (64, 4, 1))],
+        "c4_group_convolution": [((32, 32, 1), (64, 4, 1))],
+        "c5_moments": [((1024, 1, 1), (512, 1, 1))],
+    }
+    for name, launches in expected.items():
+        src, entry, shapes = W.CONFIGS[name][0], W.CONFIGS[name][1], W.CONFIGS[name][2]
+        ex = tc.compile(src, entry, [ShapeOnly(s) for s in shapes], W.TUNED[name])
+        assert [ex.launch_bounds(k) for k in range(ex.num_kernels)] == launches, name
