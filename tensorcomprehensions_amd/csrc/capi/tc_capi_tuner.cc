@@ -78,6 +78,9 @@ extern "C" int tc_autotune(
     while (std::getline(bs, line)) {
       if (!line.empty()) bases.push_back(HipMappingOptions::fromText(line));
     }
+    // (tune() refuses host memory and null data before anything is launched; this call orders
+    // that check ahead of the first HIP call, so it also works on a machine without a GPU)
+    HipBackend::checkTensorsAreLaunchable(capi::constTensors(inputs, numInputs), capi::mutTensors(outputs, numOutputs));
     int dev = 0;
     TC_HIP_CHECK(tchip_get_device(&dev));
     std::unordered_map<size_t, std::vector<const DLConstTensor*>> in;

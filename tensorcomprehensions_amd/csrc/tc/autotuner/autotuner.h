@@ -256,6 +256,12 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
     const TunerSettings& settings) {
   TC_CHECK(!inputs.empty()) << "no device to tune on";
   TC_CHECK(!baseMappings.empty()) << "need at least one base mapping";
+  // every candidate is launched on these tensors
+  for (const auto& in : inputs) {
+    auto out = outputs.find(in.first);
+    TC_CHECK(out != outputs.end()) << "no outputs for device " << in.first;
+    Backend::checkTensorsAreLaunchable(in.second, out->second, static_cast<int>(in.first));
+  }
   auto defs = tc::detail::parse(tc);
   TC_CHECK_EQ(defs.count(tcEntryPoint), 1u) << "attempting to access undefined function " << tcEntryPoint;
   lang::TreeRef tree = defs.at(tcEntryPoint);

@@ -49,6 +49,12 @@ struct HipBackend {
   static std::string backendString() { return HipGPUInfo::GPUInfo().GetGPUName(); }
   static std::string makeDeviceFilename(const std::string& fn) { return fn + ".hip"; }
 
+  // Throws unless every tensor holds non-null memory of HIP device `device` (-1: the current
+  // device).  The device-type and null tests come first and touch no HIP call, so host tensors
+  // are refused on a machine without a GPU as well.
+  static void checkTensorsAreLaunchable(
+      const std::vector<const DLConstTensor*>& inputs, const std::vector<const DLTensor*>& outputs, int device = -1);
+
   static CompilationResultType compileWithTcMapper(
       const std::string& tcName,
       const ir::Function& function,

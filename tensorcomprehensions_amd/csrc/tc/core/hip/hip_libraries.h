@@ -55,35 +55,46 @@ template <typename T> struct OpProd { static __device__ __forceinline__ T apply(
 template <typename T> struct OpMin  { static __device__ __forceinline__ T apply(T a, T b) { return tmin(a, b); } };
 template <typename T> struct OpMax  { static __device__ __forceinline__ T apply(T a, T b) { return tmax(a, b); } };
 
-// lane exchange through the DPP network (no LDS traffic); CTRL is a GFX9 dpp_ctrl code
-template <int CTRL> __device__ __forceinline__ int dppMov(int v) {
+// lane exchange through the DPP network (no LDS traffic); CTRL is a GFX9 dpp_ctrl code.  Any
+// arithmetic type of up to 64 bits: 64-bit values move as two 32-bit halves, narrower ones
+// widened to one.
+template <int CTRL> __device__ __forceinline__ int dppMov32(int v) {
   return __builtin_amdgcn_update_dpp(v, v, CTRL, 0xf, 0xf, false);
 }
-template <int CTRL> __device__ __forceinline__ float dppMov(float v) {
-  return __int_as_float(dppMov<CTRL>(__float_as_int(v)));
+template <int CTRL, typename T> __device__ __forceinline__ T dppMov(T v) {
+  static_assert(sizeof(T) <= 8, "lane exchange of at most 64 bits");
+  if constexpr (sizeof(T) == 8) {
+    const unsigned long long b = __builtin_bit_cast(unsigned long long, v);
+    const unsigned lo = (unsigned)dppMov32<CTRL>((int)(unsigned)(b & 0xffffffffULL));
+    const unsigned hi = (unsigned)dppMov32<CTRL>((int)(unsigned)(b >> 32));
+    return __builtin_bit_cast(T, ((unsigned long long)hi << 32) | lo);
+  } else if constexpr (sizeof(T) == 4) {
+    return __builtin_bit_cast(T, dppMov32<CTRL>(__builtin_bit_cast(int, v)));
+  } else {
+    return (T)dppMov32<CTRL>((int)v);
+  }
 }
-template <int CTRL> __device__ __forceinline__ unsigned dppMov(unsigned v) { return (unsigned)dppMov<CTRL>((int)v); }
-template <int CTRL> __device__ __forceinline__ double dppMov(double v) {
-  long long b = __double_as_longlong(v);
-  int lo = dppMov<CTRL>((int)(b & 0xffffffffLL)), hi = dppMov<CTRL>((int)(b >> 32));
-  return __longlong_as_double(((long long)hi << 32) | (unsigned)lo);
+// exchange with lane ^ MASK across the 16-lane rows of a wavefront
+template <int MASK, typename T> __device__ __forceinline__ T laneXor(T v) {
+  if constexpr (sizeof(T) == 8) {
+    return __builtin_bit_cast(T, __shfl_xor(__builtin_bit_cast(unsigned long long, v), MASK, 64));
+  } else if constexpr (sizeof(T) == 4) {
+    return __builtin_bit_cast(T, __shfl_xor(__builtin_bit_cast(int, v), MASK, 64));
+  } else {
+    return (T)__shfl_xor((int)v, MASK, 64);
+  }
 }
-template <int CTRL> __device__ __forceinline__ long long dppMov(long long b) {
-  int lo = dppMov<CTRL>((int)(b & 0xffffffffLL)), hi = dppMov<CTRL>((int)(b >> 32));
-  return ((long long)hi << 32) | (unsigned)lo;
-}
-template <typename T> __device__ __forceinline__ T laneRead(T v, int lane) { return __shfl(v, lane, 64); }
 
 // 0xB1 = quad_perm[1,0,3,2] (lane^1), 0x4E = quad_perm[2,3,0,1] (lane^2),
 // 0x141 = row_half_mirror (i <-> 7-i), 0x140 = row_mirror (i <-> 15-i).
 template <typename Op, int WIDTH, typename T> __device__ __forceinline__ T waveAllReduce(T v) {
   static_assert(WIDTH >= 1 && WIDTH <= 64 && (WIDTH & (WIDTH - 1)) == 0, "power of two up to 64");
-  if (WIDTH >= 2) v = Op::apply(v, dppMov<0xB1>(v));
-  if (WIDTH >= 4) v = Op::apply(v, dppMov<0x4E>(v));
-  if (WIDTH >= 8) v = Op::apply(v, dppMov<0x141>(v));
-  if (WIDTH >= 16) v = Op::apply(v, dppMov<0x140>(v));
-  if (WIDTH >= 32) v = Op::apply(v, __shfl_xor(v, 16, 64));
-  if (WIDTH >= 64) v = Op::apply(v, __shfl_xor(v, 32, 64));
+  if constexpr (WIDTH >= 2) v = Op::apply(v, dppMov<0xB1>(v));
+  if constexpr (WIDTH >= 4) v = Op::apply(v, dppMov<0x4E>(v));
+  if constexpr (WIDTH >= 8) v = Op::apply(v, dppMov<0x141>(v));
+  if constexpr (WIDTH >= 16) v = Op::apply(v, dppMov<0x140>(v));
+  if constexpr (WIDTH >= 32) v = Op::apply(v, laneXor<16>(v));
+  if constexpr (WIDTH >= 64) v = Op::apply(v, laneXor<32>(v));
   return v;
 }
 
@@ -104,17 +115,15 @@ __device__ __forceinline__ void settle(unsigned long long& v) { asm volatile("" 
 
 template <typename Op, int BX, int BY, int BZ, typename T>
 __device__ __forceinline__ T blockAllReduceX(T v, T* scratch) {
-  if (BX == 1) {
+  if constexpr (BX == 1) {
     return v;
-  }
-  if ((BX & (BX - 1)) == 0 && BX <= 64) {
+  } else if constexpr ((BX & (BX - 1)) == 0 && BX <= 64) {
     // a row of BX threads is an aligned lane group of one wavefront
     // (linear thread id = x + BX * (y + BY * z), BX divides 64)
-    return waveAllReduce<Op, (((BX & (BX - 1)) == 0 && BX <= 64) ? BX : 1)>(v);
-  }
-  const int row = threadIdx.y + BY * threadIdx.z;
-  if (BX % 64 == 0) {
+    return waveAllReduce<Op, BX>(v);
+  } else if constexpr (BX % 64 == 0) {
     // every wavefront lies inside one row: wave reduce, then combine BX/64 partials through LDS
+    const int row = threadIdx.y + BY * threadIdx.z;
     constexpr int W = BX / 64;
     v = waveAllReduce<Op, 64>(v);
     __syncthreads();
@@ -125,16 +134,18 @@ __device__ __forceinline__ T blockAllReduceX(T v, T* scratch) {
     for (int w = 1; w < W; ++w) r = Op::apply(r, scratch[row * W + w]);
     settle(r);
     return r;
-  }
-  // any other row width: rows straddle wavefronts, go through LDS
-  __syncthreads();
-  scratch[row * BX + threadIdx.x] = v;
-  __syncthreads();
-  T r = scratch[row * BX];
+  } else {
+    // any other row width: rows straddle wavefronts, go through LDS
+    const int row = threadIdx.y + BY * threadIdx.z;
+    __syncthreads();
+    scratch[row * BX + threadIdx.x] = v;
+    __syncthreads();
+    T r = scratch[row * BX];
 #pragma unroll 8
-  for (int x = 1; x < BX; ++x) r = Op::apply(r, scratch[row * BX + x]);
-  settle(r);
-  return r;
+    for (int x = 1; x < BX; ++x) r = Op::apply(r, scratch[row * BX + x]);
+    settle(r);
+    return r;
+  }
 }
 } // namespace __tc
 )HIP";

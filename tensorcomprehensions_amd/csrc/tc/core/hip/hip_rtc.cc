@@ -8,6 +8,23 @@
 
 namespace tc {
 
+namespace {
+// A pair of timing events that is destroyed on every way out of a launch, an exception thrown
+// by a failed driver call included (the tuner catches those and carries on with the next
+// candidate, so a leak per failed candidate would add up over a tuning run).
+struct EventPair {
+  tchip_event_t start = nullptr, stop = nullptr;
+  void create() {
+    TC_HIP_CHECK(tchip_event_create(&start));
+    TC_HIP_CHECK(tchip_event_create(&stop));
+  }
+  ~EventPair() {
+    if (start) tchip_event_destroy(start);
+    if (stop) tchip_event_destroy(stop);
+  }
+};
+} // namespace
+
 HipRTCFunction::~HipRTCFunction() {
   if (!cleared_) {
     try {
@@ -18,6 +35,7 @@ HipRTCFunction::~HipRTCFunction() {
 }
 
 void HipRTCFunction::clear() {
+  std::lock_guard<std::mutex> lock(mutex_);
   if (cleared_) return;
   for (auto& m : modules_) {
     int old = 0;
@@ -63,37 +81,38 @@ Duration HipRTCFunction::Launch(
     std::vector<const void*> inputs,
     bool profile,
     int repeats) const {
-  TC_CHECK(!cleared_) << "launch of a cleared RTC function";
   int dev = 0;
   TC_HIP_CHECK(tchip_get_device(&dev));
-  if (!modules_.count(dev)) {
-    tchip_module_t m = nullptr;
-    TC_HIP_CHECK(tchip_module_load(code_.data(), &m));
-    modules_[dev] = m;
+  std::vector<tchip_function_t> fns;
+  {
+    // the per-device module and function handles are filled in lazily: one thread at a time
+    std::lock_guard<std::mutex> lock(mutex_);
+    TC_CHECK(!cleared_) << "launch of a cleared RTC function";
+    if (!modules_.count(dev)) {
+      tchip_module_t m = nullptr;
+      TC_HIP_CHECK(tchip_module_load(code_.data(), &m));
+      modules_[dev] = m;
+    }
+    for (const auto& k : kernels) {
+      auto key = std::make_pair(dev, k.name);
+      auto it = functions_.find(key);
+      if (it == functions_.end()) {
+        tchip_function_t fn = nullptr;
+        TC_HIP_CHECK(tchip_module_get_function(modules_[dev], k.name.c_str(), &fn));
+        it = functions_.emplace(key, fn).first;
+      }
+      fns.push_back(it->second);
+    }
   }
   std::vector<void*> args;
   for (auto& p : params) args.push_back(&p);
   for (auto& p : outputs) args.push_back(&p);
   for (auto& p : inputs) args.push_back((void*)&p);
   TC_CHECK_LE(args.size(), 100u) << "too many kernel arguments";
-  tchip_event_t start = nullptr, stop = nullptr;
+  EventPair ev;
   if (profile) {
-    TC_HIP_CHECK(tchip_event_create(&start));
-    TC_HIP_CHECK(tchip_event_create(&stop));
-  }
-  std::vector<tchip_function_t> fns;
-  for (const auto& k : kernels) {
-    auto key = std::make_pair(dev, k.name);
-    auto it = functions_.find(key);
-    if (it == functions_.end()) {
-      tchip_function_t fn = nullptr;
-      TC_HIP_CHECK(tchip_module_get_function(modules_[dev], k.name.c_str(), &fn));
-      it = functions_.emplace(key, fn).first;
-    }
-    fns.push_back(it->second);
-  }
-  if (profile) {
-    TC_HIP_CHECK(tchip_event_record(start, stream));
+    ev.create();
+    TC_HIP_CHECK(tchip_event_record(ev.start, stream));
   }
   for (int r = 0; r < repeats; ++r) {
     for (size_t i = 0; i < kernels.size(); ++i) {
@@ -102,11 +121,9 @@ Duration HipRTCFunction::Launch(
   }
   if (profile) {
     float ms = 0;
-    TC_HIP_CHECK(tchip_event_record(stop, stream));
-    TC_HIP_CHECK(tchip_event_sync(stop));
-    TC_HIP_CHECK(tchip_event_elapsed_ms(start, stop, &ms));
-    TC_HIP_CHECK(tchip_event_destroy(start));
-    TC_HIP_CHECK(tchip_event_destroy(stop));
+    TC_HIP_CHECK(tchip_event_record(ev.stop, stream));
+    TC_HIP_CHECK(tchip_event_sync(ev.stop));
+    TC_HIP_CHECK(tchip_event_elapsed_ms(ev.start, ev.stop, &ms));
     return Duration::fromNanoSeconds(static_cast<int64_t>(static_cast<double>(ms) * 1e6 + 0.5));
   }
   return Duration::max();

@@ -6,6 +6,7 @@
 #include <array>
 #include <map>
 #include <memory>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -46,6 +47,7 @@ class HipRTCFunction {
   HipRTCFunction() = default;
   std::string name_;
   std::string code_; // code object
+  mutable std::mutex mutex_;                                                   // guards the two maps
   mutable std::map<int, tchip_module_t> modules_;                              // per device id
   mutable std::map<std::pair<int, std::string>, tchip_function_t> functions_;  // (device, kernel)
   bool cleared_ = false;

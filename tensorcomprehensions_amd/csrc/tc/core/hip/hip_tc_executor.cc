@@ -17,6 +17,35 @@ std::string specializedKernelName(const std::string& tcName, const ir::Function&
 }
 } // namespace
 
+namespace {
+template <typename DLT>
+void checkPlacement(const std::vector<const DLT*>& ts, const char* what, int currentDevice) {
+  for (size_t i = 0; i < ts.size(); ++i) {
+    const DLT* t = ts[i];
+    if (currentDevice < 0) {
+      TC_CHECK(t->ctx.device_type == kDLROCM)
+          << what << " " << i << " is not in HIP device memory (DLPack device type " << static_cast<int>(t->ctx.device_type)
+          << ", expected " << static_cast<int>(kDLROCM) << "): kernels cannot be launched on it";
+      bool empty = false;
+      for (int d = 0; d < t->ndim; ++d) empty |= t->shape[d] == 0;
+      TC_CHECK(t->data != nullptr || empty) << what << " " << i << " has a null data pointer";
+    } else {
+      TC_CHECK_EQ(t->ctx.device_id, currentDevice)
+          << what << " " << i << " lives on device " << t->ctx.device_id << " but the current device is " << currentDevice;
+    }
+  }
+}
+} // namespace
+
+void HipBackend::checkTensorsAreLaunchable(
+    const std::vector<const DLConstTensor*>& inputs, const std::vector<const DLTensor*>& outputs, int dev) {
+  checkPlacement(inputs, "input", -1);
+  checkPlacement(outputs, "output", -1);
+  if (dev < 0) TC_HIP_CHECK(tchip_get_device(&dev));
+  checkPlacement(inputs, "input", dev);
+  checkPlacement(outputs, "output", dev);
+}
+
 HipCompilationResult HipBackend::compileWithTcMapper(
     const std::string& tcName,
     const ir::Function& function,

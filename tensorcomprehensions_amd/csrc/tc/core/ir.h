@@ -35,7 +35,8 @@ struct ScalarType {
     if (isBool()) {
       return "bool";
     }
-    return std::string(code == UInt ? "unsigned " : "") +
+    // (plain `char` has no fixed signedness: int8 is spelled out)
+    return std::string(code == UInt ? "unsigned " : bits == 8 ? "signed " : "") +
         (bits == 8 ? "char" : bits == 16 ? "short" : bits == 32 ? "int" : "long long");
   }
   DLDataType toDL() const {

@@ -73,12 +73,15 @@ class TcExecutor {
 
   // Checked run; the tensors are borrowed for the duration of the call.  May be called
   // repeatedly with different base pointers of identical shapes.  Does not synchronise.
+  // Beyond the reference's checks the backend also refuses tensors a kernel must not be
+  // launched on (host memory, null data, another device): the reference launches on them.
   void run(
       const std::vector<const DLConstTensor*>& inputs,
       const std::vector<const DLTensor*>& outputs,
       typename Backend::RuntimeInformation info = typename Backend::RuntimeInformation()) const {
     detail::checkSizesAndStridesAreCompliant(inputs, inputsInfo_, "input");
     detail::checkSizesAndStridesAreCompliant(outputs, outputsInfo_, "output");
+    Backend::checkTensorsAreLaunchable(inputs, outputs);
     std::vector<const void*> in;
     std::vector<void*> out;
     for (auto t : inputs) in.push_back(static_cast<const char*>(t->data) + t->byte_offset);
@@ -94,6 +97,7 @@ class TcExecutor {
     auto t0 = std::chrono::steady_clock::now();
     detail::checkSizesAndStridesAreCompliant(inputs, inputsInfo_, "input");
     detail::checkSizesAndStridesAreCompliant(outputs, outputsInfo_, "output");
+    Backend::checkTensorsAreLaunchable(inputs, outputs);
     std::vector<const void*> in;
     std::vector<void*> out;
     for (auto t : inputs) in.push_back(static_cast<const char*>(t->data) + t->byte_offset);

@@ -167,3 +167,40 @@ def test_later_statement_cannot_narrow_into_the_tensors_first_type():
                  "def f(float(N) A) -> (O) { O(i) = 0.0 where i in 0:4\n O(i) += A(i) * 1.5 }"):
         tc.map_only(good, "f", [F(4)], "naive")
         tc_oracle.infer_output_shapes(good, "f", [(4,)])
+
+
+# ------------------------------------------------------------------------------------------------
+# tensors a kernel must never be launched on: refused before any launch, so checked without a GPU
+# (the reference launches on whatever pointer it is given, tc/core/tc_executor-inl.h:109-145)
+# ------------------------------------------------------------------------------------------------
+COPY = "def f(float(N) a) -> (b) { b(i) = a(i) }"
+
+
+def _copy_executor():
+    return tc.compile(COPY, "f", [F(8)], "naive")
+
+
+@pytest.mark.parametrize("entry", ["run", "profile", "call", "autotune"])
+def test_host_tensors_are_refused_before_any_launch(entry):
+    ex = _copy_executor()
+    a, b = torch.zeros(8), torch.zeros(8)
+    with pytest.raises(tc.TcError) as e:
+        if entry == "run":
+            tc.run(ex, [a], [b])
+        elif entry == "profile":
+            tc.profile(ex, [a], [b])
+        elif entry == "call":
+            ex(a)
+        else:
+            tc.autotune(COPY, "f", [a], "naive", outputs=[b], generations=1, pop_size=2)
+    assert "not in HIP device memory" in str(e.value), str(e.value)
+
+
+def test_null_data_pointers_are_refused_before_any_launch():
+    ex = _copy_executor()
+    with pytest.raises(tc.TcError) as e:
+        tc.run(ex, [F(8)], [F(8)])
+    assert "null data pointer" in str(e.value), str(e.value)
+    with pytest.raises(tc.TcError) as e:
+        tc.autotune(COPY, "f", [F(8)], "naive", outputs=[F(8)], generations=1, pop_size=2)
+    assert "null data pointer" in str(e.value), str(e.value)
