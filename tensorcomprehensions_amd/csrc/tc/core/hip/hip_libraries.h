@@ -30,6 +30,21 @@ template <typename T> __device__ __forceinline__ T floordiv(T n, T d) {
   return ((n % d != 0) && ((n < 0) != (d < 0))) ? q - 1 : q;
 }
 template <typename T> __device__ __forceinline__ T floormod(T n, T d) { return n - floordiv(n, d) * d; }
+// Store of element `index` of the tensor behind buffer descriptor `rs` with device-scope
+// write-through (cache policy sc1 = 16): the value goes on to memory instead of staying dirty in
+// the L2 until the end of the kernel.  An offset past the end of the buffer is dropped.
+template <typename T> __device__ __forceinline__ void storeThrough(__amdgpu_buffer_rsrc_t rs, int index, T v) {
+  typedef unsigned uintx2 __attribute__((ext_vector_type(2)));
+  if constexpr (sizeof(T) == 8) {
+    __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(uintx2, v), rs, index * 8, 0, 16);
+  } else if constexpr (sizeof(T) == 4) {
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), rs, index * 4, 0, 16);
+  } else if constexpr (sizeof(T) == 2) {
+    __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(unsigned short, v), rs, index * 2, 0, 16);
+  } else {
+    __builtin_amdgcn_raw_buffer_store_b8(__builtin_bit_cast(unsigned char, v), rs, index, 0, 16);
+  }
+}
 template <typename T> __device__ __forceinline__ T tmin(T a, T b) { return a < b ? a : b; }
 template <typename T> __device__ __forceinline__ T tmax(T a, T b) { return a > b ? a : b; }
 __device__ __forceinline__ float tmin(float a, float b) { return fminf(a, b); }

@@ -477,6 +477,18 @@ void emitKernel(KernelCtx& kc, const DeviceLimits& limits, Emitter& em) {
   em.line("const int tid_ = threadIdx.x + " + std::to_string(k.block[0]) + " * (threadIdx.y + " +
           std::to_string(k.block[1]) + " * threadIdx.z);");
   em.line("(void)tid_;");
+  {
+    // buffer descriptors (base, size in bytes, raw 32-bit data format) of the results that are
+    // stored with write-through
+    std::set<std::string> through;
+    for (size_t i = 0; i < gens.size(); ++i) {
+      if (gens[i].streamedStore()) through.insert(k.stages[i].tensor);
+    }
+    for (const auto& t : through) {
+      em.line("const __amdgpu_buffer_rsrc_t " + StageCodegen::bufferName(t) + " = __builtin_amdgcn_make_buffer_rsrc((void*)p" +
+              t + ", 0, " + std::to_string(gens[0].viewBytes(t)) + ", 0x00020000);");
+    }
+  }
   if (scratchElems > 0) {
     // one scratch area typed per use; sized for the widest element
     em.line("__shared__ double red_scratch_raw_[" + std::to_string(scratchElems) + "];");
@@ -496,6 +508,7 @@ void emitKernel(KernelCtx& kc, const DeviceLimits& limits, Emitter& em) {
       loops.push_back(&v);
     }
   }
+  kc.kernelLoops = !loops.empty();
   auto loopHeader = [&](const LoopVar& v, std::string& start, std::string& step) {
     start = v.blockAxis >= 0 ? std::string("blockIdx.") + axisName(v.blockAxis) : "0";
     step = v.blockAxis >= 0 ? std::to_string(v.gridExtent) : "1";

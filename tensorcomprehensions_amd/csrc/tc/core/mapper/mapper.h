@@ -59,7 +59,7 @@ struct Promotion {
   std::string tensor;
   std::string ldsName;
   std::vector<int64_t> extents;      // footprint box, per view dimension
-  std::vector<int64_t> ldsStrides;   // row-major with optional padding of the last extent
+  std::vector<int64_t> ldsStrides;   // row-major, pitches padded against bank conflicts
   int64_t elems = 0;                 // LDS elements including padding
   int64_t reuse = 1;                 // accesses per staged element
   bool insideReductionTiles = false;

@@ -37,6 +37,7 @@ struct KernelCtx {
   const HipMappingOptions& opts;
   KernelPlan& k;
   std::string idx = "int"; // index arithmetic type
+  bool kernelLoops = false; // the stages sit inside loops over tiles that the blocks share out
   int64_t NT() const { return k.block[0] * k.block[1] * k.block[2]; }
 };
 
@@ -163,20 +164,27 @@ class StageCodegen {
     return true;
   }
 
-  // The stage's result when nothing later in this kernel reads it back and it is too large to be
-  // found in cache by a later kernel: stores of it carry the non-temporal hint.
+  // The stage's result when nothing later in this kernel reads it back: it is stored with
+  // device-scope write-through (buffer stores with the sc1 bit).  A plain or non-temporal store
+  // leaves the line dirty in the L2 of its XCD, and everything still dirty when the last wavefront
+  // ends is written back before the kernel completes: a result of a few MB then adds its whole
+  // write-back time to the kernel (12.8 MB: 2.4 us) instead of overlapping it with the computation.
+  // Byte offsets of a buffer access are 32 bits wide, which bounds the tensors this applies to.
   bool streamedStore() const {
-    if (!kc_.opts.useReadOnlyCacheValue || viewBytes(st_.tensor) < kStreamingBytes) return false;
+    if (!kc_.opts.useReadOnlyCacheValue || viewBytes(st_.tensor) >= (int64_t(1) << 31)) return false;
     for (size_t j = stageIdx_ + 1; j < kc_.k.stages.size(); ++j) {
       if (tensorsRead(kc_.k.stages[j]).count(st_.tensor)) return false;
     }
     return true;
   }
+  static std::string bufferName(const std::string& tensor) { return "rs" + tensor + "_"; }
 
   std::string storeStmt(const std::string& cond, const std::string& value) {
-    std::string target = "p" + st_.tensor + "[" + flatIndex(st_.tensor, st_.lhsSubs, "") + "]";
-    if (streamedStore()) return "if (" + cond + ") __builtin_nontemporal_store(" + value + ", &" + target + ");";
-    return "if (" + cond + ") " + target + " = " + value + ";";
+    std::string index = flatIndex(st_.tensor, st_.lhsSubs, "");
+    if (streamedStore()) {
+      return "if (" + cond + ") __tc::storeThrough(" + bufferName(st_.tensor) + ", " + index + ", " + value + ");";
+    }
+    return "if (" + cond + ") p" + st_.tensor + "[" + index + "] = " + value + ";";
   }
 
   std::string loadStr(const ExprRef& e, const std::string& accRef) {
@@ -361,12 +369,11 @@ class StageCodegen {
       int64_t bytes;
     };
     std::vector<Cand> cands;
-    std::string residentOperand;
-    if (mfmaKeepsMOperandInRegisters()) {
-      residentOperand = s.rhs->args[st_.mfmaSwapOperands ? 1 : 0]->name; // read once per wavefront
-    }
+    // (An M-side operand that the wavefronts keep in registers is staged as well: every wavefront
+    // of the block needs all of it, a lane's share is one row, so reading it straight from global
+    // memory costs one cache line per lane and load where the cooperative copy moves whole lines.)
     for (const auto& acc : accesses) {
-      if (bad.count(acc.first) || acc.first == residentOperand) continue;
+      if (bad.count(acc.first)) continue;
       const TensorView& view = st_.views.at(acc.first);
       if (view.isOutput) continue; // may be written by another stage of this kernel
       const auto& ref = acc.second.front();
@@ -404,28 +411,66 @@ class StageCodegen {
       }
       c.p.reuse = static_cast<int64_t>(iterations * acc.second.size() / static_cast<double>(elems));
       if (c.p.reuse < 2) continue;
-      // pad the innermost extent to an odd size when lanes walk a slower dimension
-      std::vector<int64_t> padded = c.p.extents;
-      if (!padded.empty() && padded.back() > 1 && padded.back() % 2 == 0 && lanesWalkOuterDim(ref)) {
-        padded.back() += 1;
-      }
-      // Matrix-core operands: the 16 lanes of a group walk the M- (or N-) side variable.  When that
-      // variable is not in the last subscript, consecutive lanes are a whole row apart and a row
-      // length that is a multiple of 8 elements piles them onto few LDS banks: four elements of
-      // padding spread 16 rows over 8 banks groups while rows stay 16-byte aligned for the copies.
-      if (st_.mfma && ref.size() >= 2 && padded.back() % 8 == 0 && kMfmaPad > 0) {
-        bool isA = acc.first == s.rhs->args[st_.mfmaSwapOperands ? 1 : 0]->name;
+      // Pitches.  pad[j] = elements added to the distance between consecutive indices of dimension j.
+      const size_t nd = ref.size();
+      std::vector<int64_t> pad(nd, 0);
+      auto stridesWith = [&](const std::vector<int64_t>& pd) {
+        std::vector<int64_t> str(nd, 1);
+        for (size_t j = nd - 1; j-- > 0;) str[j] = str[j + 1] * c.p.extents[j + 1] + pd[j];
+        return str;
+      };
+      // lanes that walk a slower dimension: an odd row length spreads them over the banks
+      if (nd >= 2 && c.p.extents.back() > 1 && c.p.extents.back() % 2 == 0 && lanesWalkOuterDim(ref)) pad[nd - 2] += 1;
+      if (st_.mfma && nd >= 2 && kMfmaPad > 0) {
+        const bool isA = acc.first == s.rhs->args[st_.mfmaSwapOperands ? 1 : 0]->name;
+        // The 16 lanes of a group walk the M- (or N-) side variable.  When that variable is not in
+        // the last subscript, consecutive lanes are a whole pitch apart and a pitch that is a
+        // multiple of 8 elements piles them onto few LDS banks: four elements of padding spread 16
+        // rows over 8 bank groups while rows stay 16-byte aligned for the copies.
         const auto& side = isA ? st_.mfmaM : st_.mfmaN;
-        bool inLast = false, elsewhere = false;
-        for (const auto& n : side) {
-          inLast |= ref.back().coefOf(n) != 0;
-          for (size_t j = 0; j + 1 < ref.size(); ++j) elsewhere |= ref[j].coefOf(n) != 0;
+        int sideDim = -1;
+        for (size_t j = 0; j < nd; ++j) {
+          for (const auto& n : side) {
+            if (ref[j].coefOf(n) != 0) sideDim = static_cast<int>(j);
+          }
         }
-        if (elsewhere && !inLast) padded.back() += kMfmaPad;
+        if (sideDim >= 0 && sideDim + 1 < static_cast<int>(nd) && stridesWith(pad)[sideDim] % 8 == 0) pad[sideDim] += kMfmaPad;
+        // The four lane groups of a wavefront own consecutive quarters of the flattened reduction:
+        // at every step their addresses differ by the same number of elements, and when that is a
+        // multiple of the 32 banks the groups of each half of the wavefront collide.  Padding the
+        // pitch of the outermost reduction variable's dimension moves the groups apart.
+        int64_t KT = 1, innerProd = 1;
+        for (size_t i = 0; i < st_.mfmaK.size(); ++i) {
+          int64_t t = spanOf(var(st_.mfmaK[i]), inside);
+          KT *= t;
+          if (i > 0) innerProd *= t;
+        }
+        const int64_t quarter = ceilDiv(KT, 4);
+        int kDim = -1;
+        for (size_t j = 0; j < nd; ++j) {
+          if (ref[j].coefOf(st_.mfmaK[0]) != 0) kDim = static_cast<int>(j);
+        }
+        if (quarter % innerProd == 0 && kDim >= 0 && kDim + 1 < static_cast<int>(nd)) {
+          auto groupStride = [&](const std::vector<int64_t>& pd) {
+            auto str = stridesWith(pd);
+            int64_t g = 0;
+            for (size_t j = 0; j < nd; ++j) g += ref[j].coefOf(st_.mfmaK[0]) * str[j];
+            return g * (quarter / innerProd);
+          };
+          if (groupStride(pad) % 32 == 0) {
+            for (int64_t extra = kMfmaPad; extra <= 3 * kMfmaPad; extra += kMfmaPad) {
+              std::vector<int64_t> trial = pad;
+              trial[kDim] += extra;
+              if (groupStride(trial) % 32 != 0) {
+                pad = trial;
+                break;
+              }
+            }
+          }
+        }
       }
-      c.p.ldsStrides = makeStridesFromSizes(padded);
-      c.p.elems = 1;
-      for (auto e : padded) c.p.elems *= e;
+      c.p.ldsStrides = stridesWith(pad);
+      c.p.elems = nd == 0 ? 1 : c.p.ldsStrides[0] * c.p.extents[0];
       c.bytes = c.p.elems * view.type.bytes();
       cands.push_back(c);
     }
@@ -635,6 +680,23 @@ class StageCodegen {
     em_.close();
   }
 
+  // Stages several footprints at once: the global loads of all of them are issued before the
+  // first LDS store, so that their latencies overlap, when a thread's share fits in registers.
+  void emitCopyInGroup(const std::vector<const Promotion*>& ps) {
+    int64_t regs = 0;
+    for (const auto* p : ps) regs += copyRegisters(*p);
+    if (ps.size() < 2 || regs > (kc_.opts.unrollCopySharedValue ? 64 : 32)) {
+      for (const auto* p : ps) emitCopyIn(*p);
+      return;
+    }
+    for (const auto* p : ps) declareLows(*p);
+    em_.open("");
+    for (const auto* p : ps) em_.line(copyRegisterDecl(*p, "stage_" + p->tensor + "_"));
+    for (const auto* p : ps) emitCopyLoads(*p, "stage_" + p->tensor + "_");
+    for (const auto* p : ps) emitCopyStores(*p, "stage_" + p->tensor + "_");
+    em_.close();
+  }
+
   // --- loops ----------------------------------------------------------------------------------
   // Opens the per-thread point loop of `v` (uniform trip count across the block), declares
   // i_<v> and returns the predicate term this variable contributes ("" when always valid).
@@ -770,12 +832,14 @@ class StageCodegen {
         return;
       }
       em_.line("__syncthreads();");
+      std::vector<const Promotion*> group;
       for (const auto& p : st_.promotions) {
         if (p.insideReductionTiles == inside) {
-          emitCopyIn(p);
+          group.push_back(&p);
           activePromotions_.insert(p.tensor);
         }
       }
+      emitCopyInGroup(group);
       em_.line("__syncthreads();");
     };
     int opened = 0;
@@ -1186,8 +1250,11 @@ class StageCodegen {
       return masked ? "(kok_ ? " + text + " : 0.0f)" : text;
     };
     const bool resident = mfmaKeepsMOperandInRegisters();
-    if (resident) {
-      em_.line("float am_[" + std::to_string(ksteps) + "];");
+    bool residentFromLds = false;
+    for (const auto& p : st_.promotions) residentFromLds |= resident && p.tensor == loadA->name;
+    if (resident) em_.line("float am_[" + std::to_string(ksteps) + "];");
+    // fills am_: a lane's M-side operand values, one per reduction step
+    auto fillResident = [&]() {
       em_.open("");
       em_.line("const int mt_ = 0, bt_ = 0;");
       em_.line("(void)mt_; (void)bt_;");
@@ -1196,7 +1263,7 @@ class StageCodegen {
       decodeGroup(st_.mfmaM, "mposa_", true);
       // consecutive steps of a lane read consecutive elements when the operand's reduction
       // subscripts are jointly contiguous: four steps are then fetched with one 16-byte load
-      bool contiguous = aligned && quarter * 4 == KT && ksteps % 4 == 0;
+      bool contiguous = !residentFromLds && aligned && quarter * 4 == KT && ksteps % 4 == 0;
       {
         Affine fa = flatAffine(loadA->name, loadA->args);
         contiguous &= fa.valid;
@@ -1233,7 +1300,8 @@ class StageCodegen {
         em_.close();
       }
       em_.close();
-    }
+    };
+    if (resident && !residentFromLds) fillResident();
     // Epilogue operands that do not depend on the column (a bias per output row, say) are the
     // same for every tile of the wavefront: fetched once, ahead of the tile loop.
     hoistedLoads_.clear();
@@ -1290,12 +1358,15 @@ class StageCodegen {
         }
         return;
       }
-      em_.line("__syncthreads();");
+      // (nothing has touched LDS before the first stage of a kernel without kernel-level loops)
+      if (inside || stageIdx_ > 0 || kc_.kernelLoops || stageTileLoops_) em_.line("__syncthreads();");
+      std::vector<const Promotion*> group;
       for (const auto& p : st_.promotions) {
         if (p.insideReductionTiles != inside) continue;
-        emitCopyIn(p);
+        group.push_back(&p);
         activePromotions_.insert(p.tensor);
       }
+      emitCopyInGroup(group);
       em_.line("__syncthreads();");
     };
     // decodes the output tile tl_ of this wavefront: batch and column indices, nok_
@@ -1377,10 +1448,22 @@ class StageCodegen {
     em_.open("");
     ++opened;
     stagePromotions(false);
+    if (resident && residentFromLds) fillResident();
     if (!kTiled) {
       em_.line(waveRotation);
-      em_.open("for (int tl_ = wv_; tl_ < " + std::to_string(tiles) + "; tl_ += " + std::to_string(st_.waves) + ")");
-      ++opened;
+      if (tilesPerWave <= 8) {
+        // few tiles per wavefront: unrolled, so that the operand reads of a tile can be scheduled
+        // above the epilogue and the stores of the tile before it
+        em_.line("#pragma unroll");
+        em_.open("for (int j_ = 0; j_ < " + std::to_string(tilesPerWave) + "; ++j_)");
+        ++opened;
+        em_.line("const int tl_ = wv_ + j_ * " + std::to_string(st_.waves) + ";");
+        em_.open("if (tl_ < " + std::to_string(tiles) + ")");
+        ++opened;
+      } else {
+        em_.open("for (int tl_ = wv_; tl_ < " + std::to_string(tiles) + "; tl_ += " + std::to_string(st_.waves) + ")");
+        ++opened;
+      }
       decodeTile();
       em_.line("__tc::floatx4 c_ = {0.0f, 0.0f, 0.0f, 0.0f};");
       if (!s.init) loadExisting("c_");
@@ -1497,6 +1580,7 @@ class StageCodegen {
           ++openedTiles;
         }
       }
+      stageTileLoops_ = openedTiles > 1;
       emitMfma();
       closeN(openedTiles);
       return;
@@ -1569,6 +1653,7 @@ class StageCodegen {
   std::set<std::string> activePromotions_;
   std::map<std::string, std::string> hoistedLoads_; // printed global load -> register holding it
   bool inCachedReduction_ = false;
+  bool stageTileLoops_ = false; // the stage's code sits inside tile loops of its own
   std::string cacheSlot_;
   int clampId_ = 0;
 };
