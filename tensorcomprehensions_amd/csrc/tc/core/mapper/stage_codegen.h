@@ -524,6 +524,7 @@ class StageCodegen {
     int64_t extent, tensorExtent, gStride, lStride;
     std::string lo;
     int64_t loGcd; // every value of `lo` is a multiple of this (0: lo is always 0)
+    bool inside;   // the footprint never leaves the tensor in this dimension: no bounds test
   };
   struct CopyPlan {
     std::vector<CopyDim> dims;
@@ -558,6 +559,26 @@ class StageCodegen {
     return g;
   }
 
+  // Whether the footprint stays inside the tensor in view dimension j for every tile: the lowest
+  // and highest values footprintLow(p, j) can take, from the same terms.
+  bool footprintAlwaysInside(const Promotion& p, size_t j) const {
+    const Footprint& fp = footprints_.at(p.tensor);
+    int64_t lo = fp.minConst[j], hi = fp.minConst[j];
+    for (const auto& c : fp.coefs[j].coef) {
+      const LoopVar& v = var(c.first);
+      bool fixed = (v.reduction && !p.insideReductionTiles) || v.numTiles == 1;
+      int64_t vlo = v.min, vhi = fixed ? v.min : v.min + (v.numTiles - 1) * v.tile;
+      if (c.second < 0) {
+        vlo += spanOf(v, p.insideReductionTiles) - 1;
+        vhi += spanOf(v, p.insideReductionTiles) - 1;
+      }
+      int64_t a = c.second * vlo, b = c.second * vhi;
+      lo += std::min(a, b);
+      hi += std::max(a, b);
+    }
+    return lo >= 0 && hi + p.extents[j] <= st_.views.at(p.tensor).extents[j];
+  }
+
   CopyPlan copyPlan(const Promotion& p) const {
     const TensorView& view = st_.views.at(p.tensor);
     auto gStridesFull = makeStridesFromSizes(view.extents);
@@ -565,7 +586,7 @@ class StageCodegen {
     for (auto e : p.extents) plan.count *= e;
     for (size_t j = 0; j < p.extents.size(); ++j) {
       plan.dims.push_back(CopyDim{p.extents[j], view.extents[j], gStridesFull[j], p.ldsStrides[j],
-                                  loPrefix(p) + std::to_string(j), footprintLowGcd(p, j)});
+                                  loPrefix(p) + std::to_string(j), footprintLowGcd(p, j), footprintAlwaysInside(p, j)});
     }
     auto& dims = plan.dims;
     while (dims.size() >= 2) {
@@ -577,6 +598,7 @@ class StageCodegen {
       // (out, in) -> one dimension of extent out*in starting at out.lo * in.extent (in.lo is 0)
       out.lo = "(" + out.lo + ") * " + std::to_string(in.extent);
       out.loGcd *= in.extent;
+      out.inside = out.inside && in.inside;
       out.extent *= in.extent;
       out.tensorExtent *= in.tensorExtent;
       out.gStride = in.gStride;
@@ -611,24 +633,42 @@ class StageCodegen {
   // One copy iteration of every thread: the global load of its element (vector) into
   // regs[slot], unconditional and from a clamped address so that loads issue back to back, or
   // the LDS store of regs[slot].
+  // `loopIters`: iterations the enclosing loops run in total (a chunked loop may overshoot
+  // plan.iters).
   void emitCopyStep(const Promotion& p, const CopyPlan& plan, const std::string& itExpr, const std::string& regs,
-                    const std::string& slot, bool loads) {
+                    const std::string& slot, bool loads, int64_t loopIters) {
     const auto& dims = plan.dims;
     std::string unit = "(" + itExpr + ") * " + std::to_string(kc_.NT()) + " + tid_";
     em_.line("const int c_ = " + (plan.vec > 1 ? std::to_string(plan.vec) + " * (" + unit + ")" : unit) + ";");
+    // Only the last iterations can reach past the end of the footprint, and only when the
+    // footprint is not a whole number of the steps the loops make: the test names the iteration, so it
+    // folds away in the unrolled copies of the others.  Threads past the end skip their access
+    // (whole wavefronts of them skip the instruction).
+    const int64_t perIter = kc_.NT() * plan.vec;
+    const int64_t fullIters = plan.count / perIter;
+    const bool ragged = loopIters * perIter > plan.count;
+    const std::string live = ragged ? "(" + itExpr + ") < " + std::to_string(fullIters) + " || c_ < " + std::to_string(plan.count) : "";
     int64_t div = plan.count;
-    std::string cond = "c_ < " + std::to_string(plan.count), gidx, lidx;
+    std::string cond, gidx, lidx;
+    bool outermost = true; // the first dimension with more than one element needs no wrap-around
     for (size_t j = 0; j < dims.size(); ++j) {
       div /= dims[j].extent;
       std::string l = "l" + std::to_string(j) + "_";
-      std::string e = "c_";
-      if (div > 1) e = "(" + e + " / " + std::to_string(div) + ")";
-      if (j > 0) e = e + " % " + std::to_string(dims[j].extent);
-      em_.line("const int " + l + " = " + e + ";");
+      if (dims[j].extent == 1) {
+        em_.line("const int " + l + " = 0;");
+      } else {
+        std::string e = "c_";
+        if (div > 1) e = "(" + e + " / " + std::to_string(div) + ")";
+        if (!outermost) e = e + " % " + std::to_string(dims[j].extent);
+        outermost = false;
+        em_.line("const int " + l + " = " + e + ";");
+      }
       if (loads) {
         std::string g = "g" + std::to_string(j) + "_";
         em_.line("const int " + g + " = " + dims[j].lo + " + " + l + ";");
-        cond += " && (unsigned)" + g + " < " + std::to_string(dims[j].tensorExtent) + "u";
+        if (!dims[j].inside) {
+          cond += (cond.empty() ? "" : " && ") + std::string("(unsigned)") + g + " < " + std::to_string(dims[j].tensorExtent) + "u";
+        }
         gidx += (j ? " + " : "") + g + (dims[j].gStride != 1 ? " * " + std::to_string(dims[j].gStride) : "");
       }
       lidx += (j ? " + " : "") + l + (dims[j].lStride != 1 ? " * " + std::to_string(dims[j].lStride) : "");
@@ -636,10 +676,14 @@ class StageCodegen {
     if (dims.empty()) gidx = lidx = "0";
     std::string cast = plan.vec > 1 ? "*(const __tc::floatx4u*)&" : "";
     std::string lcast = plan.vec > 1 ? "*(__tc::floatx4*)&" : "";
+    std::string guard = live.empty() ? "" : "if (" + live + ") ";
     if (loads) {
-      em_.line(regs + "[" + slot + "] = " + cast + "p" + p.tensor + "[(" + cond + ") ? (" + gidx + ") : 0];");
+      // inside the footprint but outside the tensor (halo of a partial tile): a clamped address,
+      // so that the loads stay unconditional and issue back to back; the value is never used
+      std::string addr = cond.empty() ? gidx : "(" + cond + ") ? (" + gidx + ") : 0";
+      em_.line(guard + regs + "[" + slot + "] = " + cast + "p" + p.tensor + "[" + addr + "];");
     } else {
-      em_.line("if (c_ < " + std::to_string(plan.count) + ") " + lcast + p.ldsName + "[" + lidx + "] = " + regs + "[" + slot + "];");
+      em_.line(guard + lcast + p.ldsName + "[" + lidx + "] = " + regs + "[" + slot + "];");
     }
   }
 
@@ -652,7 +696,7 @@ class StageCodegen {
     CopyPlan plan = copyPlan(p);
     em_.line("#pragma unroll");
     em_.open("for (int it_ = 0; it_ < " + std::to_string(plan.iters) + "; ++it_)");
-    emitCopyStep(p, plan, "it_", regs, "it_", loads);
+    emitCopyStep(p, plan, "it_", regs, "it_", loads, plan.iters);
     em_.close();
   }
 
@@ -674,7 +718,7 @@ class StageCodegen {
     for (bool loads : {true, false}) {
       em_.line("#pragma unroll");
       em_.open("for (int it_ = 0; it_ < " + std::to_string(chunk) + "; ++it_)");
-      emitCopyStep(p, plan, base + "it_", "stage_", "it_", loads);
+      emitCopyStep(p, plan, base + "it_", "stage_", "it_", loads, ceilDiv(plan.iters, chunk) * chunk);
       em_.close();
     }
     em_.close();
