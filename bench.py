@@ -4,9 +4,20 @@
 One "step" = one launch of the compiled TC over one batch of synthetic, seeded inputs that are
 already resident in HBM.  The headline workload is the HBM-bound tensordot
 O(n,c1,c3,h,w) +=! I0(n,c1,r_c2,h,w) * I1(n,r_c2,c3,h,w) at N=32, C1=512, C2=8, C3=2, H=W=28;
-`--config` selects another of the five workloads, `--all` appends their figures under "others",
-`--suite` appends the reference's other benchmark programs at their default sizes under "suite".
-Prints ONE JSON line.
+`--config` selects another of the five workloads; the other four are always measured too and
+reported under "others" (kernel time, roofline, traffic); `--suite` appends the reference's other
+benchmark programs at their default sizes under "suite".  Prints ONE JSON line.
+
+Before the W warm-up steps of a workload the kernel is launched back to back for a fixed time
+(--spin-ms, 150 ms): the kernels here run for 3 to 90 us, a handful of launches end before the
+device has left its idle clocks, and what is measured is the steady state.  The spin is not part
+of the warm-up or of the K timed steps.
+
+Device memory comes from the library's own thin HIP layer (tensorcomprehensions_amd.DeviceBuffer):
+PyTorch is not loaded, so the kernels are compiled by the hipRTC of the ROCm installation and
+launched through its runtime (PyTorch bundles older copies of both).  Only `--suite`, which times
+PyTorch's own GPU routines next to the comprehensions, loads PyTorch, first, for the whole process;
+the ATen CPU baseline runs in a child process.
 """
 import argparse
 import json
@@ -38,27 +49,65 @@ def flops(name, shapes):
     return 6 * m * n
 
 
+SPIN_MS = 150.0
+
+
+def spin(ex, ins, outs, ms):
+    """Back-to-back launches for about `ms` milliseconds of device time."""
+    import tensorcomprehensions_amd as tc
+    spent = 0.0
+    while spent < ms * 1e3:
+        spent += tc.profile_repeated(ex, ins, outs, 200)
+
+
+def algorithmic_bytes(src, entry, ins):
+    """Every input read once and every output written once."""
+    import numpy as np
+    import tensorcomprehensions_amd as tc
+    n = sum(t.numel() * t.element_size() for t in ins)
+    for dtype, shape, _ in tc.infer_output_tensor_info(src, entry, ins):
+        count = 1
+        for e in shape:
+            count *= e
+        n += count * np.dtype(dtype).itemsize
+    return n
+
+
+def to_device(array):
+    """numpy -> device memory: a torch tensor when PyTorch is loaded (--suite), else a DeviceBuffer."""
+    import tensorcomprehensions_amd as tc
+    torch = sys.modules.get("torch")
+    if torch is not None:
+        return torch.from_numpy(array).cuda()
+    return tc.DeviceBuffer.from_numpy(array)
+
+
+def device_sync():
+    torch = sys.modules.get("torch")
+    if torch is not None:
+        torch.cuda.synchronize()          # (profile_repeated has synchronised the stream already)
+
+
 def measure(name, steps, warmup, options=None):
-    import torch
     import tensorcomprehensions_amd as tc
     from tests import workloads as W
 
     src, entry, shapes, _, _ = W.CONFIGS[name]
-    ins = [torch.from_numpy(a).cuda() for a in W.make_inputs(name)]
+    ins = [to_device(a) for a in W.make_inputs(name)]
     opts = options or W.TUNED[name]
     ex = tc.compile(src, entry, ins, opts)
     outs = tc.prepare_outputs(src, entry, ins)
-    for _ in range(warmup):
-        tc.unchecked_run(ex, ins, outs)
-    torch.cuda.synchronize()
+    spin(ex, ins, outs, SPIN_MS)
+    if warmup > 0:
+        tc.profile_repeated(ex, ins, outs, warmup)      # W untimed steps; returns once they have finished
     # timed region: K steps issued back to back inside the library, bracketed by HIP events on the
     # launch stream (device time) and by the host clock around the synchronised whole
     t0 = time.perf_counter()
     device_us = tc.profile_repeated(ex, ins, outs, steps)
-    torch.cuda.synchronize()
+    device_sync()
     wall = time.perf_counter() - t0
     kernel_ms = device_us / 1e3 / steps
-    nbytes = W.algorithmic_bytes(name)
+    nbytes = algorithmic_bytes(src, entry, ins)
     return {
         "name": name, "options": opts, "wall_s": wall, "kernel_ms": kernel_ms, "bytes": nbytes,
         "flops": flops(name, shapes), "launch": [ex.launch_bounds(k) for k in range(ex.num_kernels)],
@@ -73,24 +122,27 @@ COPY_ELEMS = 64 * 1024 * 1024           # 256 MiB read + 256 MiB written per lau
 def calibrate_copy(steps):
     """A plain copy through the same backend: what FETCH_SIZE / WRITE_SIZE read for a kernel whose
     HBM traffic is known (268 435 456 B each way) scales the counters of the measured kernel."""
-    import torch
+    import numpy as np
     import tensorcomprehensions_amd as tc
-    src = torch.ones(COPY_ELEMS, device="cuda")
+    src = to_device(np.ones(COPY_ELEMS, dtype=np.float32))
     ex = tc.compile(COPY_TC, "copy", [src], "naive;tile=4096;mapToThreads=256;mapToBlocks=16384;vectorWidth=4;unroll=16")
     (dst,) = tc.prepare_outputs(COPY_TC, "copy", [src])
     us = tc.profile_repeated(ex, [src], [dst], steps) / steps
-    torch.cuda.synchronize()
     sys.stderr.write(f"copy calibration: {2 * 4 * COPY_ELEMS / us / 1e3:.1f} GB/s, {us:.1f} us per launch\n")
 
 
-def measured_traffic(name):
-    """HBM bytes per launch from the committed counter summary of this workload, if there is one."""
+def measured_traffic(name, options):
+    """HBM bytes per launch from the committed counter summary of this workload, if there is one
+    and it was taken under the options being timed."""
     short = {"c2_tensordot": "tensordot_c2", "c3_batch_matmul": "batch_matmul_c3",
              "c4_group_convolution": "group_convolution_c4", "c5_moments": "moments_c5"}.get(name)
     path = os.path.join(ROOT, "profiles", f"{short}_hbm_traffic.txt")
     if not short or not os.path.exists(path):
         return None
-    for line in open(path):
+    lines = open(path).read().splitlines()
+    if f"options: {options}" not in lines:
+        return None
+    for line in lines:
         if line.startswith("traffic_bytes_per_launch:"):
             return int(line.split(":")[1])
     return None
@@ -101,12 +153,12 @@ def roofline(m):
     tfl = m["flops"] / (m["kernel_ms"] * 1e-3) / 1e12
     if "group_convolution" in m["name"]:
         return {"bound": "mfma", "achieved": round(tfl, 3), "peak": FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(tfl / FP32_PEAK_TFLOPS, 4), "traffic": measured_traffic(m["name"])}
+                "frac": round(tfl / FP32_PEAK_TFLOPS, 4), "traffic": measured_traffic(m["name"], m["options"])}
     return {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": measured_traffic(m["name"])}
+            "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": measured_traffic(m["name"], m["options"])}
 
 
-def cpu_baseline(name, budget_s=15.0):
+def cpu_baseline(name, nbytes, budget_s=15.0):
     """The oracle's sequential loop nest (-O3 -march=native, one core) on the same inputs."""
     from oracle import tc_oracle
     from tests import workloads as W
@@ -120,11 +172,26 @@ def cpu_baseline(name, budget_s=15.0):
         tc_oracle.run(src, entry, ins, native=True)
         times.append(time.perf_counter() - t0)
     med = sorted(times)[len(times) // 2]
-    return {"value": round(W.algorithmic_bytes(name) / med / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+    return {"value": round(nbytes / med / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
             "sample": f"full {name} workload, median of {len(times)} runs of the sequential loop nest, {med * 1e3:.1f} ms each"}
 
 
-def aten_cpu_baseline(name, budget_s=10.0):
+def aten_cpu_baseline(name, nbytes, budget_s=10.0):
+    """aten_cpu_baseline_here in a child process (PyTorch stays out of the measuring process)."""
+    import subprocess
+    code = (f"import json, sys; sys.path.insert(0, {ROOT!r}); import bench; "
+            f"print('ATEN_JSON' + json.dumps(bench.aten_cpu_baseline_here({name!r}, {nbytes}, {budget_s})))")
+    try:
+        out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=budget_s * 6 + 120)
+        for text in out.stdout.splitlines():
+            if text.startswith("ATEN_JSON"):
+                return json.loads(text[len("ATEN_JSON"):])
+    except subprocess.TimeoutExpired:
+        pass
+    return None
+
+
+def aten_cpu_baseline_here(name, nbytes, budget_s=10.0):
     """The library routine the reference's own benchmarks compare with (at::einsum / bmm / conv2d / mean, var)
     on the host cores with torch's default intra-op threads; None for workloads without one."""
     import torch
@@ -148,7 +215,7 @@ def aten_cpu_baseline(name, budget_s=10.0):
         fn()
         times.append(time.perf_counter() - t0)
     med = sorted(times)[len(times) // 2]
-    return {"value": round(W.algorithmic_bytes(name) / med / 1e9, 3), "unit": "GB/s", "threads": torch.get_num_threads(),
+    return {"value": round(nbytes / med / 1e9, 3), "unit": "GB/s", "threads": torch.get_num_threads(),
             "sample": f"ATen CPU routine on the full {name} workload, median of {len(times)} runs, {med * 1e3:.1f} ms each"}
 
 
@@ -186,6 +253,7 @@ def measure_suite(steps, warmup):
         ins = [torch.from_numpy(a).cuda() for a in B.make_inputs(name, reference_sizes=True)]
         ex = tc.compile(src, entry, ins, options)
         outs = tc.prepare_outputs(src, entry, ins)
+        spin(ex, ins, outs, SPIN_MS / 3)
         for _ in range(warmup):
             tc.unchecked_run(ex, ins, outs)
         us = tc.profile_repeated(ex, ins, outs, steps) / steps
@@ -218,7 +286,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--config", default="c2_tensordot")
     ap.add_argument("--options", default=None)
-    ap.add_argument("--all", action="store_true")
+    ap.add_argument("--all", action="store_true", help="(kept for old command lines: the other workloads are always measured)")
+    ap.add_argument("--only", action="store_true", help="measure the selected workload alone (profiling runs)")
+    ap.add_argument("--spin-ms", type=float, default=SPIN_MS,
+                    help="back-to-back launches for this long before the warm-up steps (device clocks)")
     ap.add_argument("--tune", default=None, metavar="GENERATIONSxPOPULATION",
                     help="autotune the workload from the naive options first (e.g. 5x40) and measure the best")
     ap.add_argument("--suite", action="store_true",
@@ -227,20 +298,21 @@ def main():
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain copy kernel of known size (reference point for HBM byte counters)")
     a = ap.parse_args()
+    globals()["SPIN_MS"] = a.spin_ms
     if a.gpus != 1:
         sys.exit("bench.py measures one GPU: this backend has no multi-GPU path (run with --gpus 1)")
-    import torch
-    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    if a.suite:
+        import torch  # noqa: F401  (first, so that the whole process runs on PyTorch's HIP runtime)
+    import tensorcomprehensions_amd as tc
     from tests import workloads as W
 
     if a.calibrate:
         calibrate_copy(a.steps)
     tuned_in = None
     if a.tune:
-        import tensorcomprehensions_amd as tc
         gens, pop = (int(x) for x in a.tune.lower().split("x"))
         src, entry = W.CONFIGS[a.config][0], W.CONFIGS[a.config][1]
-        ins = [torch.from_numpy(x).cuda() for x in W.make_inputs(a.config)]
+        ins = [to_device(x) for x in W.make_inputs(a.config)]
         t0 = time.perf_counter()
         best = tc.autotune(src, entry, ins, "naive", generations=gens, pop_size=pop, threads=16, seed=1, top_k=1)
         tuned_in = time.perf_counter() - t0
@@ -258,15 +330,15 @@ def main():
         "config": {"workload": a.config, "shapes": [list(s) for s in W.CONFIGS[a.config][2]],
                    "options": m["options"], "launch": m["launch"], "algorithmic_bytes": m["bytes"]},
         "roofline": roofline(m),
-        "device": torch.cuda.get_device_name(0),
+        "device": tc.device_name(),
     }
     if tuned_in is not None:
         line["config"]["options_from"] = f"autotuned from the naive options, {a.tune} candidates, {tuned_in:.0f} s"
     if not a.no_cpu:
-        line["cpu_baseline"] = cpu_baseline(a.config)
+        line["cpu_baseline"] = cpu_baseline(a.config, m["bytes"])
         line["cpu_baseline"]["host_cores"] = os.cpu_count()
-        line["cpu_baseline"]["aten"] = aten_cpu_baseline(a.config)
-    if a.all:
+        line["cpu_baseline"]["aten"] = aten_cpu_baseline(a.config, m["bytes"])
+    if not a.only:
         others = {}
         for name in W.CONFIGS:
             if name == a.config:

@@ -30,6 +30,13 @@ int tchip_device_compute_units(int device, int* count);
 int tchip_sync_device(void);                                   /* cuda.cc:88-90 */
 int tchip_stream_sync(tchip_stream_t stream);
 
+/* device memory for callers that hold no tensor library of their own (the reference leaves
+ * allocation to ATen, tc/aten/aten_compiler.cc:46-67): hipMalloc / hipFree and synchronous copies */
+int tchip_malloc(void** ptr, size_t bytes);
+int tchip_free_device(void* ptr);
+int tchip_memcpy_to_device(void* dst, const void* src, size_t bytes);
+int tchip_memcpy_to_host(void* dst, const void* src, size_t bytes);
+
 /* JIT — nvrtcCreateProgram / CompileProgram / GetProgramLog / GetPTX
  * (tc/core/cuda/cuda_rtc.cc:208-262).  `arch` like "gfx950"; `flags` are extra compiler
  * options.  On return *code / *log are malloc'ed (free with tchip_free); *log is set even

@@ -19,11 +19,12 @@ import ctypes
 
 from . import _capi
 from ._capi import TcError
+from .device_memory import DeviceBuffer, device_name
 from .mapping_options import MappingOptions, FusionStrategy
 
 __all__ = [
     "compile", "prepare_outputs", "infer_output_tensor_info", "run", "profile", "profile_repeated", "unchecked_run", "autotune",
-    "map_only", "lang_dump", "host_query", "set_compiler_options", "ShapeOnly", "Executor", "MappingOptions", "FusionStrategy", "ProfilingInfo", "TcError",
+    "map_only", "lang_dump", "host_query", "set_compiler_options", "ShapeOnly", "DeviceBuffer", "device_name", "Executor", "MappingOptions", "FusionStrategy", "ProfilingInfo", "TcError",
 ]
 
 ProfilingInfo = namedtuple("ProfilingInfo", ["cpu_overhead_us", "kernel_runtime_us"])
@@ -38,6 +39,9 @@ def _dtype_name(t):
 def _metas(tensors):
     out = []
     for t in tensors:
+        if isinstance(t, DeviceBuffer):
+            out.append((t.data_ptr(), t.dtype_name, t.shape, t.stride(), 10, t.device_index))
+            continue
         dev_type = 10 if t.is_cuda else 1           # kDLROCM / kDLCPU
         dev_id = t.device.index or 0
         out.append((t.data_ptr(), _dtype_name(t), tuple(t.shape), tuple(t.stride()), dev_type, dev_id))
@@ -73,8 +77,11 @@ def _pack(tensors):
 
 
 def _stream():
-    import torch
-    if torch.cuda.is_available():
+    """PyTorch's current stream when the caller has PyTorch loaded, else the default stream.
+    (PyTorch is never imported from here: a process that works on DeviceBuffers stays without it.)"""
+    import sys
+    torch = sys.modules.get("torch")
+    if torch is not None and torch.cuda.is_available():
         return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     return ctypes.c_void_p(0)
 
@@ -159,9 +166,11 @@ def infer_output_tensor_info(tc, entry_point, inputs):
 def prepare_outputs(tc, entry_point, inputs):
     """Allocate output tensors on the device of inputs[0] (tc::aten::prepareOutputs,
     tc/aten/aten_compiler.cc:46-67): needs at least one input; memory is uninitialised."""
-    import torch
     if len(inputs) == 0:
         raise TcError("NYI: Need >0 inputs to determine the backend for the outputs")
+    if isinstance(inputs[0], DeviceBuffer):
+        return [DeviceBuffer(shape, name) for name, shape, _ in infer_output_tensor_info(tc, entry_point, inputs)]
+    import torch
     return [torch.empty(shape, dtype=getattr(torch, name), device=inputs[0].device)
             for name, shape, _ in infer_output_tensor_info(tc, entry_point, inputs)]
 

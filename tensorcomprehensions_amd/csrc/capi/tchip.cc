@@ -42,6 +42,9 @@ struct HipApi {
   TCHIP_FN(hipEventDestroy);
   TCHIP_FN(hipGetLastError);
   TCHIP_FN(hipGetErrorString);
+  hipError_t (*hipMallocFn)(void**, size_t) = nullptr;
+  TCHIP_FN(hipFree);
+  TCHIP_FN(hipMemcpy);
   TCHIP_FN(hiprtcCreateProgram);
   TCHIP_FN(hiprtcCompileProgram);
   TCHIP_FN(hiprtcGetProgramLogSize);
@@ -100,6 +103,9 @@ struct HipApi {
       TCHIP_BIND(hipEventDestroy);
       TCHIP_BIND(hipGetLastError);
       TCHIP_BIND(hipGetErrorString);
+      bind(hipLib, "hipMalloc", hipMallocFn);
+      TCHIP_BIND(hipFree);
+      TCHIP_BIND(hipMemcpy);
 #undef TCHIP_BIND
     }
     if (rtcLib) {
@@ -180,10 +186,28 @@ int tchip_set_device(int device) {
   TCHIP_TRY(hipSetDevice(device));
   return 0;
 }
+int tchip_malloc(void** ptr, size_t bytes) {
+  TCHIP_TRY(hipMallocFn(ptr, bytes));
+  return 0;
+}
+int tchip_free_device(void* ptr) {
+  TCHIP_TRY(hipFree(ptr));
+  return 0;
+}
+int tchip_memcpy_to_device(void* dst, const void* src, size_t bytes) {
+  TCHIP_TRY(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice));
+  return 0;
+}
+int tchip_memcpy_to_host(void* dst, const void* src, size_t bytes) {
+  TCHIP_TRY(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost));
+  return 0;
+}
 int tchip_device_name(int device, char* buf, size_t n) {
   hipDeviceProp_t p;
   if (int st = deviceProps(device, &p)) return st;
-  std::strncpy(buf, p.name, n);
+  // (the marketing name comes from a table that an installation may lack: the architecture
+  // string then identifies the device)
+  std::strncpy(buf, p.name[0] ? p.name : p.gcnArchName, n);
   if (n) buf[n - 1] = '\0';
   return 0;
 }

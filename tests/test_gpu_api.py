@@ -216,3 +216,24 @@ def test_run_can_be_captured_in_a_hip_graph_and_replayed():
         torch.cuda.synchronize()
         assert torch.equal(outs[0], eager[0]), replay
         assert (outs[0] - torch.bmm(ins[0], ins[1])).abs().max().item() <= 1e-5 * 72 ** 0.5 * float(outs[0].abs().max())
+
+
+@pytest.mark.gpu
+def test_device_buffers_stand_in_for_tensors():
+    """The package's own device arrays (no tensor library) go through compile, prepare_outputs,
+    run and profile like torch tensors and give the oracle's values."""
+    from oracle import tc_oracle
+    from tests import workloads as W
+    name = "c1_tensordot_small"
+    src, entry, _, _, k = W.CONFIGS[name]
+    ins_np = W.make_inputs(name)
+    ins = [tc.DeviceBuffer.from_numpy(a) for a in ins_np]
+    ex = tc.compile(src, entry, ins, W.TUNED[name])
+    outs = tc.prepare_outputs(src, entry, ins)
+    assert isinstance(outs[0], tc.DeviceBuffer) and outs[0].shape == (16, 8, 2, 17, 25)
+    tc.run(ex, ins, outs)
+    info = tc.profile(ex, ins, outs)
+    assert info.kernel_runtime_us > 0
+    ref = tc_oracle.run(src, entry, ins_np)[0]
+    assert np.abs(outs[0].numpy() - ref).max() <= W.tolerance(k, ref)
+    assert "MI3" in tc.device_name() or "AMD" in tc.device_name()

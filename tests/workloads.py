@@ -41,7 +41,7 @@ CONFIGS = {
 TUNED = {
     "c1_tensordot_small": "naive;tile=1,1,0,0,0;mapToThreads=425;mapToBlocks=256,256;unroll=128;vectorWidth=4;useReadOnlyCache=1",
     "c2_tensordot": "naive;tile=1,8,2,0;mapToThreads=256;mapToBlocks=32,64;unroll=128;vectorWidth=4;useReadOnlyCache=1",
-    "c3_batch_matmul": "naive;tile=1,26,26;mapToThreads=64,4;mapToBlocks=500;useMfma=1;useSharedMemory=0",
+    "c3_batch_matmul": "naive;tile=1,26,26;mapToThreads=64,4;mapToBlocks=500;useMfma=1;useSharedMemory=1",
     "c4_group_convolution": "naive;tile=1,1,16,14,14;mapToThreads=64,4;mapToBlocks=32,32;useMfma=1;useSharedMemory=1;useReadOnlyCache=1",
     "c5_moments": "naive;tile=1;mapToThreads=512;mapToBlocks=1024;matchLibraryCalls=1;unroll=8;vectorWidth=4;usePrivateMemory=1;useReadOnlyCache=1",
 }
@@ -63,12 +63,3 @@ def make_inputs(name, seed=0xC0FFEE):
 def tolerance(reduction_length, ref):
     """fp32 bound of the acceptance rule: 1e-5 * sqrt(K) * max|ref|."""
     return 1e-5 * math.sqrt(reduction_length) * max(float(np.abs(ref).max()), 1e-30)
-
-
-def algorithmic_bytes(name):
-    """Every input read once and every output written once, fp32."""
-    from oracle import tc_oracle
-    tc, entry, shapes, _, _ = CONFIGS[name]
-    n = sum(int(np.prod(s)) for s in shapes)
-    n += sum(int(np.prod(s)) for _, _, s in tc_oracle.infer_output_shapes(tc, entry, shapes))
-    return 4 * n
