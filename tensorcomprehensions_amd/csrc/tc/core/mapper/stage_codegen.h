@@ -1441,11 +1441,28 @@ class StageCodegen {
       em_.line("const int mposa_ = mt_ * 16 + lm_;");
       em_.line("const bool moka_ = bok_ && " + decodeGroup(st_.mfmaM, "mposa_", true) + ";");
       em_.line("(void)moka_;");
-      bool masked = openSteps();
-      em_.line("const float a_ = " + (resident ? std::string("am_[ks_]") : operandValue(loadA, masked)) + ";");
-      em_.line("const float b_ = " + operandValue(loadB, masked) + ";");
-      em_.line(acc + " = __builtin_amdgcn_mfma_f32_16x16x4f32(a_, b_, " + acc + ", 0, 0, 0);");
-      em_.close();
+      if (ksteps <= kMaxResidentSteps) {
+        // The operand values of all steps first, then the chain of multiplications: every read is
+        // in flight before the first result is needed, and the multiplications wait for nothing
+        // but their own operands (10.5 -> 10.0 us on the 16-channel 3x3 group convolution).
+        em_.line("float bq_[" + std::to_string(ksteps) + "];");
+        if (!resident) em_.line("float aq_[" + std::to_string(ksteps) + "];");
+        bool masked = openSteps();
+        if (!resident) em_.line("aq_[ks_] = " + operandValue(loadA, masked) + ";");
+        em_.line("bq_[ks_] = " + operandValue(loadB, masked) + ";");
+        em_.close();
+        em_.line("#pragma unroll");
+        em_.open("for (int ks_ = 0; ks_ < " + std::to_string(ksteps) + "; ++ks_)");
+        em_.line(acc + " = __builtin_amdgcn_mfma_f32_16x16x4f32(" + (resident ? "am_" : "aq_") + "[ks_], bq_[ks_], " + acc +
+                 ", 0, 0, 0);");
+        em_.close();
+      } else {
+        bool masked = openSteps();
+        em_.line("const float a_ = " + (resident ? std::string("am_[ks_]") : operandValue(loadA, masked)) + ";");
+        em_.line("const float b_ = " + operandValue(loadB, masked) + ";");
+        em_.line(acc + " = __builtin_amdgcn_mfma_f32_16x16x4f32(a_, b_, " + acc + ", 0, 0, 0);");
+        em_.close();
+      }
       em_.close();
     };
     // Epilogue and store: a lane holds rows 4*lj_ .. 4*lj_+3 of column lm_.  Indices are clamped
