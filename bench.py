@@ -131,6 +131,25 @@ def calibrate_copy(steps):
     sys.stderr.write(f"copy calibration: {2 * 4 * COPY_ELEMS / us / 1e3:.1f} GB/s, {us:.1f} us per launch\n")
 
 
+def launch_floor(steps):
+    """Per-launch time of copy kernels that do next to nothing, issued back to back like the
+    workloads (one wavefront; 64 and 500 blocks of 256 threads, 4 KiB each): what a launch costs
+    on this device whatever the kernel does.  The 3 us workloads are to be read against it."""
+    import numpy as np
+    import tensorcomprehensions_amd as tc
+    out = {}
+    for label, n, opts in [("copy_1_block_of_64", 64, "naive;mapToThreads=64;mapToBlocks=1;tile=64"),
+                           ("copy_64_blocks_of_256", 64 * 1024, "naive;mapToThreads=256;mapToBlocks=64;tile=1024;vectorWidth=4"),
+                           ("copy_500_blocks_of_256", 500 * 1024, "naive;mapToThreads=256;mapToBlocks=500;tile=1024;vectorWidth=4")]:
+        src = to_device(np.ones(n, dtype=np.float32))
+        ex = tc.compile(COPY_TC, "copy", [src], opts)
+        (dst,) = tc.prepare_outputs(COPY_TC, "copy", [src])
+        spin(ex, [src], [dst], SPIN_MS)
+        out[label] = {"us_per_launch": round(tc.profile_repeated(ex, [src], [dst], steps) / steps, 3),
+                      "kernel": ex.kernel_name(), "launch": ex.launch_bounds()}
+    return out
+
+
 def measured_traffic(name, options):
     """HBM bytes per launch from the committed counter summary of this workload, if there is one
     and it was taken under the options being timed."""
@@ -295,6 +314,8 @@ def main():
     ap.add_argument("--suite", action="store_true",
                     help="also time the reference's other benchmark comprehensions at their default sizes")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--floor", action="store_true",
+                    help="also time near-empty copy kernels of 1, 64 and 500 blocks (the cost of a launch)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain copy kernel of known size (reference point for HBM byte counters)")
     a = ap.parse_args()
@@ -347,6 +368,8 @@ def main():
             others[name] = {"kernel_us": round(o["kernel_ms"] * 1e3, 3), "roofline": roofline(o),
                             "gflops": round(o["flops"] / (o["kernel_ms"] * 1e-3) / 1e9, 1), "launch": o["launch"]}
         line["others"] = others
+    if a.floor:
+        line["launch_floor"] = launch_floor(a.steps)
     if a.suite:
         line["suite"] = measure_suite(a.steps, a.warmup)
     print(json.dumps(line))

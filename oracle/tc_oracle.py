@@ -743,7 +743,13 @@ def _identity(op: str, scalar: str) -> str:
     v = info.max if base == "min" else info.min
     if scalar == "float":
         return f"{float(v)!r}f".replace("e+", "e")
-    return repr(float(v)) if fl else (f"{int(v)}LL" if "64" in scalar else str(int(v)))
+    if fl:
+        return repr(float(v))
+    if scalar == "uint64":
+        return f"{int(v)}ULL"
+    if scalar == "int64":
+        return f"({int(v) + 1}LL - 1)" if v < 0 else f"{int(v)}LL"   # (-2^63 has no literal of its own)
+    return str(int(v))
 
 
 class _CEmitter:
@@ -799,6 +805,8 @@ class _CEmitter:
                     return f"{'fminf' if e.op == 'min' else 'fmaxf'}({sa}, {sb})" if mt == "float" else f"f{e.op}({sa}, {sb})"
                 return f"(({sa}) {'<' if e.op == 'min' else '>'} ({sb}) ? ({sa}) : ({sb}))"
             if e.op in ("/", "%") and mt not in ("float", "double") and not pretty:
+                if mt.startswith("uint") or mt == "bool":
+                    return f"({sa} {e.op} {sb})"     # unsigned: rounding down is truncation (and 2^63.. must not pass through int64)
                 return f"tc_floor{'div' if e.op == '/' else 'mod'}({sa}, {sb})"   # Halide integer semantics
             if e.op == "%" and mt in ("float", "double") and not pretty:
                 return f"fmod{'f' if mt == 'float' else ''}({sa}, {sb})"
@@ -945,6 +953,8 @@ def run(tc: str, entry: str, inputs: Sequence[np.ndarray], outputs: Optional[Seq
     an = analyze(tc, entry, [a.shape for a in inputs])
     for name, a in zip(an.inputs, inputs):
         want = _NPTYPE[an.tensors[name].scalar]
+        if an.tensors[name].scalar == "bool" and a.dtype == np.bool_:
+            continue                                   # numpy's own bool: one byte holding 0 or 1, as the kernel reads it
         if a.dtype != want:
             raise TcError(f"expected type {an.tensors[name].scalar} but found {a.dtype}")
     lib = build(an, native)

@@ -50,7 +50,10 @@ void checkInputsCompliant(const ir::Function& f, const std::vector<const DLConst
     const ir::Tensor& decl = f.inputs[i];
     int want = scalarToken(static_cast<uint8_t>(decl.type.code), static_cast<uint8_t>(decl.type.bits));
     int got = scalarToken(t->dtype.code, t->dtype.bits);
-    if (want != got) {
+    // a bool tensor is a byte per element holding 0 or 1: DLPack's (uint, 8) stands for it as
+    // well as the one-bit type the front end infers
+    bool boolAsByte = decl.type.isBool() && t->dtype.code == kDLUInt && t->dtype.bits == 8;
+    if (want != got && !boolAsByte) {
       throw lang::errorAt(def.params()[i]) << "expected type " << lang::kindToString(want) << " but found "
                                            << lang::kindToString(got);
     }

@@ -13,8 +13,16 @@ from tests.test_benchmark_tcs import OPTION_SETS
 
 pytestmark = pytest.mark.gpu
 
-# reductions feeding later reductions: tolerance on the product of the lengths
-CHAINED = {"2fcrelu": 48 * 36, "kronecker3": 60, "batchnorm": 140, "wavenet1": 16 * 8,
+
+
+def chain(*lengths):
+    """Effective reduction length of reductions that feed one another: each stage adds its own
+    1e-5 * sqrt(K_i) (relative to the common scale), so the bound is 1e-5 * sum(sqrt(K_i)),
+    written as the K whose square root that is."""
+    return float(sum(np.sqrt(k) for k in lengths)) ** 2
+
+
+CHAINED = {"2fcrelu": chain(48, 36), "kronecker3": chain(5, 4, 3), "batchnorm": 140, "wavenet1": chain(16, 8, 8),
            "group_normalization_single_kernel": 210}
 
 
@@ -53,9 +61,10 @@ def test_parity_at_the_reference_sizes_with_the_tuned_options(name):
         o.fill_(float("nan"))
     tc.run(ex, ins, outs)
     torch.cuda.synchronize()
-    # reduction lengths at these sizes (chains: the product of the lengths)
-    k = {"tmm": 256, "matmul": 1000, "convolution": 36, "group_convolution": 36, "2fcrelu": 2000 * 128, "lut": 50, "moments2": 36864,
-         "group_normalization_single_kernel": 36864, "kronecker3": 16 ** 3, "wavenet1": 32 * 64}[name]
+    # reduction lengths at these sizes (chains: see chain())
+    k = {"tmm": 256, "matmul": 1000, "convolution": 36, "group_convolution": 36, "2fcrelu": chain(2000, 128), "lut": 50,
+         "moments2": 36864, "group_normalization_single_kernel": 36864, "kronecker3": chain(16, 16, 16),
+         "wavenet1": chain(64, 32, 32)}[name]
     for o, r in zip(outs, ref):
         got = o.cpu().numpy()
         assert got.shape == r.shape
@@ -75,3 +84,25 @@ def test_lookup_indices_are_exact():
         (out,) = tc.prepare_outputs(B.LUT, "lut", ins)
         tc.run(ex, ins, [out])
         assert np.array_equal(out.cpu().numpy(), ref)
+
+
+@pytest.mark.parametrize("options", sorted(OPTION_SETS))
+@pytest.mark.parametrize("name", ["2fcrelu", "kronecker3", "matmul", "tmm_odd", "convolution"])
+def test_chains_and_contractions_are_exact_on_small_integers(name, options):
+    """Inputs in {-2..2}: every product, partial sum and intermediate result is an integer far
+    below 2^24, so any order of summation gives the same bits and a dropped or doubled partial
+    result cannot hide inside a tolerance."""
+    src, entry, _, _ = B.CASES[name]
+    rng = np.random.Generator(np.random.Philox(77))
+    ins_np = [rng.integers(-2, 3, size=a.shape).astype(a.dtype) for a in B.make_inputs(name)]
+    ref = tc_oracle.run(src, entry, ins_np)
+    assert all(np.abs(r).max() < 2 ** 22 and np.array_equal(r, np.round(r)) for r in ref)
+    ins = [torch.from_numpy(a).cuda() for a in ins_np]
+    ex = tc.compile(src, entry, ins, OPTION_SETS[options])
+    outs = tc.prepare_outputs(src, entry, ins)
+    for o in outs:
+        o.fill_(float("nan"))
+    tc.run(ex, ins, outs)
+    torch.cuda.synchronize()
+    for o, r in zip(outs, ref):
+        assert np.array_equal(o.cpu().numpy(), r), (name, options, ex.launch_bounds())

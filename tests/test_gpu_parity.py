@@ -68,12 +68,22 @@ def test_indexing_bit_exact_with_integer_inputs(name):
     """Small integers make every fp32 product and sum exact, so any mis-indexing shows up as a
     non-zero integer difference regardless of summation order."""
     src, entry, shapes, _ = SMALL[name]
-    if name == "moments":
-        pytest.skip("divides by N: not exact in fp32")
     rng = np.random.Generator(np.random.Philox(99))
     ins = [rng.integers(-4, 5, size=s).astype(np.float32) for s in shapes]
+    variants = ("naive", W.TUNED["c2_tensordot"] if name == "tensordot" else "pointwise")
+    if name == "moments":
+        # Rows of 1024 = 2^10 small integers whose sum is a multiple of 1024: X/N, the mean (an
+        # integer), (X - mean)^2 / N and every partial sum of either reduction are exact in fp32.
+        half = rng.integers(-4, 5, size=(9, 512))
+        rows = np.concatenate([half, -rng.permuted(half, axis=1)], axis=1) + rng.integers(-2, 3, size=(9, 1))
+        ins = [rng.permuted(rows, axis=1).astype(np.float32)]
+        assert np.all(ins[0].sum(1) % 1024 == 0)
+        variants = ("naive", "naive;tile=1;mapToThreads=256;mapToBlocks=9;matchLibraryCalls=1;unroll=4;vectorWidth=4;usePrivateMemory=1")
     ref = tc_oracle.run(src, entry, ins)
-    for opts in ("naive", W.TUNED["c2_tensordot"] if name == "tensordot" else "pointwise"):
+    if name == "moments":
+        assert np.array_equal(ref[0], ins[0].mean(1, dtype=np.float64).astype(np.float32))
+        assert np.array_equal(ref[1], ins[0].var(1, dtype=np.float64).astype(np.float32))
+    for opts in variants:
         got, _ = run_hip(src, entry, ins, opts)
         for g, r in zip(got, ref):
             assert np.array_equal(g, r)

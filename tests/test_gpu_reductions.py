@@ -177,3 +177,143 @@ def test_tensor_rewritten_by_a_later_stage_of_the_same_kernel(options):
     A = np.random.Generator(np.random.Philox(9)).standard_normal((50, 384), dtype=np.float32)
     ex = check(ROW_NORMALISE, "f", [A], options, 384)
     assert ex.num_kernels == (3 if "Min" in options else 1)
+
+
+# ------------------------------------------------------------------------------------------------
+# products through the block reduction (the reference's library matches `+` only,
+# tc/core/polyhedral/cuda/mapped_scop.cc:253-311): lane-group, whole-wavefront and LDS row widths
+# ------------------------------------------------------------------------------------------------
+PROD_WIDTHS = [(32, 32), (64, 64), (128, 128), (192, 192), (48, 48), (33, 33), (7, 7)]
+
+
+def run_one(src, entry, ins_np, options, prefill=None):
+    ins = [torch.from_numpy(a).cuda() for a in ins_np]
+    ex = tc.compile(src, entry, ins, options)
+    outs = tc.prepare_outputs(src, entry, ins)
+    for i, o in enumerate(outs):
+        if prefill is not None:
+            o.copy_(torch.from_numpy(prefill[i]))
+        elif o.dtype.is_floating_point:
+            o.fill_(float("nan"))
+    tc.run(ex, ins, outs)
+    torch.cuda.synchronize()
+    return [o.cpu().numpy() for o in outs], ex
+
+
+@pytest.mark.parametrize("threads,block_x", PROD_WIDTHS)
+def test_row_products_near_one(threads, block_x):
+    """Factors 1 + N(0, 0.01): the product stays finite and its relative error is bounded like a
+    sum's (log of the product = sum of the logs)."""
+    src = "def prod(float(M, N) A) -> (C) { C(m) *=! A(m, r_n) }"
+    A = (1.0 + 0.01 * np.random.Generator(np.random.Philox(threads)).standard_normal((29, 1000))).astype(np.float32)
+    (got,), ex = run_one(src, "prod", [A], f"naive;matchLibraryCalls=1;mapToThreads={threads};mapToBlocks=29;tile=1")
+    assert ex.launch_bounds()[1][0] == block_x
+    assert "blockAllReduceX<__tc::OpProd<float>" in ex.compiled_source
+    (ref,) = tc_oracle.run(src, "prod", [A])
+    exact = A.astype(np.float64).prod(1)
+    assert np.abs(ref - exact).max() <= 1e-5 * np.sqrt(1000) * np.abs(exact).max()      # the oracle itself
+    assert np.abs(got - ref).max() <= W.tolerance(1000, ref)
+
+
+@pytest.mark.parametrize("threads,block_x", PROD_WIDTHS)
+def test_row_products_of_small_integers_are_exact(threads, block_x):
+    """Signs and at most twenty factors of two per row: every partial product is an exact fp32
+    value whatever the order, so the result is bit for bit the oracle's and the closed form."""
+    src = "def prod(float(M, N) A) -> (C) { C(m) *=! A(m, r_n) }"
+    rng = np.random.Generator(np.random.Philox(1000 + threads))
+    A = rng.choice(np.array([1.0, -1.0], np.float32), size=(31, 777))
+    twos = np.zeros(31, np.int64)
+    for m in range(31):
+        cols = rng.choice(777, size=int(rng.integers(0, 21)), replace=False)
+        A[m, cols] *= 2.0
+        twos[m] = len(cols)
+    (got,), _ = run_one(src, "prod", [A], f"naive;matchLibraryCalls=1;mapToThreads={threads};mapToBlocks=16;tile=1")
+    closed = np.where((A < 0).sum(1) % 2 == 1, -1.0, 1.0) * 2.0 ** twos
+    (ref,) = tc_oracle.run(src, "prod", [A])
+    assert np.array_equal(ref, closed.astype(np.float32))
+    assert np.array_equal(got, ref)
+
+
+@pytest.mark.parametrize("threads", [32, 128, 48])
+def test_non_initialising_product_multiplies_into_existing_values(threads):
+    src = "def prod(float(M, N) A) -> (C) { C(m) *= A(m, r_n) }"
+    A = np.full((8, 300), 1.0, np.float32)
+    A[:, ::100] = 2.0                                   # three factors of two per row
+    prior = np.arange(1, 9, dtype=np.float32)
+    (got,), _ = run_one(src, "prod", [A], f"naive;matchLibraryCalls=1;mapToThreads={threads};mapToBlocks=8;tile=1",
+                        prefill=[prior.copy()])
+    assert np.array_equal(got, prior * 8.0)
+
+
+# ------------------------------------------------------------------------------------------------
+# unsigned and boolean tensors on the device (test/cuda/test_compile_and_run.cc:259-310 runs
+# uint8, the signed integers and the floats; the other unsigned widths and bool complete the set)
+# ------------------------------------------------------------------------------------------------
+UNSIGNED = [("uint8", np.uint8), ("uint16", np.uint16), ("uint32", np.uint32), ("uint64", np.uint64)]
+
+
+def device_tensor(array):
+    """torch has no arithmetic for the wider unsigned types, but it can hold their bits."""
+    return torch.from_numpy(array).cuda()
+
+
+@pytest.mark.parametrize("tc_type,np_type", UNSIGNED)
+@pytest.mark.parametrize("threads", [1, 32, 48, 128])
+def test_unsigned_reductions_match_the_oracle_bit_for_bit(tc_type, np_type, threads):
+    src = f"""
+def red({tc_type}(M, N) A) -> (s, lo, hi) {{
+    s(m) +=! A(m, r_n)
+    lo(m) min=! A(m, r_n)
+    hi(m) max=! A(m, r_n)
+}}
+"""
+    info = np.iinfo(np_type)
+    rng = np.random.Generator(np.random.Philox(7))
+    # values in the upper half of the range tell unsigned comparisons from signed ones; the sums wrap
+    A = rng.integers(info.max // 2, info.max, size=(9, 500), dtype=np_type, endpoint=True)
+    A[:, 3] = rng.integers(0, 5, size=9).astype(np_type)
+    lib = "matchLibraryCalls=1;" if threads > 1 else ""
+    got, ex = run_one(src, "red", [A], f"naive;{lib}mapToThreads={max(threads, 1)};mapToBlocks=9;tile=1")
+    ref = tc_oracle.run(src, "red", [A])
+    for g, r, name in zip(got, ref, ("sum", "min", "max")):
+        assert g.dtype == r.dtype == np.dtype(np_type), name
+        assert np.array_equal(g, r), name
+    assert np.array_equal(ref[0], A.sum(1, dtype=np_type))           # wrap-around sum
+    assert np.array_equal(ref[1], A.min(1)) and np.array_equal(ref[2], A.max(1))
+
+
+@pytest.mark.parametrize("tc_type,np_type", UNSIGNED)
+def test_unsigned_pointwise_arithmetic(tc_type, np_type):
+    src = f"def f({tc_type}(N) A, {tc_type}(N) B) -> (C, D) {{ C(i) = A(i) / B(i) + A(i) % B(i)\n D(i) = max(A(i), B(i)) - min(A(i), B(i)) }}"
+    info = np.iinfo(np_type)
+    rng = np.random.Generator(np.random.Philox(8))
+    A = rng.integers(info.max // 2, info.max, size=1000, dtype=np_type, endpoint=True)
+    B = rng.integers(1, 1000 if info.max > 1000 else info.max, size=1000, dtype=np_type)
+    got, _ = run_one(src, "f", [A, B], "naive")
+    ref = tc_oracle.run(src, "f", [A, B])
+    for g, r in zip(got, ref):
+        assert g.dtype == r.dtype and np.array_equal(g, r)
+    assert np.array_equal(ref[0].astype(np_type), (A // B + A % B).astype(np_type))
+    assert np.array_equal(ref[1].astype(np_type), np.maximum(A, B) - np.minimum(A, B))
+
+
+def test_bool_tensors_on_the_device():
+    src = """
+def f(bool(M, N) P, float(M, N) X) -> (cnt, sel, any) {
+    cnt(m) +=! P(m, r_n) ? 1 : 0
+    sel(m, n) = P(m, n) ? X(m, n) : 0.0
+    any(m) max=! P(m, r_n) ? 1 : 0
+}
+"""
+    rng = np.random.Generator(np.random.Philox(9))
+    P = rng.random((12, 130)) > 0.7
+    P[5] = False
+    X = rng.standard_normal((12, 130), dtype=np.float32)
+    for options in ("naive", "naive;matchLibraryCalls=1;mapToThreads=64;mapToBlocks=12;tile=1,0"):
+        got, _ = run_one(src, "f", [P, X], options)
+        ref = tc_oracle.run(src, "f", [P, X])
+        for g, r in zip(got, ref):
+            assert np.array_equal(g, r), options
+        assert np.array_equal(ref[0], P.sum(1).astype(ref[0].dtype))
+        assert np.array_equal(ref[1], np.where(P, X, np.float32(0)))
+        assert np.array_equal(ref[2], P.any(1).astype(ref[2].dtype))

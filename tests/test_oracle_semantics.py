@@ -162,8 +162,11 @@ def f(float(M, N) X) -> (mx, mn, pr, cnt) {
     cnt(m) +=! (X(m, n) > 0.0) ? 1.0 : 0.0
 }
 """
+    X[1] = -np.abs(X[1]) - 1.0      # an all-negative row: max=! must start below every value, not at 0
+    X[2] = np.abs(X[2]) + 1.0       # an all-positive row: min=! must start above every value
     mx, mn, pr, cnt = tc_oracle.run(src, "f", [X])
     assert np.array_equal(mx, X.max(1)) and np.array_equal(mn, X.min(1))
+    assert mx[1] < 0 and mn[2] > 0
     assert np.allclose(pr, X.astype(np.float64).prod(1), rtol=1e-5)
     assert np.array_equal(cnt, (X > 0).sum(1).astype(np.float32))
 
