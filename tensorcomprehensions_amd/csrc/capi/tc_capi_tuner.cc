@@ -192,65 +192,92 @@ struct FakeBackend {
   static std::string backendString() { return "fake device"; }
 };
 
-std::string cacheSelfTest(const std::string& scratch) {
-#define EXPECT(cond) \
-  if (!(cond)) return std::string("failed: ") + #cond
+// The cache the host queries below work on: two TCs, three options for the first one, one of
+// them measured three times.
+struct SampleCache {
+  TensorInfo in0{{2, 32, 1}, 0, {10, 16}, {16, 1}}, in1{{2, 32, 1}, 0, {16, 20}, {20, 1}};
+  TensorInfo out0{{2, 32, 1}, 0, {10, 20}, {20, 1}};
+  HipMappingOptions o1 = HipMappingOptions::makeNaiveMappingOptions();
+  HipMappingOptions o2 = HipMappingOptions::makeNaiveMappingOptions().tile(4, 4).unroll(8);
+  HipMappingOptions o3 = HipMappingOptions::makePointwiseMappingOptions();
   OptionsCache<FakeBackend> cache;
-  TensorInfo in0({2, 32, 1}, 0, {10, 16}, {16, 1}), in1({2, 32, 1}, 0, {16, 20}, {20, 1});
-  TensorInfo out0({2, 32, 1}, 0, {10, 20}, {20, 1});
-  auto o1 = HipMappingOptions::makeNaiveMappingOptions();
-  auto o2 = HipMappingOptions::makeNaiveMappingOptions().tile(4, 4).unroll(8);
-  auto o3 = HipMappingOptions::makePointwiseMappingOptions();
-  auto us = [](double v) { return Duration::fromMicroSeconds(v); };
-  cache.recordRuntime("tcA", {in0, in1}, {out0}, "dev", o1, us(10));
-  cache.recordRuntime("tcA", {in0, in1}, {out0}, "dev", o1, us(30));
-  cache.recordRuntime("tcA", {in0, in1}, {out0}, "dev", o1, us(20));
-  cache.recordRuntime("tcA", {in0, in1}, {out0}, "dev", o2, us(15));
-  cache.recordRuntime("tcA", {in0, in1}, {out0}, "dev", o3, us(50));
-  cache.recordRuntime("tcB", {in0, in1}, {out0}, "dev", o3, us(5));
-  EXPECT(cache.size() == 4);
-  EXPECT((cache.count({"tcA", {in0, in1}, {out0}, "dev"}) == 3));
-  EXPECT(cache.getKeys().size() == 2);
-  // ranking by the median of all recorded runtimes: o2 (15) < o1 (median 20) < o3 (50)
-  auto top = cache.getTopKEntries("tcA", {in0, in1}, {out0}, "dev", 2);
-  EXPECT(top.size() == 2);
-  EXPECT(top[0].first == o2 && top[0].second == us(15));
-  EXPECT(top[1].first == o1 && top[1].second == us(20));
-  // misses: other TC, other sizes, other device, other alignment
-  EXPECT(cache.getTopKOptions("tcC", {in0, in1}, {out0}, "dev", 1).empty());
-  EXPECT(cache.getTopKOptions("tcA", {in1, in0}, {out0}, "dev", 1).empty());
-  EXPECT(cache.getTopKOptions("tcA", {in0, in1}, {out0}, "other", 1).empty());
-  TensorInfo misaligned = in0;
+  SampleCache() {
+    auto us = [](double v) { return Duration::fromMicroSeconds(v); };
+    cache.recordRuntime("tcA", {in0, in1}, {out0}, "dev", o1, us(10));
+    cache.recordRuntime("tcA", {in0, in1}, {out0}, "dev", o1, us(30));
+    cache.recordRuntime("tcA", {in0, in1}, {out0}, "dev", o1, us(20));
+    cache.recordRuntime("tcA", {in0, in1}, {out0}, "dev", o2, us(15));
+    cache.recordRuntime("tcA", {in0, in1}, {out0}, "dev", o3, us(50));
+    cache.recordRuntime("tcB", {in0, in1}, {out0}, "dev", o3, us(5));
+  }
+};
+
+// Every entry of a cache as text, one per line: id | backend | inputs | outputs | options | runtimes (ns)
+std::string dumpCache(const OptionsCache<FakeBackend>& cache) {
+  std::ostringstream ss;
+  auto tensors = [&](const std::vector<TensorInfo>& ts) {
+    for (size_t i = 0; i < ts.size(); ++i) ss << (i ? ";" : "") << ts[i];
+  };
+  for (const auto& key : cache.getKeys()) {
+    for (const auto& e : cache.getTopKEntries(key.id, key.inputs, key.outputs, key.backendStr, 1000)) {
+      ss << key.id << " | " << key.backendStr << " | ";
+      tensors(key.inputs);
+      ss << " | ";
+      tensors(key.outputs);
+      ss << " | " << e.first.toText() << " | median " << e.second.toNanoSeconds() << "\n";
+    }
+  }
+  return ss.str();
+}
+
+// The behaviours the reference pins for its compilation cache (test/cuda/test_compilation_cache.cc:
+// 133-510: multimap semantics, ranking by the median of all recorded runs, misses, pruning, the
+// wire round trip, store / load / append of files) as "name=value" lines for the caller to check.
+std::string cacheSelfTest(const std::string& scratch) {
+  SampleCache s;
+  auto& cache = s.cache;
+  std::ostringstream out;
+  auto names = [&](const std::vector<std::pair<HipMappingOptions, Duration>>& es) {
+    std::string t;
+    for (const auto& e : es) {
+      t += (t.empty() ? "" : ",") + std::string(e.first == s.o1 ? "o1" : e.first == s.o2 ? "o2" : e.first == s.o3 ? "o3" : "?") +
+          "@" + std::to_string(e.second.toNanoSeconds());
+    }
+    return t;
+  };
+  out << "size=" << cache.size() << "\n";
+  out << "count_tcA=" << cache.count({"tcA", {s.in0, s.in1}, {s.out0}, "dev"}) << "\n";
+  out << "keys=" << cache.getKeys().size() << "\n";
+  out << "top2_tcA=" << names(cache.getTopKEntries("tcA", {s.in0, s.in1}, {s.out0}, "dev", 2)) << "\n";
+  out << "miss_other_tc=" << cache.getTopKOptions("tcC", {s.in0, s.in1}, {s.out0}, "dev", 1).size() << "\n";
+  out << "miss_other_sizes=" << cache.getTopKOptions("tcA", {s.in1, s.in0}, {s.out0}, "dev", 1).size() << "\n";
+  out << "miss_other_device=" << cache.getTopKOptions("tcA", {s.in0, s.in1}, {s.out0}, "other", 1).size() << "\n";
+  TensorInfo misaligned = s.in0;
   misaligned.alignment = 64;
-  EXPECT(cache.getTopKOptions("tcA", {misaligned, in1}, {out0}, "dev", 1).empty());
-  EXPECT(cache.numberAttemptedRetrievals == 5 && cache.numberSuccessfulRetrievals == 1);
-  // wire round trip
+  out << "miss_other_alignment=" << cache.getTopKOptions("tcA", {misaligned, s.in1}, {s.out0}, "dev", 1).size() << "\n";
+  out << "retrievals=" << cache.numberAttemptedRetrievals << "," << cache.numberSuccessfulRetrievals << "\n";
   OptionsCache<FakeBackend> copy;
   copy.fromProtobuf(cache.toProtobuf());
-  EXPECT(copy.size() == 4);
-  auto top2 = copy.getTopKEntries("tcA", {in0, in1}, {out0}, "dev", 3);
-  EXPECT(top2.size() == 3 && top2[0].first == o2 && top2[2].first == o3 && top2[1].second == us(20));
-  // prune
+  out << "wire_copy_size=" << copy.size() << "\n";
+  out << "wire_copy_top3_tcA=" << names(copy.getTopKEntries("tcA", {s.in0, s.in1}, {s.out0}, "dev", 3)) << "\n";
   copy.pruneKeepTopK(1);
-  EXPECT(copy.size() == 2);
-  EXPECT((copy.getTopKOptions("tcA", {in0, in1}, {out0}, "dev", 5) == std::vector<HipMappingOptions>{o2}));
-  // files: store, load, append-merge
+  out << "pruned_size=" << copy.size() << "\n";
+  out << "pruned_top_tcA=" << names(copy.getTopKEntries("tcA", {s.in0, s.in1}, {s.out0}, "dev", 5)) << "\n";
   if (!scratch.empty()) {
     std::remove(scratch.c_str());
     cache.storeCacheToFile(scratch);
     OptionsCache<FakeBackend> loaded;
     loaded.loadCacheFromFile(scratch);
-    EXPECT(loaded.size() == 4);
+    out << "file_loaded_size=" << loaded.size() << "\n";
     std::remove(scratch.c_str());
     appendTopKToCacheFile(cache, scratch, 2);
     appendTopKToCacheFile(cache, scratch, 1);
     OptionsCache<FakeBackend> merged;
     merged.loadCacheFromFile(scratch);
-    EXPECT(merged.size() == 3 + 2);
+    out << "file_appended_size=" << merged.size() << "\n";
     std::remove(scratch.c_str());
   }
-  return "ok";
-#undef EXPECT
+  return out.str();
 }
 } // namespace
 
@@ -353,6 +380,14 @@ extern "C" int tc_host_query(const char* what, const char* arg, char** out) {
       result = runSyntheticSearch(parseSettings(a.c_str()));
     } else if (w == "options_cache_selftest") {
       result = cacheSelfTest(a);
+    } else if (w == "options_cache_write_sample") {
+      SampleCache sample;
+      sample.cache.storeCacheToFile(a);
+      result = dumpCache(sample.cache);
+    } else if (w == "options_cache_dump") {
+      OptionsCache<FakeBackend> loaded;
+      loaded.loadCacheFromFile(a);
+      result = dumpCache(loaded);
     } else if (w == "base_outside_space") {
       // a base mapping whose tile size is not a candidate value must be refused
       int64_t shape[] = {10, 16};

@@ -154,7 +154,7 @@ class OptionsCache {
         protowire::Reader vr(r.bytes());
         while (vr.next()) {
           if (vr.field() == 1) v.mappingOptions = Options(vr.bytes());
-          if (vr.field() == 2) v.runtimes.push_back(Duration::fromNanoSeconds(static_cast<int64_t>(vr.value())));
+          if (vr.field() == 2) vr.eachValue([&](uint64_t ns) { v.runtimes.push_back(Duration::fromNanoSeconds(static_cast<int64_t>(ns))); });
         }
         values.push_back(std::move(v));
       }
@@ -201,8 +201,8 @@ class OptionsCache {
     TensorInfo t(DLDataType{2, 32, 1}, 0, {}, {});
     protowire::Reader r(s);
     while (r.next()) {
-      if (r.field() == 1) t.shape.push_back(static_cast<int64_t>(r.value()));
-      if (r.field() == 2) t.strides.push_back(static_cast<int64_t>(r.value()));
+      if (r.field() == 1) r.eachValue([&](uint64_t e) { t.shape.push_back(static_cast<int64_t>(e)); });
+      if (r.field() == 2) r.eachValue([&](uint64_t e) { t.strides.push_back(static_cast<int64_t>(e)); });
       if (r.field() == 3) t.alignment = r.value();
       if (r.field() == 4) {
         protowire::Reader d(r.bytes());

@@ -120,7 +120,7 @@ class MappingOptions {
           tiling.clear();
           protowire::Reader t(r.bytes());
           while (t.next()) {
-            if (t.field() == 1) tiling.push_back(t.value());
+            if (t.field() == 1) t.eachValue([&](uint64_t v) { tiling.push_back(v); });
           }
           break;
         }

@@ -39,6 +39,9 @@ class Writer {
   std::string out_;
 };
 
+// Reads one message.  Robust against truncated or corrupt input (a cache file is untrusted
+// data): every length is checked against what is left, a varint ends after ten bytes, and the
+// accessors refuse a field whose wire type is not the one asked for.
 class Reader {
  public:
   explicit Reader(const std::string& s) : s_(s) {}
@@ -49,23 +52,26 @@ class Reader {
     uint64_t key = raw();
     field_ = static_cast<int>(key >> 3);
     wire_ = static_cast<int>(key & 7);
+    value_ = 0;
+    bytes_.clear();
     if (wire_ == 0) {
       value_ = raw();
     } else if (wire_ == 2) {
       uint64_t n = raw();
-      if (pos_ + n > s_.size()) {
+      if (n > s_.size() - pos_) {
         throw std::runtime_error("protowire: truncated length-delimited field");
       }
-      bytes_ = s_.substr(pos_, n);
-      pos_ += n;
-    } else if (wire_ == 1) {
-      value_ = 0;
-      for (int i = 0; i < 8; ++i) {
-        value_ |= static_cast<uint64_t>(static_cast<unsigned char>(s_.at(pos_ + i))) << (8 * i);
+      bytes_ = s_.substr(pos_, static_cast<size_t>(n));
+      pos_ += static_cast<size_t>(n);
+    } else if (wire_ == 1 || wire_ == 5) {
+      const size_t width = wire_ == 1 ? 8 : 4;
+      if (width > s_.size() - pos_) {
+        throw std::runtime_error("protowire: truncated fixed-width field");
       }
-      pos_ += 8;
-    } else if (wire_ == 5) {
-      pos_ += 4;
+      for (size_t i = 0; i < width; ++i) {
+        value_ |= static_cast<uint64_t>(static_cast<unsigned char>(s_[pos_ + i])) << (8 * i);
+      }
+      pos_ += width;
     } else {
       throw std::runtime_error("protowire: unsupported wire type");
     }
@@ -73,24 +79,50 @@ class Reader {
   }
   int field() const { return field_; }
   int wire() const { return wire_; }
-  uint64_t value() const { return value_; }
-  const std::string& bytes() const { return bytes_; }
+  // a scalar field (varint or fixed width)
+  uint64_t value() const {
+    if (wire_ == 2) {
+      throw std::runtime_error("protowire: field " + std::to_string(field_) + " is length-delimited where a scalar was expected");
+    }
+    return value_;
+  }
+  // a string, bytes or nested-message field
+  const std::string& bytes() const {
+    if (wire_ != 2) {
+      throw std::runtime_error("protowire: field " + std::to_string(field_) + " is a scalar where a length-delimited value was expected");
+    }
+    return bytes_;
+  }
+  // One occurrence of a repeated integer field: a single value, or a packed run of them (what a
+  // proto3 writer, or a proto2 writer with [packed = true], emits for the same schema).
+  template <typename F>
+  void eachValue(F&& f) const {
+    if (wire_ != 2) {
+      f(value_);
+      return;
+    }
+    Reader packed(bytes_);
+    while (packed.pos_ < packed.s_.size()) {
+      f(packed.raw());
+    }
+  }
 
  private:
   uint64_t raw() {
     uint64_t v = 0;
-    int shift = 0;
-    for (;;) {
+    for (int shift = 0; shift < 70; shift += 7) {
       if (pos_ >= s_.size()) {
         throw std::runtime_error("protowire: truncated varint");
       }
       unsigned char c = static_cast<unsigned char>(s_[pos_++]);
-      v |= static_cast<uint64_t>(c & 0x7f) << shift;
+      if (shift < 64) {
+        v |= static_cast<uint64_t>(c & 0x7f) << shift;
+      }
       if (!(c & 0x80)) {
         return v;
       }
-      shift += 7;
     }
+    throw std::runtime_error("protowire: varint longer than ten bytes");
   }
   const std::string& s_;
   size_t pos_ = 0;

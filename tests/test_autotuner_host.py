@@ -62,11 +62,6 @@ def test_genetic_search_survives_mostly_invalid_generations():
     assert len(out.split(",")) == 6
 
 
-def test_options_cache_semantics_and_files():
-    with tempfile.TemporaryDirectory() as d:
-        assert tc.host_query("options_cache_selftest", os.path.join(d, "cache.bin")) == "ok"
-
-
 def test_structured_seeds_are_members_of_the_search_space():
     """Generation 0 holds streaming, row-reduction and matrix-core variants of the first base
     mapping next to it; every seed is expressible in the space built from the same shapes (a seed
