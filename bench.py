@@ -311,6 +311,8 @@ def main():
                     help="back-to-back launches for this long before the warm-up steps (device clocks)")
     ap.add_argument("--tune", default=None, metavar="GENERATIONSxPOPULATION",
                     help="autotune the workload from the naive options first (e.g. 5x40) and measure the best")
+    ap.add_argument("--tune-settings", default="", metavar="KEY=VALUE;...",
+                    help="further tuner settings for --tune (seed_heuristics=0, refinement_rounds=0, seed=3, ...)")
     ap.add_argument("--suite", action="store_true",
                     help="also time the reference's other benchmark comprehensions at their default sizes")
     ap.add_argument("--no-cpu", action="store_true")
@@ -335,7 +337,9 @@ def main():
         src, entry = W.CONFIGS[a.config][0], W.CONFIGS[a.config][1]
         ins = [to_device(x) for x in W.make_inputs(a.config)]
         t0 = time.perf_counter()
-        best = tc.autotune(src, entry, ins, "naive", generations=gens, pop_size=pop, threads=16, seed=1, top_k=1)
+        settings = {"generations": gens, "pop_size": pop, "threads": 16, "seed": 1, "top_k": 1}
+        settings.update(kv.split("=", 1) for kv in a.tune_settings.split(";") if kv)
+        best = tc.autotune(src, entry, ins, "naive", **settings)
         tuned_in = time.perf_counter() - t0
         if not best:
             sys.exit("the autotuner found no runnable candidate")
@@ -354,7 +358,8 @@ def main():
         "device": tc.device_name(),
     }
     if tuned_in is not None:
-        line["config"]["options_from"] = f"autotuned from the naive options, {a.tune} candidates, {tuned_in:.0f} s"
+        line["config"]["options_from"] = (f"autotuned from the naive options, {a.tune} candidates, {tuned_in:.0f} s"
+                                          + (f", {a.tune_settings}" if a.tune_settings else ""))
     if not a.no_cpu:
         line["cpu_baseline"] = cpu_baseline(a.config, m["bytes"])
         line["cpu_baseline"]["host_cores"] = os.cpu_count()

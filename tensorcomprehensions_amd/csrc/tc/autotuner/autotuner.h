@@ -52,6 +52,10 @@ struct TunerSettings {
   // after the last generation: rounds of one-gene steps around the best candidate (every gene
   // moved to its neighbouring values, one at a time); a round that finds nothing better ends it
   size_t refinementRounds = 2;
+  // Options the mapper of this backend gives no meaning to (fixParametersBeforeScheduling,
+  // tileImperfectlyNested, privateDepth: they exist for the reference's isl scheduler and its
+  // promotion heuristic) keep the value of the first base mapping instead of being searched.
+  bool fixInertParameters = true;
 };
 
 namespace detail {
@@ -289,6 +293,12 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
   }
   TuningConfiguration space = detail::setupTuningParameters(firstInputs, bases, settings.maxUnroll, outputSizes);
   space.fixParameters(fixedParams);
+  if (settings.fixInertParameters) {
+    const auto& b0 = bases.front();
+    space.fixParametersBeforeScheduling.fixValue(b0.generic.fixParametersBeforeSchedulingValue);
+    space.tileImperfectlyNested.fixValue(b0.generic.tileImperfectlyNestedValue);
+    space.privateDepth.fixValue(b0.privateDepthValue);
+  }
   std::vector<TuningConfiguration> configs;
   for (const auto& b : bases) {
     TuningConfiguration c = space;
@@ -340,37 +350,75 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
   const char* traceEnv = std::getenv("TC_TUNER_TRACE");
   const bool trace = traceEnv != nullptr && traceEnv[0] != '\0' && traceEnv[0] != '0';
   using Population = std::vector<std::unique_ptr<CandidateConfiguration>>;
+  // Different option sets often map to the very same kernels (an option that does not apply to
+  // this TC, a tile size beyond an extent, a thread count the mapper tightens): a mapping is
+  // compiled and measured once per tuning run, and every later candidate that maps to the same
+  // source and launch shapes takes over its result.
+  struct Outcome {
+    bool done = false, invalid = false;
+    Duration runtime = Duration::zero();
+  };
+  std::map<std::string, std::shared_ptr<Outcome>> outcomes; // guarded by `mu` of the population under evaluation
+  size_t duplicates = 0;
+  const ir::Function function = tc::detail::translate(tree, firstInputs, quiet);
+  tc::detail::checkInputsCompliant(function, firstInputs);
   // compiles (worker threads) and measures (this device) every candidate of `population`;
   // returns the runtimes of the valid ones
   auto evaluatePopulation = [&](Population& population) {
     std::atomic<size_t> cursor{0};
     std::mutex mu;
     std::condition_variable cv;
-    std::deque<std::pair<std::unique_ptr<ExecutorType>, CandidateConfiguration*>> ready;
+    struct Job {
+      std::unique_ptr<ExecutorType> executor;   // null: failed to compile, or a duplicate
+      CandidateConfiguration* candidate = nullptr;
+      std::shared_ptr<Outcome> outcome;         // null: failed to compile
+      bool duplicate = false;
+    };
+    std::deque<Job> ready;
     size_t produced = 0;
 
     auto compileWorker = [&]() {
       for (;;) {
         size_t i = cursor.fetch_add(1);
         if (i >= population.size() || detail::tunerSignal == SIGTERM) return;
-        CandidateConfiguration* cand = population[i].get();
-        std::unique_ptr<ExecutorType> ex;
+        Job job;
+        job.candidate = population[i].get();
         try {
           MappingOptionsType options = baseMapping;
-          cand->configuration.applyToHipMappingOptions(options);
+          job.candidate->configuration.applyToHipMappingOptions(options);
           if (trace) {
             std::lock_guard<std::mutex> lock(mu);
             std::cerr << "[tuner] " << std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count()
                       << " compiling " << options.toText() << std::endl;
           }
-          ex = tc::detail::compile<Backend>(tree, firstInputs, options, quiet);
+          auto mapped = Backend::compileWithTcMapper(function.name, function, firstInputs, options);
+          std::string key = mapped.source;
+          for (const auto& k : mapped.kernels) {
+            for (int a = 0; a < 3; ++a) key += "|" + std::to_string(k.grid[a]) + "," + std::to_string(k.block[a]);
+          }
+          {
+            std::lock_guard<std::mutex> lock(mu);
+            auto found = outcomes.find(key);
+            if (found != outcomes.end()) {
+              job.outcome = found->second;
+              job.duplicate = true;
+              ++duplicates;
+            } else {
+              job.outcome = outcomes.emplace(key, std::make_shared<Outcome>()).first->second;
+            }
+          }
+          if (!job.duplicate) job.executor = tc::detail::makeExecutor<Backend>(function, firstInputs, mapped);
         } catch (const std::exception& e) {
           if (settings.verbose) std::cerr << "[tuner] candidate failed to compile: " << e.what() << std::endl;
-          ex.reset();
+          job.executor.reset();
+          if (job.outcome && !job.duplicate) {
+            std::lock_guard<std::mutex> lock(mu);
+            job.outcome->done = job.outcome->invalid = true;
+          }
         }
         {
           std::lock_guard<std::mutex> lock(mu);
-          ready.emplace_back(std::move(ex), cand);
+          ready.push_back(std::move(job));
           ++produced;
         }
         cv.notify_one();
@@ -383,8 +431,31 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
       const auto& ins = inputs.at(device);
       const auto& outs = outputs.at(device);
       size_t consumed = 0;
+      std::vector<Job> duplicateJobs; // settled once every original of this population has run
+      // marks the mapping's outcome when the job goes out of scope, whichever way
+      struct Settle {
+        Job& job;
+        std::mutex& mu;
+        ~Settle() {
+          if (!job.outcome || job.duplicate) return;
+          std::lock_guard<std::mutex> lock(mu);
+          job.outcome->done = true;
+          job.outcome->invalid = job.candidate->invalid;
+          job.outcome->runtime = job.candidate->runtime;
+        }
+      };
+      struct SettleDuplicates {
+        std::vector<Job>& jobs;
+        ~SettleDuplicates() {
+          for (auto& j : jobs) {
+            // (an original that never ran, e.g. after an abort, leaves its duplicates invalid)
+            j.candidate->invalid = !j.outcome->done || j.outcome->invalid;
+            j.candidate->runtime = j.outcome->runtime;
+          }
+        }
+      } settleDuplicates{duplicateJobs};
       while (consumed < population.size()) {
-        std::pair<std::unique_ptr<ExecutorType>, CandidateConfiguration*> job;
+        Job job;
         {
           std::unique_lock<std::mutex> lock(mu);
           cv.wait(lock, [&] { return !ready.empty() || detail::tunerSignal == SIGTERM; });
@@ -393,12 +464,17 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
           ready.pop_front();
         }
         ++consumed;
-        CandidateConfiguration* cand = job.second;
-        if (!job.first) {
+        CandidateConfiguration* cand = job.candidate;
+        if (job.duplicate) {
+          duplicateJobs.push_back(std::move(job));
+          continue;
+        }
+        Settle settle{job, mu};
+        if (!job.executor) {
           cand->invalid = true;
           continue;
         }
-        ExecutorType& ex = *job.first;
+        ExecutorType& ex = *job.executor;
         if (trace) {
           MappingOptionsType options = baseMapping;
           cand->configuration.applyToHipMappingOptions(options);
@@ -471,7 +547,7 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
     if (settings.verbose || flags().tuner_gen_log_generations) {
       std::sort(generationTimes.begin(), generationTimes.end());
       std::cerr << "[tuner] " << what << ": " << generationTimes.size() << "/" << size
-                << " valid";
+                << " valid, " << duplicates << " duplicate mappings so far";
       if (!generationTimes.empty()) {
         std::cerr << " (best/median/worst) " << generationTimes.front().toMicroSecondsF() << "/"
                   << generationTimes[generationTimes.size() / 2].toMicroSecondsF() << "/"

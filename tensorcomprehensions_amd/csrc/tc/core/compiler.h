@@ -28,6 +28,22 @@ ir::Function translate(
 std::vector<TensorInfo> inferOutputTensorInfo(
     const lang::TreeRef& def, const std::vector<const DLConstTensor*>& inputs, const CompilerOptions& options);
 
+// The executor of a mapped function: JIT-compiles `result` (the second half of compile(), for
+// callers that look at the mapper's output before they decide to compile it).
+template <typename Backend>
+std::unique_ptr<typename Backend::ExecutorType> makeExecutor(
+    const ir::Function& f,
+    const std::vector<const DLConstTensor*>& inputs,
+    const typename Backend::CompilationResultType& result) {
+  std::vector<TensorInfo> inputsInfo = makeTensorInfoVector(inputs);
+  std::vector<TensorInfo> outputsInfo;
+  for (const auto& o : f.outputs) {
+    outputsInfo.emplace_back(o.type.toDL(), 0, o.extents, makeStridesFromSizes(o.extents));
+  }
+  return std::unique_ptr<typename Backend::ExecutorType>(
+      new typename Backend::ExecutorType(inputsInfo, outputsInfo, f, result));
+}
+
 template <typename Backend>
 std::unique_ptr<typename Backend::ExecutorType> compile(
     const lang::TreeRef& def,
@@ -36,14 +52,7 @@ std::unique_ptr<typename Backend::ExecutorType> compile(
     const CompilerOptions& compilerOptions = CompilerOptions()) {
   ir::Function f = translate(def, inputs, compilerOptions);
   checkInputsCompliant(f, inputs);
-  std::vector<TensorInfo> inputsInfo = makeTensorInfoVector(inputs);
-  std::vector<TensorInfo> outputsInfo;
-  for (const auto& o : f.outputs) {
-    outputsInfo.emplace_back(o.type.toDL(), 0, o.extents, makeStridesFromSizes(o.extents));
-  }
-  auto result = Backend::compileWithTcMapper(f.name, f, inputs, options);
-  return std::unique_ptr<typename Backend::ExecutorType>(
-      new typename Backend::ExecutorType(inputsInfo, outputsInfo, f, result));
+  return makeExecutor<Backend>(f, inputs, Backend::compileWithTcMapper(f.name, f, inputs, options));
 }
 
 } // namespace detail

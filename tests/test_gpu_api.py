@@ -237,3 +237,34 @@ def test_device_buffers_stand_in_for_tensors():
     ref = tc_oracle.run(src, entry, ins_np)[0]
     assert np.abs(outs[0].numpy() - ref).max() <= W.tolerance(k, ref)
     assert "MI3" in tc.device_name() or "AMD" in tc.device_name()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["c2_tensordot", "c5_moments"])
+def test_autotune_from_the_naive_options_reaches_the_stored_options(name):
+    """What 'after autotuning' means for the benchmark configurations: a short, seeded search that
+    starts from the naive options ends within 15 % of the options the benchmark stores, and its
+    winner computes the oracle's values (test/cuda/test_autotuner.cc:43-51 tunes and runs;
+    tc/autotuner/autotuner-inl.h:418-518)."""
+    src, entry, _, _, k = W.CONFIGS[name]
+    ins_np = W.make_inputs(name)
+    ins = [torch.from_numpy(a).cuda() for a in ins_np]
+    outs = tc.prepare_outputs(src, entry, ins)
+
+    def kernel_us(options):
+        ex = tc.compile(src, entry, ins, options)
+        tc.profile_repeated(ex, ins, outs, 200)
+        return min(tc.profile_repeated(ex, ins, outs, 50) / 50 for _ in range(5))
+
+    best = tc.autotune(src, entry, ins, "naive", outputs=outs, generations=3, pop_size=30, threads=16, seed=1)
+    assert len(best) == 1
+    t_stored, t_tuned, t_naive = kernel_us(W.TUNED[name]), kernel_us(best[0]), kernel_us("naive")
+    print(f"{name}: naive {t_naive:.1f} us, stored {t_stored:.1f} us, tuned from naive {t_tuned:.1f} us with {best[0]}", flush=True)
+    assert t_tuned <= 1.15 * t_stored
+    ex = tc.compile(src, entry, ins, best[0])
+    for o in outs:
+        o.fill_(float("nan"))
+    tc.run(ex, ins, outs)
+    torch.cuda.synchronize()
+    for o, r in zip(outs, tc_oracle.run(src, entry, ins_np)):
+        assert np.abs(o.cpu().numpy() - r).max() <= W.tolerance(k, r)
