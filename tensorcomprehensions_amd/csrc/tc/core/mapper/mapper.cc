@@ -392,6 +392,26 @@ void emitKernel(KernelCtx& kc, const DeviceLimits& limits, Emitter& em) {
     gens.emplace_back(kc, k.stages[i], static_cast<int>(i), em);
     gens.back().plan(ldsBudget);
   }
+  // One copy per kernel: a later stage whose footprint of a tensor is the one an earlier stage has
+  // staged (same box, same origin, fixed for the whole kernel-level iteration) reads the earlier
+  // stage's array.  Staged tensors are inputs of the TC, so nothing in the kernel changes them.
+  {
+    std::map<std::string, std::string> staged; // footprint key -> LDS array of the first stage that stages it
+    for (size_t i = 0; i < gens.size(); ++i) {
+      for (auto& p : gens[i].mutablePromotions()) {
+        if (!gens[i].footprintFixedPerKernelIteration(p)) continue;
+        std::string key = gens[i].footprintKey(p);
+        auto found = staged.find(key);
+        if (found == staged.end()) {
+          staged.emplace(key, p.ldsName);
+        } else {
+          p.sharedWithEarlierStage = true;
+          p.ldsName = found->second;
+          ldsBudget += p.elems * k.stages[i].views.at(p.tensor).type.bytes();
+        }
+      }
+    }
+  }
   k.ldsBytes = (before - ldsBudget) + scratchElems * 8;
 
   // Register promotion across stages (usePrivateMemory): an input that several stages read with

@@ -63,6 +63,9 @@ struct Promotion {
   int64_t elems = 0;                 // LDS elements including padding
   int64_t reuse = 1;                 // accesses per staged element
   bool insideReductionTiles = false;
+  // An earlier stage of the kernel staged the very same footprint and nothing has overwritten it:
+  // this stage reads that copy (`ldsName` names the earlier stage's array) and copies nothing.
+  bool sharedWithEarlierStage = false;
 };
 
 // One statement of a stage, rewritten on the stage's variables and tensor views.

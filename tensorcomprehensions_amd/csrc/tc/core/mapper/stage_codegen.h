@@ -336,7 +336,8 @@ class StageCodegen {
   }
 
   void planPromotions(const StageStmt& s, int64_t& ldsBudgetBytes) {
-    if (!kc_.opts.useSharedMemoryValue || s.redVars.empty()) return;
+    if (!kc_.opts.useSharedMemoryValue) return;
+    if (s.redVars.empty() && st_.mfma) return;
     for (const auto& v : st_.vars) {
       if (!st_.mfma && !v.reduction && !v.unrolled && v.perThread > 1) return; // needs a full register tile
     }
@@ -502,6 +503,7 @@ class StageCodegen {
 
   void emitLdsDecls() {
     for (const auto& p : st_.promotions) {
+      if (p.sharedWithEarlierStage) continue;
       em_.line("__shared__ __attribute__((aligned(16))) " + st_.views.at(p.tensor).type.cName() + " " + p.ldsName +
                "[" + std::to_string(p.elems) + "];");
     }
@@ -824,6 +826,43 @@ class StageCodegen {
 
   // --- statements -----------------------------------------------------------------------------
   void emitPointwise(const StageStmt& s) {
+    const bool staged = &s == promotedPointwise_;
+    if (staged) {
+      em_.open("");
+      stageOutsideFootprints();
+    }
+    emitPointwiseBody(s);
+    if (staged) {
+      for (const auto& p : st_.promotions) activePromotions_.erase(p.tensor);
+      em_.close();
+    }
+  }
+
+  // Copies the stage's footprints of one kind (inside / outside the reduction tile loop) into LDS,
+  // between two barriers, and makes the statement's loads read them; footprints an earlier stage
+  // has staged are only addressed.  The barrier in front protects the readers of what the arrays
+  // held before: there are none ahead of the first copy of the first stage of a kernel without
+  // kernel-level loops.
+  void stageFootprints(bool inside) {
+    std::vector<const Promotion*> group;
+    for (const auto& p : st_.promotions) {
+      if (p.insideReductionTiles != inside) continue;
+      activePromotions_.insert(p.tensor);
+      if (p.sharedWithEarlierStage) {
+        declareLows(p);
+      } else {
+        group.push_back(&p);
+      }
+    }
+    if (group.empty()) return;
+    if (inside || stageIdx_ > 0 || kc_.kernelLoops || stageTileLoops_ || copiedBefore_) em_.line("__syncthreads();");
+    copiedBefore_ = true;
+    emitCopyInGroup(group);
+    em_.line("__syncthreads();");
+  }
+  void stageOutsideFootprints() { stageFootprints(false); }
+
+  void emitPointwiseBody(const StageStmt& s) {
     int n = openUnrolled();
     inCachedReduction_ = cachedPointwise_;
     cacheSlot_ = "a_";
@@ -875,16 +914,7 @@ class StageCodegen {
         }
         return;
       }
-      em_.line("__syncthreads();");
-      std::vector<const Promotion*> group;
-      for (const auto& p : st_.promotions) {
-        if (p.insideReductionTiles == inside) {
-          group.push_back(&p);
-          activePromotions_.insert(p.tensor);
-        }
-      }
-      emitCopyInGroup(group);
-      em_.line("__syncthreads();");
+      stageFootprints(inside);
     };
     int opened = 0;
     if (anyOutside) {
@@ -1179,14 +1209,52 @@ class StageCodegen {
   }
 
   // --- whole stage ----------------------------------------------------------------------------
+  // Footprints are planned for the stage's reduction statement; a stage without one (a stencil,
+  // say: several accesses per element through overlapping windows) plans them for its first
+  // statement that loads anything.
   void plan(int64_t& ldsBudgetBytes) {
     for (const auto& s : st_.stmts) {
       if (!s.redVars.empty()) {
         planPromotions(s, ldsBudgetBytes);
-        break;
+        return;
+      }
+    }
+    for (const auto& s : st_.stmts) {
+      bool loads = false;
+      visit(s.rhs, [&](const ExprRef& e) { loads |= e->kind == Expr::Load && e->name != st_.tensor; });
+      if (loads) {
+        planPromotions(s, ldsBudgetBytes);
+        promotedPointwise_ = st_.promotions.empty() ? nullptr : &s;
+        return;
       }
     }
   }
+
+  // The footprint origins of promotion `p` as text, for comparing the footprints of two stages.
+  std::string footprintKey(const Promotion& p) const {
+    std::ostringstream ss;
+    ss << p.tensor << (p.insideReductionTiles ? "|inside" : "|outside");
+    for (size_t j = 0; j < p.extents.size(); ++j) ss << "|" << p.extents[j] << ":" << p.ldsStrides[j] << ":" << footprintLow(p, j);
+    return ss.str();
+  }
+  // Whether every footprint origin is fixed by the block ids and the kernel-level tile loops: the
+  // staged data then stays valid from one stage of a kernel-level iteration to the next.
+  bool footprintFixedPerKernelIteration(const Promotion& p) const {
+    if (p.insideReductionTiles) return false;
+    const Footprint& fp = footprints_.at(p.tensor);
+    for (const auto& dim : fp.coefs) {
+      for (const auto& c : dim.coef) {
+        if (c.second == 0) continue;
+        const LoopVar& v = var(c.first);
+        if (v.reduction || v.numTiles == 1) continue;
+        bool kernelLevel = false;
+        for (int i = 0; i < kc_.k.sharedDepth && i < st_.numParallel; ++i) kernelLevel |= st_.vars[i].name == v.name;
+        if (!kernelLevel) return false;
+      }
+    }
+    return true;
+  }
+  std::vector<Promotion>& mutablePromotions() { return st_.promotions; }
 
   // Declares i_<v> (and p_<v>) for every variable of `group` from the flattened position `pos`
   // inside the block tile (row-major over the group's tile extents, last variable fastest) and
@@ -1402,16 +1470,7 @@ class StageCodegen {
         }
         return;
       }
-      // (nothing has touched LDS before the first stage of a kernel without kernel-level loops)
-      if (inside || stageIdx_ > 0 || kc_.kernelLoops || stageTileLoops_) em_.line("__syncthreads();");
-      std::vector<const Promotion*> group;
-      for (const auto& p : st_.promotions) {
-        if (p.insideReductionTiles != inside) continue;
-        group.push_back(&p);
-        activePromotions_.insert(p.tensor);
-      }
-      emitCopyInGroup(group);
-      em_.line("__syncthreads();");
+      stageFootprints(inside);
     };
     // decodes the output tile tl_ of this wavefront: batch and column indices, nok_
     auto decodeTile = [&]() {
@@ -1715,6 +1774,8 @@ class StageCodegen {
   std::map<std::string, std::string> hoistedLoads_; // printed global load -> register holding it
   bool inCachedReduction_ = false;
   bool stageTileLoops_ = false; // the stage's code sits inside tile loops of its own
+  bool copiedBefore_ = false;   // this stage has already written LDS once
+  const StageStmt* promotedPointwise_ = nullptr; // statement of a reduction-free stage that reads staged footprints
   std::string cacheSlot_;
   int clampId_ = 0;
 };

@@ -1,0 +1,72 @@
+"""LDS promotion beyond the reduction operands of one stage, against the oracle: a footprint two
+stages of a kernel share, a stage without a reduction (overlapping windows), copies whose last
+block-wide step is ragged or whose loops overshoot."""
+import numpy as np
+import pytest
+import torch
+
+import tensorcomprehensions_amd as tc
+from oracle import tc_oracle
+from tests import workloads as W
+from tests.test_mapper import STENCIL, TWO_CONVOLUTIONS
+
+pytestmark = pytest.mark.gpu
+
+
+def run(src, entry, ins_np, options):
+    ins = [torch.from_numpy(a).cuda() for a in ins_np]
+    ex = tc.compile(src, entry, ins, options)
+    outs = tc.prepare_outputs(src, entry, ins)
+    for o in outs:
+        o.fill_(float("nan"))
+    tc.run(ex, ins, outs)
+    torch.cuda.synchronize()
+    return [o.cpu().numpy() for o in outs], ex
+
+
+@pytest.mark.parametrize("options", [
+    "naive;tile=1,8,10,10;mapToThreads=10,10;mapToBlocks=4;unroll=8;useSharedMemory=1;outerScheduleFusionStrategy=Max",
+    "naive;tile=2,4,5,10;mapToThreads=10,5;mapToBlocks=2,2,2;unroll=8;useSharedMemory=1;outerScheduleFusionStrategy=Max",
+    "naive;tile=1,8,10,10;mapToThreads=10,10;mapToBlocks=2;unroll=8;useSharedMemory=1;outerScheduleFusionStrategy=Max",   # kernel-level loop over n
+    "naive;tile=1,8,0,0;mapToThreads=64,4;mapToBlocks=4;useMfma=1;useSharedMemory=1;outerScheduleFusionStrategy=Max",
+])
+def test_two_convolutions_over_one_staged_input(options):
+    rng = np.random.Generator(np.random.Philox(41))
+    ins = [rng.integers(-3, 4, size=s).astype(np.float32) for s in [(4, 3, 12, 12), (8, 3, 3, 3), (8, 3, 3, 3)]]
+    got, ex = run(TWO_CONVOLUTIONS, "two", ins, options)
+    ref = tc_oracle.run(TWO_CONVOLUTIONS, "two", ins)
+    torch_ref = [torch.nn.functional.conv2d(torch.from_numpy(ins[0]), torch.from_numpy(w)).numpy() for w in ins[1:]]
+    for g, r, t in zip(got, ref, torch_ref):
+        assert np.array_equal(r, t)                       # small integers: exact whatever the order
+        assert np.array_equal(g, r), (options, ex.launch_bounds())
+
+
+@pytest.mark.parametrize("options", [
+    "naive;tile=8,64;mapToThreads=64,2;mapToBlocks=16,16;unroll=4;useSharedMemory=1",
+    "naive;tile=8,64;mapToThreads=64,2;mapToBlocks=3,2;unroll=4;useSharedMemory=1",          # blocks loop over tiles
+    "naive;tile=16,32;mapToThreads=32,4;mapToBlocks=16,16;unroll=8;useSharedMemory=1;vectorWidth=2",
+    "naive;tile=5,7;mapToThreads=7,5;mapToBlocks=32,32;unroll=1;useSharedMemory=1",
+])
+def test_stencil_through_lds(options):
+    A = np.random.Generator(np.random.Philox(42)).standard_normal((100, 200), dtype=np.float32)
+    (got,), ex = run(STENCIL, "blur", [A], options)
+    (ref,) = tc_oracle.run(STENCIL, "blur", [A])
+    assert "lds0_A" in ex.compiled_source, options
+    assert got.shape == (99, 198)
+    assert np.abs(got - ref).max() <= W.tolerance(6, ref)
+    closed = (A[:-1, :-2] + A[:-1, 1:-1] + A[:-1, 2:] + A[1:, :-2] + A[1:, 1:-1] + A[1:, 2:]) / 6.0
+    assert np.abs(ref - closed).max() <= W.tolerance(6, ref)
+
+
+@pytest.mark.parametrize("threads,shapes", [((19, 2), [(5, 26, 40), (5, 40, 19)]), ((32, 3), [(3, 33, 48), (3, 48, 37)]),
+                                            ((64, 1), [(2, 70, 25), (2, 25, 90)])])
+def test_staging_copies_whose_loops_overshoot_the_footprint(threads, shapes):
+    """A chunked copy loop runs more iterations than the footprint needs, and the last needed one
+    is ragged: nothing may be written past the LDS array (batched matmul, whole batch per block)."""
+    rng = np.random.Generator(np.random.Philox(43))
+    ins = [rng.integers(-3, 4, size=s).astype(np.float32) for s in shapes]
+    options = f"naive;tile=64,5;mapToThreads={threads[0]},{threads[1]};mapToBlocks=16;unroll=64;useSharedMemory=1;vectorWidth=4"
+    got, ex = run(W.BATCH_MATMUL, "batch_matmul", ins, options)
+    (ref,) = tc_oracle.run(W.BATCH_MATMUL, "batch_matmul", ins)
+    assert ex.lds_bytes() > 0
+    assert np.array_equal(got[0], ref) and np.array_equal(ref, np.matmul(ins[0], ins[1]))

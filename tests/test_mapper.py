@@ -77,7 +77,11 @@ def test_lds_promotion_footprints():
     # per block: X[1][26][72] and Y[1][72][26] (footprint = min(tile, size) per dimension)
     assert "float lds0_X[1872];" in src
     assert re.search(r"float lds0_Y\[(1872|1944)\];", src)
-    assert src.count("__syncthreads();") >= 2                 # before and after the copies
+    # a barrier after the copies; none before them: nothing has read LDS ahead of the first copy of
+    # a kernel whose blocks do not loop over tiles
+    assert src.count("__syncthreads();") == 1
+    looped, _ = mapped(W.BATCH_MATMUL, "batch_matmul", [(500, 26, 72), (500, 72, 26)], o.mapToBlocks(100))
+    assert looped.count("__syncthreads();") == 2              # the next tile's copy waits for this tile's readers
     # without the switch nothing is staged
     src, _ = mapped(W.BATCH_MATMUL, "batch_matmul", [(500, 26, 72), (500, 72, 26)], o.useSharedMemory(False))
     assert "__shared__" not in src
@@ -279,3 +283,43 @@ def test_tuned_options_of_the_five_workloads_compile_with_the_expected_launches(
         src, entry, shapes = W.CONFIGS[name][0], W.CONFIGS[name][1], W.CONFIGS[name][2]
         ex = tc.compile(src, entry, [ShapeOnly(s) for s in shapes], W.TUNED[name])
         assert [ex.launch_bounds(k) for k in range(ex.num_kernels)] == launches, name
+
+
+TWO_CONVOLUTIONS = """
+def two(float(N,C,H,W) I, float(O,C,KH,KW) W1, float(O,C,KH,KW) W2) -> (A, B) {
+    A(n, o, h, w) +=! I(n, c, h + kh, w + kw) * W1(o, c, kh, kw)
+    B(n, o, h, w) +=! I(n, c, h + kh, w + kw) * W2(o, c, kh, kw)
+}
+"""
+STENCIL = ("def blur(float(N, M) A) -> (O) { O(i, j) = (A(i, j) + A(i, j + 1) + A(i, j + 2) + "
+           "A(i + 1, j) + A(i + 1, j + 1) + A(i + 1, j + 2)) / 6.0 }")
+
+
+def test_stages_of_a_kernel_share_one_staged_copy_of_a_footprint():
+    """Two stages that read the same window of the same input (the reference forms one reference
+    group per tensor and scope, tc/core/polyhedral/memory_promotion.cc:63-321): one LDS array, one
+    copy, the second stage only addresses it."""
+    options = "naive;tile=1,8,10,10;mapToThreads=10,10;mapToBlocks=4;unroll=8;useSharedMemory=1;outerScheduleFusionStrategy=Max"
+    src, launches = mapped(TWO_CONVOLUTIONS, "two", [(4, 3, 12, 12), (8, 3, 3, 3), (8, 3, 3, 3)], options)
+    assert len(launches) == 1
+    assert src.count("__shared__") == 1 and "lds0_I[432]" in src and "lds1_I" not in src
+    assert len(re.findall(r"lds0_I\[[^\]]*\] = stage_", src)) == 1          # copied once
+    stage1 = src[src.index("// stage 1: B"):]
+    assert "lds0_I[" in stage1 and "pI[" not in stage1                         # read from the shared copy
+    # kept apart, each kernel stages its own
+    src2, launches2 = mapped(TWO_CONVOLUTIONS, "two", [(4, 3, 12, 12), (8, 3, 3, 3), (8, 3, 3, 3)],
+                             options.replace("outerScheduleFusionStrategy=Max", "outerScheduleFusionStrategy=Min"))
+    assert len(launches2) == 2 and src2.count("__shared__") == 2
+
+
+def test_a_stage_without_a_reduction_stages_overlapping_windows():
+    """Promotion is decided by reuse, not by the kind of statement: six accesses per element of a
+    (tile + halo) window (memory_promotion_heuristic.cc:211-244, 'has reuse')."""
+    options = "naive;tile=8,64;mapToThreads=64,2;mapToBlocks=16,16;unroll=4;useSharedMemory=1"
+    src, _ = mapped(STENCIL, "blur", [(100, 200)], options)
+    assert "__shared__ __attribute__((aligned(16))) float lds0_A[594];" in src           # (8 + 1) x (64 + 2)
+    body = src[src.index("acc_[a_] = ("):]
+    assert body.count("lds0_A[") >= 6 and "pA[" not in body.split("\n")[0]
+    # no reuse, no staging
+    src2, _ = mapped(ADD, "fun", [(100, 200), (100, 200)], options)
+    assert "__shared__" not in src2
