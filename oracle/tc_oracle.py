@@ -38,6 +38,7 @@ from __future__ import annotations
 
 import ctypes
 import hashlib
+import tempfile
 import math
 import os
 import re
@@ -923,15 +924,18 @@ _CFLAGS = ["-O3", "-ffp-contract=off", "-fno-fast-math", "-shared", "-fPIC"]
 _cache: Dict[str, ctypes.CDLL] = {}
 
 
-def build(an: Analysis, native: bool = False) -> ctypes.CDLL:
-    """Compile the nest.  `native=True` adds -march=native and keeps the library in a per-host
-    temporary directory (a library tuned for one CPU must not travel to another machine)."""
+def build(an: Analysis, native: bool = False, in_tree: bool = False) -> ctypes.CDLL:
+    """Compile the nest.  The library goes to a per-host temporary directory (hundreds of test
+    nests do not belong next to the sources, and one built with `native=True`, i.e. -march=native,
+    must not travel to another machine); `in_tree=True` keeps it under oracle/_build instead (the
+    build check of the benchmark configurations)."""
     src = emit_c(an)
     flags = _CFLAGS + (["-march=native"] if native else [])
     key = hashlib.sha1((src + " ".join(flags)).encode()).hexdigest()[:16]
     if key in _cache:
         return _cache[key]
-    bdir = os.path.join("/tmp", "tc_oracle_native") if native else _BUILD_DIR
+    tmp_root = os.environ.get("TC_ORACLE_BUILD_DIR") or os.path.join(tempfile.gettempdir(), f"tc_oracle_{os.getuid()}")
+    bdir = _BUILD_DIR if in_tree else os.path.join(tmp_root, "native" if native else "portable")
     os.makedirs(bdir, exist_ok=True)
     so = os.path.join(bdir, f"oracle_{an.d.name}_{key}.so")
     if not os.path.exists(so):

@@ -194,27 +194,29 @@ TUNED_AT_REFERENCE_SIZES = {
     # 54 threads along w; hand-set: the search's thread counts do not contain 54 x 9
     "group_convolution": "naive;tile=1,1,4,27,0;mapToThreads=54,9;mapToBlocks=32,32,8;useSharedMemory=1;unroll=16;"
                          "useReadOnlyCache=1",
-    "tmm": "naive;tile=64,2;unroll=2;matchLibraryCalls=1;mapToThreads=128,1;mapToBlocks=256,1;usePrivateMemory=1;"
-           "unrollCopyShared=1;useReadOnlyCache=1;vectorWidth=2;collapseContiguous=0;useMfma=1;prefetchShared=1",
+    "tmm": "naive;tile=1,32,0;unroll=128;matchLibraryCalls=1;mapToThreads=64,4,4;mapToBlocks=256,256;"
+           "useSharedMemory=1;unrollCopyShared=1;useReadOnlyCache=1;sharedDepth=2;vectorWidth=2;useMfma=1;"
+           "prefetchShared=1",
     "matmul": "naive;intraTileScheduleFusionStrategy=Max;tile=16,32;unroll=256;matchLibraryCalls=1;mapToThreads=512,2;"
               "mapToBlocks=125,1000;unrollCopyShared=1;useReadOnlyCache=1;useMfma=1;prefetchShared=1",
     "convolution": "naive;intraTileScheduleFusionStrategy=Min;fixParametersBeforeScheduling=1;tile=1,27,1,0;unroll=128;"
                    "tileImperfectlyNested=1;mapToThreads=256,1;mapToBlocks=256,64,1;useSharedMemory=1;useReadOnlyCache=1;"
                    "collapseContiguous=0",
-    "2fcrelu": "naive;outerScheduleFusionStrategy=Min;fixParametersBeforeScheduling=1;tile=1,32;unroll=256;mapToThreads=64;"
-               "mapToBlocks=2000,256;useSharedMemory=1;useReadOnlyCache=1;sharedDepth=1",
+    "2fcrelu": "naive;intraTileScheduleFusionStrategy=Max;fixParametersBeforeScheduling=1;tile=1,64;unroll=256;"
+               "mapToThreads=250,4;mapToBlocks=512,256;useSharedMemory=1;usePrivateMemory=1;unrollCopyShared=1;"
+               "sharedDepth=1",
     "lut": "naive;outerScheduleFusionStrategy=Min;tile=4,32,32;unroll=64;usePrivateMemory=1;unrollCopyShared=1;"
            "collapseContiguous=0",
-    "moments2": "naive;outerScheduleFusionStrategy=Max;fixParametersBeforeScheduling=1;tile=1;unroll=64;tileImperfectlyNested=1;"
-                "matchLibraryCalls=1;mapToThreads=1024;mapToBlocks=1152;usePrivateMemory=1;unrollCopyShared=1;"
-                "useReadOnlyCache=1;vectorWidth=2;collapseContiguous=0;useMfma=1",
+    "moments2": "naive;outerScheduleFusionStrategy=Max;fixParametersBeforeScheduling=1;tile=1;unroll=128;"
+                "tileImperfectlyNested=1;matchLibraryCalls=1;mapToThreads=256;mapToBlocks=1152;usePrivateMemory=1;"
+                "unrollCopyShared=1;vectorWidth=2;collapseContiguous=0;useMfma=1",
     # 576 threads x float4 = one 48x48 plane per pass: the normalising stage then finds every
     # element in the register cache the two reductions filled (one read of the input)
-    "group_normalization_single_kernel": "naive;outerScheduleFusionStrategy=Max;tile=1,1;unroll=64;matchLibraryCalls=1;"
-                                         "mapToThreads=576;mapToBlocks=32,32;usePrivateMemory=1;vectorWidth=4",
-    "kronecker3": "naive;outerScheduleFusionStrategy=Max;intraTileScheduleFusionStrategy=Max;tile=1,16,256;unroll=8;"
-                  "tileImperfectlyNested=1;mapToThreads=32,32;mapToBlocks=256,32;useSharedMemory=1;useReadOnlyCache=1;"
-                  "privateDepth=5;collapseContiguous=0;useMfma=1;prefetchShared=1",
+    "group_normalization_single_kernel": "naive;outerScheduleFusionStrategy=Max;tile=1,1;unroll=64;matchLibraryCalls=1;mapToThreads=576;"
+                                         "mapToBlocks=256,256;usePrivateMemory=1;useReadOnlyCache=1;vectorWidth=4",
+    "kronecker3": "naive;outerScheduleFusionStrategy=Max;intraTileScheduleFusionStrategy=Max;tile=1,32,16;unroll=8;"
+                  "tileImperfectlyNested=1;mapToThreads=32,32;mapToBlocks=256,32;useReadOnlyCache=1;privateDepth=5;"
+                  "collapseContiguous=0;useMfma=1;prefetchShared=1",
     "wavenet1": "naive;intraTileScheduleFusionStrategy=Max;fixParametersBeforeScheduling=1;tile=2,2000,16,1;mapToThreads=16,64;"
                 "mapToBlocks=2000,256;useSharedMemory=1;usePrivateMemory=1;privateDepth=8;sharedDepth=3;vectorWidth=4;"
                 "collapseContiguous=0;prefetchShared=1",
