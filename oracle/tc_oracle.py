@@ -762,6 +762,8 @@ class _CEmitter:
         if not args:
             return f"{name}[0]"
         flat = args[0] if t.mins[0] == 0 else f"({args[0]} - {t.mins[0]})"
+        if int(np.prod([int(e) for e in t.extents], dtype=np.int64)) >= 2 ** 31:
+            flat = f"(int64_t)({flat})"                 # element offsets beyond 32 bits
         for d in range(1, len(args)):
             flat = f"({flat})*{t.extents[d]} + ({args[d]})"
         return f"{name}[{flat}]"

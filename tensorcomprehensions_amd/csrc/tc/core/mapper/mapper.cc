@@ -709,10 +709,18 @@ MappedProgram mapToHip(
     prog.paramNames.push_back(p.first);
     prog.paramValues.push_back(p.second);
   }
+  // Loop variables and size parameters are 32-bit: every single extent must fit; a tensor as a
+  // whole may hold 2^31 elements or more, element offsets are then formed in 64 bits.
   int64_t maxNumel = 0;
-  for (const auto& t : f.inputs) maxNumel = std::max(maxNumel, t.numel());
-  for (const auto& t : f.outputs) maxNumel = std::max(maxNumel, t.numel());
-  TC_CHECK_LT(maxNumel, (1LL << 31)) << "tensors with 2^31 or more elements are not supported yet";
+  for (const auto* ts : {&f.inputs, &f.outputs}) {
+    for (const auto& t : *ts) {
+      maxNumel = std::max(maxNumel, t.numel());
+      for (auto e : t.extents) {
+        TC_CHECK_LT(e, (1LL << 31)) << "tensor " << t.name << " has a dimension of 2^31 or more elements; not supported";
+      }
+    }
+  }
+  const bool wide = maxNumel >= (1LL << 31);
 
   bool anyThreadReduction = false;
   std::vector<std::unique_ptr<Emitter>> bodies;
@@ -780,6 +788,8 @@ MappedProgram mapToHip(
   std::ostringstream src;
   for (auto& k : prog.kernels) {
     KernelCtx kc{f, options, k};
+    kc.wide = wide;
+    if (wide) kc.idx = "int64";
     mapKernel(kc, limits);
     for (const auto& st : k.stages) anyThreadReduction |= st.threadReduction;
     bodies.emplace_back(new Emitter());

@@ -217,6 +217,7 @@ struct StageBuilder {
   bool tryCollapse(size_t k) {
     LoopVar &a = st.vars[k], &b = st.vars[k + 1];
     if (a.min != 0 || b.min != 0 || a.reduction != b.reduction) return false;
+    if (a.extent * b.extent >= (int64_t(1) << 31)) return false; // loop variables are 32-bit
     StageStmt* owner = nullptr;
     if (a.reduction) {
       for (auto& s : st.stmts) {

@@ -36,7 +36,10 @@ struct KernelCtx {
   const ir::Function& f;
   const HipMappingOptions& opts;
   KernelPlan& k;
-  std::string idx = "int"; // index arithmetic type
+  std::string idx = "int"; // type of non-affine subscript values inside an element offset
+  // Some tensor has 2^31 or more elements: element offsets into global memory are formed in 64
+  // bits (loop variables stay int: every extent is below 2^31).
+  bool wide = false;
   bool kernelLoops = false; // the stages sit inside loops over tiles that the blocks share out
   int64_t NT() const { return k.block[0] * k.block[1] * k.block[2]; }
 };
@@ -66,8 +69,8 @@ class StageCodegen {
     return st_.vars[0];
   }
 
-  // affine over i_<var> values -> C
-  std::string affineStr(const Affine& a) const {
+  // affine over i_<var> values -> C; `wide`: every term is formed in 64 bits
+  std::string affineStr(const Affine& a, bool wide = false) const {
     std::ostringstream ss;
     bool first = true;
     for (const auto& c : a.coef) {
@@ -76,7 +79,11 @@ class StageCodegen {
       if (!first) ss << (k < 0 ? " - " : " + ");
       else if (k < 0) ss << "-";
       int64_t m = k < 0 ? -k : k;
-      if (m != 1) ss << m << " * ";
+      if (wide) {
+        ss << "(int64)" << m << " * ";
+      } else if (m != 1) {
+        ss << m << " * ";
+      }
       ss << "i_" << c.first;
       first = false;
     }
@@ -129,7 +136,7 @@ class StageCodegen {
         extra += " + " + std::to_string(strides[j]) + " * (" + kc_.idx + ")(" + expr(subs[j], accRef) + ")";
       }
     }
-    return affineStr(total) + extra;
+    return affineStr(total, kc_.wide) + extra;
   }
 
   // Larger than what the L2 of one XCD keeps between uses.
@@ -671,7 +678,8 @@ class StageCodegen {
         if (!dims[j].inside) {
           cond += (cond.empty() ? "" : " && ") + std::string("(unsigned)") + g + " < " + std::to_string(dims[j].tensorExtent) + "u";
         }
-        gidx += (j ? " + " : "") + g + (dims[j].gStride != 1 ? " * " + std::to_string(dims[j].gStride) : "");
+        gidx += (j ? " + " : "") + std::string(kc_.wide ? "(int64)" : "") + g +
+            (dims[j].gStride != 1 ? " * " + std::to_string(dims[j].gStride) : "");
       }
       lidx += (j ? " + " : "") + l + (dims[j].lStride != 1 ? " * " + std::to_string(dims[j].lStride) : "");
     }

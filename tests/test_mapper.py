@@ -323,3 +323,17 @@ def test_a_stage_without_a_reduction_stages_overlapping_windows():
     # no reuse, no staging
     src2, _ = mapped(ADD, "fun", [(100, 200), (100, 200)], options)
     assert "__shared__" not in src2
+
+
+def test_offsets_are_64_bit_once_a_tensor_reaches_2_to_the_31_elements():
+    """Element offsets are formed in 64 bits when some tensor has 2^31 elements or more; every
+    single extent still has to stay below 2^31 (loop variables are int)."""
+    big = "def big(int8(M, N) X) -> (s, Y) { s(m) +=! int32(X(m, n))\n Y(m, n) = int8(X(m, n) + 1) }"
+    opts = "naive;tile=4,1024;mapToThreads=256;mapToBlocks=256,32;unroll=4"
+    src, _ = tc.map_only(big, "big", [ShapeOnly((65544, 32768), "int8")], opts)
+    assert "(int64)32768 * " in src
+    small, _ = tc.map_only(big, "big", [ShapeOnly((655, 32768), "int8")], opts)
+    assert "(int64)" not in small
+    with pytest.raises(tc.TcError) as e:
+        tc.map_only("def f(int8(N) A) -> (B) { B(i) = A(i) }", "f", [ShapeOnly((2 ** 31 + 8,), "int8")], "naive")
+    assert "dimension of 2^31 or more" in str(e.value)
