@@ -761,11 +761,14 @@ class _CEmitter:
         t = self.an.tensors[name]
         if not args:
             return f"{name}[0]"
-        flat = args[0] if t.mins[0] == 0 else f"({args[0]} - {t.mins[0]})"
+        # storage starts at the inferred lower bound: element k of a dimension holds point min + k
+        # (a Halide buffer whose min is set, tc2halide.cc:903, is addressed this way by the CPU JIT)
+        rel = [a if t.mins[d] == 0 else f"({a} - {t.mins[d]})" for d, a in enumerate(args)]
+        flat = rel[0]
         if int(np.prod([int(e) for e in t.extents], dtype=np.int64)) >= 2 ** 31:
             flat = f"(int64_t)({flat})"                 # element offsets beyond 32 bits
         for d in range(1, len(args)):
-            flat = f"({flat})*{t.extents[d]} + ({args[d]})"
+            flat = f"({flat})*{t.extents[d]} + ({rel[d]})"
         return f"{name}[{flat}]"
 
     def pretty_index(self, name, args):
@@ -911,9 +914,6 @@ def emit_c(an: Analysis, fname: str = "tc_oracle_kernel") -> str:
         sig.append(f"{_CTYPE[an.tensors[o].scalar]}* __restrict__ {o}")
     body: List[str] = []
     for s in an.d.stmts:
-        t = an.tensors[s.lhs]
-        if any(m != 0 for m in t.mins):
-            raise TcError(f"oracle cannot execute {s.lhs}: inferred minimum {t.mins} is not zero")
         body += ["  " + l for l in em.stmt_nests(s)]
     return _PRELUDE + f"void {fname}(" + ", ".join(sig) + ") {\n" + "\n".join(body) + "\n}\n"
 
@@ -992,7 +992,7 @@ def run_python(tc: str, entry: str, inputs: Sequence[np.ndarray], acc_dtype=None
         if k == "ident":
             return idx[e.op]
         if k == "access":
-            v = env[e.op][tuple(int(ev(a, idx)) for a in e.args)]
+            v = env[e.op][tuple(int(ev(a, idx)) - m for a, m in zip(e.args, an.tensors[e.op].mins))]
             return acc_dtype(v) if acc_dtype and e.type in ("float", "double") else v
         if k == "bin":
             a, b = ev(e.args[0], idx), ev(e.args[1], idx)
@@ -1027,13 +1027,15 @@ def run_python(tc: str, entry: str, inputs: Sequence[np.ndarray], acc_dtype=None
         out = env[s.lhs]
         base = s.assign.rstrip("!")
         lhs_ranges = [range(s.ranges[v][0], s.ranges[v][1] + 1) for v in s.indices]
+        lo = tuple(an.tensors[s.lhs].mins)               # storage starts at the inferred lower bound
         red_ranges = [range(s.ranges[v][0], s.ranges[v][1] + 1) for v in s.reduction_vars]
         if s.assign.endswith("!"):
             ident = {"+=": 0, "*=": 1, "min=": np.inf, "max=": -np.inf}[base]
-            for p in itertools.product(*lhs_ranges):
-                out[p] = ident
-        for p in itertools.product(*lhs_ranges):
-            idx = dict(zip(s.indices, p))
+            for q in itertools.product(*lhs_ranges):
+                out[tuple(a - b for a, b in zip(q, lo))] = ident
+        for q in itertools.product(*lhs_ranges):
+            idx = dict(zip(s.indices, q))
+            p = tuple(a - b for a, b in zip(q, lo))
             for r in itertools.product(*red_ranges):
                 idx.update(zip(s.reduction_vars, r))
                 v = ev(s.rhs, idx)

@@ -642,16 +642,72 @@ void emitKernel(KernelCtx& kc, const DeviceLimits& limits, Emitter& em) {
 
 } // namespace
 
+namespace {
+// e + c with the constant folded into an existing "+ constant"
+ExprRef addConstant(const ExprRef& e, int64_t c) {
+  if (e->kind == Expr::IntImm) return mkInt(e->ival + c);
+  if (e->kind == Expr::Binary && e->name == "+" && e->args[1]->kind == Expr::IntImm) {
+    return addConstant(e->args[0], e->args[1]->ival + c);
+  }
+  return c == 0 ? e : mkBin("+", e, mkInt(c));
+}
+
+// The storage of an output starts at its inferred lower bound: element k of dimension d holds
+// the point mins[d] + k, the way a Halide buffer with a non-zero min is addressed (the bounds
+// are set in tc/core/tc2halide.cc:903).  Rewrites the function to zero-based outputs: an index
+// variable that subscripts a shifted dimension on the left-hand side is shifted by the bound
+// (range and every use), and every other subscript of such a tensor has the bound subtracted.
+ir::Function withZeroBasedOutputs(const ir::Function& in) {
+  ir::Function f = in;
+  std::map<std::string, std::vector<int64_t>> mins;
+  for (auto& t : f.outputs) {
+    mins[t.name] = t.mins;
+    std::fill(t.mins.begin(), t.mins.end(), 0);
+  }
+  for (auto& s : f.statements) {
+    std::map<std::string, int64_t> shift;
+    const auto& m = mins.at(s.tensor);
+    for (size_t d = 0; d < s.lhsVars.size(); ++d) {
+      auto it = shift.find(s.lhsVars[d]);
+      TC_CHECK(it == shift.end() || it->second == m[d])
+          << "index " << s.lhsVars[d] << " subscripts two dimensions of " << s.tensor << " with different lower bounds";
+      shift[s.lhsVars[d]] = m[d];
+    }
+    for (const auto& sh : shift) {
+      ir::Range& r = s.ranges.at(sh.first);
+      r.min -= sh.second;
+      r.max -= sh.second;
+    }
+    s.rhs = rewrite(s.rhs, [&](const ExprRef& e) -> ExprRef {
+      if (e->kind == Expr::Var) {
+        auto it = shift.find(e->name);
+        return it == shift.end() || it->second == 0 ? nullptr : mkBin("+", e, mkInt(it->second));
+      }
+      if (e->kind == Expr::Load) {
+        auto it = mins.find(e->name);
+        if (it == mins.end()) return nullptr;
+        auto c = std::make_shared<Expr>(*e);
+        for (size_t d = 0; d < c->args.size(); ++d) c->args[d] = addConstant(c->args[d], -it->second[d]);
+        return c;
+      }
+      return nullptr;
+    });
+  }
+  return f;
+}
+} // namespace
+
 MappedProgram mapToHip(
-    const ir::Function& f,
+    const ir::Function& given,
     const HipMappingOptions& options,
     const std::string& specializedName,
     const DeviceLimits& limits) {
-  for (const auto& t : f.outputs) {
-    for (auto m : t.mins) {
-      TC_CHECK_EQ(m, 0) << "output " << t.name << " has a non-zero inferred lower bound; not supported";
-    }
+  bool shifted = false;
+  for (const auto& t : given.outputs) {
+    for (auto m : t.mins) shifted |= m != 0;
   }
+  const ir::Function zeroBased = shifted ? withZeroBasedOutputs(given) : ir::Function();
+  const ir::Function& f = shifted ? zeroBased : given;
   // 1. stages
   std::vector<RawStage> raw;
   bool allowStageFusion = options.generic.intraTileScheduleOptions.fusionStrategy != FusionStrategy::Min ||

@@ -337,3 +337,11 @@ def test_offsets_are_64_bit_once_a_tensor_reaches_2_to_the_31_elements():
     with pytest.raises(tc.TcError) as e:
         tc.map_only("def f(int8(N) A) -> (B) { B(i) = A(i) }", "f", [ShapeOnly((2 ** 31 + 8,), "int8")], "naive")
     assert "dimension of 2^31 or more" in str(e.value)
+
+
+def test_outputs_with_a_lower_bound_are_stored_from_it():
+    """Element k of a shifted dimension holds the point min + k: the write and every later read of
+    the tensor subtract the bound (inferred by test/test_inference.cc:158-186)."""
+    src, _ = mapped("def fun(float(I_0) I) -> (O, P) { O(i) = I(i - 1)\n P(j) = O(j + 1) }", "fun", [(100,)], "naive")
+    assert "pO[i_i] = " in src and "acc_[a_] = pI[i_i];" in src     # i shifted to 0..99, I(i - 1) with it
+    assert "acc_[a_] = pO[i_i];" in src and "pP[i_i] = " in src     # P(j) reads point j + 1 = element j

@@ -192,3 +192,22 @@ def test_python_interpreter_agrees_with_compiled_nest():
     b = tc_oracle.run_python(W.MOMENTS, "moments", [X])
     for x, y in zip(a, b):
         assert np.allclose(x, y, atol=1e-6)
+
+
+def test_storage_of_an_output_starts_at_its_inferred_lower_bound():
+    """Shifts of test/test_inference.cc:158-186 executed: the point min + k is element k, so a
+    shifted copy returns the input itself, and a reader of the shifted tensor sees its points."""
+    I = rng(14).standard_normal(7, dtype=np.float32)
+    for stmt in ("O(i) = I(i - 1)", "O(i) = I(i + 5)"):
+        src = "def fun(float(I_0) I) -> (O) { %s }" % stmt
+        for runner in (tc_oracle.run, tc_oracle.run_python):
+            (O,) = runner(src, "fun", [I])
+            assert np.array_equal(O, I)
+    src = """def f(float(N, M) A) -> (O, P) {
+        O(i, j) = A(i, j) * 2.0 where i in 3:N, j in 1:5
+        P(i) +=! O(i, j) + A(i - 3, j) }"""
+    A = rng(15).integers(-9, 10, size=(12, 7)).astype(np.float32)
+    for runner in (tc_oracle.run, tc_oracle.run_python):
+        O, P = runner(src, "f", [A])
+        assert np.array_equal(O, 2 * A[3:, 1:5])
+        assert np.array_equal(P, (2 * A[3:, 1:5] + A[:9, 1:5]).sum(1))
