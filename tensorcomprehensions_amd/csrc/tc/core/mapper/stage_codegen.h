@@ -342,16 +342,24 @@ class StageCodegen {
     return MT <= 16 && BT == 1 && ceilDiv(KT, 4) <= kMaxResidentSteps;
   }
 
+  bool fullRegisterTile() const {
+    for (const auto& v : st_.vars) {
+      if (!st_.mfma && !v.reduction && !v.unrolled && v.perThread > 1) return false;
+    }
+    return true;
+  }
+
   void planPromotions(const StageStmt& s, int64_t& ldsBudgetBytes) {
     if (!kc_.opts.useSharedMemoryValue) return;
     if (s.redVars.empty() && st_.mfma) return;
-    for (const auto& v : st_.vars) {
-      if (!st_.mfma && !v.reduction && !v.unrolled && v.perThread > 1) return; // needs a full register tile
-    }
     bool reductionTiled = false;
     for (const auto& r : s.redVars) reductionTiled |= var(r).numTiles > 1;
     bool inside = reductionTiled &&
         (!kc_.opts.hasSharedDepth || kc_.opts.sharedDepthValue > static_cast<uint32_t>(st_.numParallel));
+    // Per-thread loops that stay loops enclose the whole statement, the reduction tile loop
+    // included: a copy per reduction tile would be repeated by every one of their iterations.
+    // Footprints of the whole block tile are staged once, in front of those loops.
+    if (inside && !fullRegisterTile()) return;
     // iterations of the statement inside the promoted region
     std::set<std::string> stmtVars;
     for (int i = 0; i < st_.numParallel; ++i) stmtVars.insert(st_.vars[i].name);
@@ -837,7 +845,11 @@ class StageCodegen {
     const bool staged = &s == promotedPointwise_;
     if (staged) {
       em_.open("");
-      stageOutsideFootprints();
+      if (stagedAheadOfPointLoops_) {
+        for (const auto& p : st_.promotions) activePromotions_.insert(p.tensor);
+      } else {
+        stageOutsideFootprints();
+      }
     }
     emitPointwiseBody(s);
     if (staged) {
@@ -913,6 +925,10 @@ class StageCodegen {
     bool anyOutside = false, anyInside = false;
     for (const auto& p : st_.promotions) (p.insideReductionTiles ? anyInside : anyOutside) = true;
     auto copyIn = [&](bool inside) {
+      if (stagedAheadOfPointLoops_ && !inside) {
+        for (const auto& p : st_.promotions) activePromotions_.insert(p.tensor);
+        return;
+      }
       if (suppressCopy && !inside) {
         for (const auto& p : st_.promotions) {
           if (!p.insideReductionTiles) {
@@ -1723,6 +1739,18 @@ class StageCodegen {
         ++opened;
       }
     }
+    // footprints of the block tile are staged ahead of per-thread loops that stay loops
+    stageTileLoops_ = opened > 1;
+    stagedAheadOfPointLoops_ = false;
+    if (!st_.promotions.empty() && !fullRegisterTile()) {
+      if (suppressCopy) {
+        for (const auto& p : st_.promotions) declareLows(p);
+      } else {
+        stageFootprints(false);
+        for (const auto& p : st_.promotions) activePromotions_.erase(p.tensor);
+      }
+      stagedAheadOfPointLoops_ = true;
+    }
     // per-thread point loops that stay loops
     outerPred_ = idleAxesPredForCompute();
     for (int i = 0; i < st_.numParallel; ++i) {
@@ -1783,6 +1811,7 @@ class StageCodegen {
   bool inCachedReduction_ = false;
   bool stageTileLoops_ = false; // the stage's code sits inside tile loops of its own
   bool copiedBefore_ = false;   // this stage has already written LDS once
+  bool stagedAheadOfPointLoops_ = false; // the footprints were staged before the per-thread loops opened
   const StageStmt* promotedPointwise_ = nullptr; // statement of a reduction-free stage that reads staged footprints
   std::string cacheSlot_;
   int clampId_ = 0;

@@ -46,6 +46,8 @@ def test_two_convolutions_over_one_staged_input(options):
     "naive;tile=8,64;mapToThreads=64,2;mapToBlocks=3,2;unroll=4;useSharedMemory=1",          # blocks loop over tiles
     "naive;tile=16,32;mapToThreads=32,4;mapToBlocks=16,16;unroll=8;useSharedMemory=1;vectorWidth=2",
     "naive;tile=5,7;mapToThreads=7,5;mapToBlocks=32,32;unroll=1;useSharedMemory=1",
+    "naive;tile=16,32;mapToThreads=32,4;mapToBlocks=16,16;unroll=1;useSharedMemory=1",        # per-thread loop stays a loop
+    "naive;tile=16,64;mapToThreads=16,2;mapToBlocks=2,2;unroll=2;useSharedMemory=1",          # and under block-level tile loops
 ])
 def test_stencil_through_lds(options):
     A = np.random.Generator(np.random.Philox(42)).standard_normal((100, 200), dtype=np.float32)
@@ -70,3 +72,20 @@ def test_staging_copies_whose_loops_overshoot_the_footprint(threads, shapes):
     (ref,) = tc_oracle.run(W.BATCH_MATMUL, "batch_matmul", ins)
     assert ex.lds_bytes() > 0
     assert np.array_equal(got[0], ref) and np.array_equal(ref, np.matmul(ins[0], ins[1]))
+
+
+@pytest.mark.parametrize("options", [
+    "naive;tile=32,32;mapToThreads=16,16;mapToBlocks=8,8;unroll=1;useSharedMemory=1",
+    "naive;tile=32,32,0;mapToThreads=16,8;mapToBlocks=2,2;unroll=2;useSharedMemory=1",
+    "naive;tile=8,64;mapToThreads=32,2;mapToBlocks=16,4;unroll=4;useSharedMemory=1;usePrivateMemory=1",
+])
+def test_matmul_staged_ahead_of_per_thread_loops(options):
+    """A register tile that is not fully unrolled: the block tile's operands are staged once, in
+    front of the per-thread loops."""
+    rng = np.random.Generator(np.random.Philox(44))
+    A = rng.integers(-3, 4, size=(100, 72)).astype(np.float32)
+    B = rng.integers(-3, 4, size=(72, 130)).astype(np.float32)
+    src = "def mm(float(M, K) A, float(K, N) B) -> (C) { C(m, n) +=! A(m, k) * B(k, n) }"
+    (got,), ex = run(src, "mm", [A, B], options)
+    assert "lds0_A" in ex.compiled_source or "lds0_B" in ex.compiled_source, options
+    assert np.array_equal(got, A @ B)
