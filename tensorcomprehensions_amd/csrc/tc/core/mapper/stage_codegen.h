@@ -426,7 +426,11 @@ class StageCodegen {
         elems *= ext;
       }
       c.p.reuse = static_cast<int64_t>(iterations * acc.second.size() / static_cast<double>(elems));
-      if (c.p.reuse < 2) continue;
+      // Worth a copy when elements are used more than once, or when the threads of a wavefront
+      // walk a slower dimension of the tensor while the cooperative copy reads whole rows
+      // (promotionImprovesCoalescing, tc/core/polyhedral/cuda/memory_promotion_heuristic.cc:211-244).
+      const bool coalesces = lanesWalkOuterDim(ref) && c.p.extents.back() >= 8;
+      if (c.p.reuse < 2 && !coalesces) continue;
       // Pitches.  pad[j] = elements added to the distance between consecutive indices of dimension j.
       const size_t nd = ref.size();
       std::vector<int64_t> pad(nd, 0);

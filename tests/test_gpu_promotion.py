@@ -89,3 +89,20 @@ def test_matmul_staged_ahead_of_per_thread_loops(options):
     (got,), ex = run(src, "mm", [A, B], options)
     assert "lds0_A" in ex.compiled_source or "lds0_B" in ex.compiled_source, options
     assert np.array_equal(got, A @ B)
+
+
+@pytest.mark.parametrize("options", [
+    "naive;tile=32,32;mapToThreads=32,8;mapToBlocks=128,128;unroll=4;useSharedMemory=1",
+    "naive;tile=64,64;mapToThreads=64,4;mapToBlocks=3,5;unroll=16;useSharedMemory=1",
+    "naive;tile=16,24;mapToThreads=24,4;mapToBlocks=64,64;unroll=1;useSharedMemory=1",
+])
+def test_transposed_read_is_staged_for_coalescing(options):
+    """No element is used twice, but the threads of a wavefront walk the slow dimension of A: the
+    copy reads whole rows instead (the reference's promotionImprovesCoalescing rule)."""
+    src = "def tr(float(N, M) A) -> (O) { O(j, i) = A(i, j) }"
+    A = np.random.Generator(np.random.Philox(45)).standard_normal((300, 500), dtype=np.float32)
+    (got,), ex = run(src, "tr", [A], options)
+    assert "lds0_A" in ex.compiled_source
+    assert np.array_equal(got, A.T)
+    (ref,) = tc_oracle.run(src, "tr", [A])
+    assert np.array_equal(got, ref)

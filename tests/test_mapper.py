@@ -345,3 +345,13 @@ def test_outputs_with_a_lower_bound_are_stored_from_it():
     src, _ = mapped("def fun(float(I_0) I) -> (O, P) { O(i) = I(i - 1)\n P(j) = O(j + 1) }", "fun", [(100,)], "naive")
     assert "pO[i_i] = " in src and "acc_[a_] = pI[i_i];" in src     # i shifted to 0..99, I(i - 1) with it
     assert "acc_[a_] = pO[i_i];" in src and "pP[i_i] = " in src     # P(j) reads point j + 1 = element j
+
+
+def test_promotion_for_coalescing_alone():
+    """An operand without reuse is staged when the threads along x walk a slower dimension of it
+    (memory_promotion_heuristic.cc:211-244), and not when they walk its rows."""
+    o = "naive;tile=32,32;mapToThreads=32,8;mapToBlocks=128,128;unroll=4;useSharedMemory=1"
+    src, _ = mapped("def tr(float(N, M) A) -> (O) { O(j, i) = A(i, j) }", "tr", [(4096, 4096)], o)
+    assert "lds0_A[1056]" in src                        # 32 x 32 tile, pitch 33
+    src, _ = mapped("def cp(float(N, M) A) -> (O) { O(i, j) = A(i, j) }", "cp", [(4096, 4096)], o)
+    assert "lds0_A" not in src
