@@ -339,8 +339,41 @@ class StageCodegen {
     for (const auto& n : st_.mfmaK) {
       if (var(n).numTiles > 1) return false;
     }
-    return MT <= 16 && BT == 1 && ceilDiv(KT, 4) <= kMaxResidentSteps;
+    // (with the reduction split over wavefronts a wavefront has one tile: nothing to keep)
+    return MT <= 16 && BT == 1 && ceilDiv(KT, 4) <= kMaxResidentSteps && mfmaKSplit() == 1;
   }
+
+  // Output tiles of 16x16 per block and reduction steps per lane of a matrix-core stage.
+  void mfmaCounts(int64_t& tiles, int64_t& ksteps) const {
+    int64_t MT = 1, NT = 1, BT = 1, KT = 1;
+    for (const auto& n : st_.mfmaM) MT *= var(n).tile;
+    for (const auto& n : st_.mfmaN) NT *= var(n).tile;
+    for (const auto& n : st_.mfmaBatch) BT *= var(n).tile;
+    for (const auto& n : st_.mfmaK) KT *= var(n).tile;
+    tiles = BT * ceilDiv(MT, 16) * ceilDiv(NT, 16);
+    ksteps = ceilDiv(KT, 4);
+  }
+  // Reduction split over wavefronts.  A block with fewer output tiles than wavefronts would leave
+  // wavefronts idle while the busy ones walk the whole reduction: the steps of a tile are divided
+  // evenly among `split` wavefronts instead, whose partial tiles meet in LDS (one 16-byte write per
+  // lane, a barrier, the owner of the tile adds them up).  1: no split.
+  static constexpr int64_t kMinStepsPerSplit = 8;
+  int64_t mfmaKSplit() const {
+    if (!st_.mfma || !kSplitAllowed_) return 1;
+    int64_t tiles, ksteps;
+    mfmaCounts(tiles, ksteps);
+    if (tiles >= st_.waves) return 1;
+    int64_t split = std::min(st_.waves / tiles, ksteps / kMinStepsPerSplit);
+    if (split < 2) return 1;
+    // the fewest wavefronts that keep the steps of the busiest one at that minimum
+    return ceilDiv(ksteps, ceilDiv(ksteps, split));
+  }
+  int64_t mfmaKSplitBytes() const {
+    int64_t tiles, ksteps;
+    mfmaCounts(tiles, ksteps);
+    return (mfmaKSplit() - 1) * tiles * 64 * 16;
+  }
+  std::string kSplitName() const { return "ksplit" + std::to_string(stageIdx_) + "_"; }
 
   bool fullRegisterTile() const {
     for (const auto& v : st_.vars) {
@@ -521,6 +554,9 @@ class StageCodegen {
   }
 
   void emitLdsDecls() {
+    if (mfmaKSplit() > 1) {
+      em_.line("__shared__ __attribute__((aligned(16))) float " + kSplitName() + "[" + std::to_string(mfmaKSplitBytes() / 4) + "];");
+    }
     for (const auto& p : st_.promotions) {
       if (p.sharedWithEarlierStage) continue;
       em_.line("__shared__ __attribute__((aligned(16))) " + st_.views.at(p.tensor).type.cName() + " " + p.ldsName +
@@ -1241,6 +1277,13 @@ class StageCodegen {
   // say: several accesses per element through overlapping windows) plans them for its first
   // statement that loads anything.
   void plan(int64_t& ldsBudgetBytes) {
+    if (mfmaKSplit() > 1) {
+      if (mfmaKSplitBytes() > ldsBudgetBytes) {
+        kSplitAllowed_ = false;
+      } else {
+        ldsBudgetBytes -= mfmaKSplitBytes();
+      }
+    }
     for (const auto& s : st_.stmts) {
       if (!s.redVars.empty()) {
         planPromotions(s, ldsBudgetBytes);
@@ -1351,11 +1394,21 @@ class StageCodegen {
     int64_t innerProd = 1;
     for (size_t i = 1; i < st_.mfmaK.size(); ++i) innerProd *= var(st_.mfmaK[i]).tile;
     const bool aligned = quarter % innerProd == 0;
+    const int64_t split = mfmaKSplit();
+    const int64_t stepsPerWave = ceilDiv(ksteps, split);
+    const bool unevenSplit = stepsPerWave * split != ksteps; // the last slice has surplus steps
+    const std::string kx = split > 1 ? "kq_" : "ks_"; // counter of a wavefront's own steps
     // Opens the loop over the reduction steps of a lane, decodes the reduction indices of the
     // step and declares kok_ when surplus steps exist; returns whether it did.
-    auto openSteps = [&]() {
-      em_.line(ksteps <= 128 ? "#pragma unroll" : "#pragma unroll 4");
-      em_.open("for (int ks_ = 0; ks_ < " + std::to_string(ksteps) + "; ++ks_)");
+    auto openSteps = [&](int64_t count) {
+      em_.line(count <= 128 ? "#pragma unroll" : "#pragma unroll 4");
+      if (split > 1) {
+        // slice sl_ of the steps: ks_ is the step within the whole reduction
+        em_.open("for (int kq_ = 0; kq_ < " + std::to_string(count) + "; ++kq_)");
+        em_.line("const int ks_ = sl_ * " + std::to_string(stepsPerWave) + " + kq_;");
+      } else {
+        em_.open("for (int ks_ = 0; ks_ < " + std::to_string(ksteps) + "; ++ks_)");
+      }
       std::string kok;
       if (aligned) {
         int64_t div = innerProd;
@@ -1435,7 +1488,7 @@ class StageCodegen {
         em_.line("am_[ks_] = v_[0]; am_[ks_ + 1] = v_[1]; am_[ks_ + 2] = v_[2]; am_[ks_ + 3] = v_[3];");
         em_.close();
       } else {
-        bool masked = openSteps();
+        bool masked = openSteps(ksteps);
         em_.line("am_[ks_] = " + operandValue(loadA, masked) + ";");
         em_.close();
       }
@@ -1528,27 +1581,41 @@ class StageCodegen {
       em_.line("const int mposa_ = mt_ * 16 + lm_;");
       em_.line("const bool moka_ = bok_ && " + decodeGroup(st_.mfmaM, "mposa_", true) + ";");
       em_.line("(void)moka_;");
-      if (ksteps <= kMaxResidentSteps) {
-        // The operand values of all steps first, then the chain of multiplications: every read is
-        // in flight before the first result is needed, and the multiplications wait for nothing
-        // but their own operands (10.5 -> 10.0 us on the 16-channel 3x3 group convolution).
-        em_.line("float bq_[" + std::to_string(ksteps) + "];");
-        if (!resident) em_.line("float aq_[" + std::to_string(ksteps) + "];");
-        bool masked = openSteps();
-        if (!resident) em_.line("aq_[ks_] = " + operandValue(loadA, masked) + ";");
-        em_.line("bq_[ks_] = " + operandValue(loadB, masked) + ";");
+      // `count` steps of this wavefront
+      auto steps = [&](int64_t count) {
+        if (count <= kMaxResidentSteps) {
+          // The operand values of all steps first, then the chain of multiplications: every read is
+          // in flight before the first result is needed, and the multiplications wait for nothing
+          // but their own operands (10.5 -> 10.0 us on the 16-channel 3x3 group convolution).
+          em_.line("float bq_[" + std::to_string(count) + "];");
+          if (!resident) em_.line("float aq_[" + std::to_string(count) + "];");
+          bool masked = openSteps(count);
+          if (!resident) em_.line("aq_[" + kx + "] = " + operandValue(loadA, masked) + ";");
+          em_.line("bq_[" + kx + "] = " + operandValue(loadB, masked) + ";");
+          em_.close();
+          em_.line("#pragma unroll");
+          em_.open("for (int " + kx + " = 0; " + kx + " < " + std::to_string(count) + "; ++" + kx + ")");
+          em_.line(acc + " = __builtin_amdgcn_mfma_f32_16x16x4f32(" + (resident ? "am_" : "aq_") + "[" + kx + "], bq_[" + kx + "], " +
+                   acc + ", 0, 0, 0);");
+          em_.close();
+        } else {
+          bool masked = openSteps(count);
+          em_.line("const float a_ = " + (resident ? std::string("am_[ks_]") : operandValue(loadA, masked)) + ";");
+          em_.line("const float b_ = " + operandValue(loadB, masked) + ";");
+          em_.line(acc + " = __builtin_amdgcn_mfma_f32_16x16x4f32(a_, b_, " + acc + ", 0, 0, 0);");
+          em_.close();
+        }
+      };
+      if (unevenSplit) {
+        // the last slice is shorter: its own copy of the loop, chosen per wavefront
+        em_.open("if (sl_ < " + std::to_string(split - 1) + ")");
+        steps(stepsPerWave);
         em_.close();
-        em_.line("#pragma unroll");
-        em_.open("for (int ks_ = 0; ks_ < " + std::to_string(ksteps) + "; ++ks_)");
-        em_.line(acc + " = __builtin_amdgcn_mfma_f32_16x16x4f32(" + (resident ? "am_" : "aq_") + "[ks_], bq_[ks_], " + acc +
-                 ", 0, 0, 0);");
+        em_.open("else");
+        steps(ksteps - (split - 1) * stepsPerWave);
         em_.close();
       } else {
-        bool masked = openSteps();
-        em_.line("const float a_ = " + (resident ? std::string("am_[ks_]") : operandValue(loadA, masked)) + ";");
-        em_.line("const float b_ = " + operandValue(loadB, masked) + ";");
-        em_.line(acc + " = __builtin_amdgcn_mfma_f32_16x16x4f32(a_, b_, " + acc + ", 0, 0, 0);");
-        em_.close();
+        steps(stepsPerWave);
       }
       em_.close();
     };
@@ -1588,6 +1655,30 @@ class StageCodegen {
       em_.close();
       em_.close();
     };
+    // Which tile a wavefront works on, who multiplies and who finishes it.  Without a split
+    // wavefront wv_ takes tiles wv_, wv_ + waves, ...; with one, wavefront wv_ takes slice
+    // wv_ / tiles of the reduction of tile wv_ % tiles and slice 0 owns the tile.
+    const std::string T = std::to_string(tiles), W = std::to_string(st_.waves), S = std::to_string(split);
+    const std::string tileDecl = split > 1 ? "const int tl_ = wv_ % " + T + ", sl_ = wv_ / " + T + ";"
+                                           : "const int tl_ = wv_ + j_ * " + W + ";";
+    const std::string worksOnTile = split > 1 ? "sl_ < " + S : "tl_ < " + T;
+    const std::string ownsTile = split > 1 ? "sl_ == 0" : "tl_ < " + T;
+    const std::string partialAt = kSplitName() + "[((%s * " + T + " + tl_) * 64 + threadIdx.x) * 4]";
+    auto partial = [&](const std::string& slice) {
+      std::string t = partialAt;
+      return t.replace(t.find("%s"), 2, slice);
+    };
+    // every wavefront of the block passes here: the partial tiles of slices 1.. go to LDS
+    auto exchange = [&](const std::string& acc) {
+      em_.line("if (sl_ > 0 && sl_ < " + S + ") *(__tc::floatx4*)&" + partial("(sl_ - 1)") + " = " + acc + ";");
+      em_.line("__syncthreads();");
+    };
+    auto gather = [&](const std::string& acc) {
+      em_.line("#pragma unroll");
+      em_.open("for (int o_ = 0; o_ < " + std::to_string(split - 1) + "; ++o_)");
+      em_.line(acc + " += *(const __tc::floatx4*)&" + partial("o_") + ";");
+      em_.close();
+    };
     // which wavefront takes the surplus tile rotates with the block, so that the blocks sharing a
     // compute unit load its four SIMDs evenly
     const std::string waveRotation =
@@ -1597,7 +1688,26 @@ class StageCodegen {
     ++opened;
     stagePromotions(false);
     if (resident && residentFromLds) fillResident();
-    if (!kTiled) {
+    if (!kTiled && split > 1) {
+      em_.line(waveRotation);
+      em_.line(tileDecl);
+      em_.line("__tc::floatx4 c_ = {0.0f, 0.0f, 0.0f, 0.0f};");
+      em_.open("if (" + worksOnTile + ")");
+      decodeTile();
+      if (!s.init) {
+        em_.open("if (" + ownsTile + ")");
+        loadExisting("c_");
+        em_.close();
+      }
+      multiply("c_");
+      em_.close();
+      exchange("c_");
+      em_.open("if (" + ownsTile + ")");
+      ++opened;
+      decodeTile();
+      gather("c_");
+      finish("c_");
+    } else if (!kTiled) {
       em_.line(waveRotation);
       if (tilesPerWave <= 8) {
         // few tiles per wavefront: unrolled, so that the operand reads of a tile can be scheduled
@@ -1624,8 +1734,8 @@ class StageCodegen {
       em_.open("for (int j_ = 0; j_ < " + std::to_string(tilesPerWave) + "; ++j_)");
       em_.line("cacc_[j_] = __tc::floatx4{0.0f, 0.0f, 0.0f, 0.0f};");
       if (!s.init) {
-        em_.line("const int tl_ = wv_ + j_ * " + std::to_string(st_.waves) + ";");
-        em_.open("if (tl_ < " + std::to_string(tiles) + ")");
+        em_.line(tileDecl);
+        em_.open("if (" + ownsTile + ")");
         decodeTile();
         loadExisting("cacc_[j_]");
         em_.close();
@@ -1686,8 +1796,8 @@ class StageCodegen {
       }
       em_.line("#pragma unroll");
       em_.open("for (int j_ = 0; j_ < " + std::to_string(tilesPerWave) + "; ++j_)");
-      em_.line("const int tl_ = wv_ + j_ * " + std::to_string(st_.waves) + ";");
-      em_.open("if (tl_ < " + std::to_string(tiles) + ")");
+      em_.line(tileDecl);
+      em_.open("if (" + worksOnTile + ")");
       decodeTile();
       multiply("cacc_[j_]");
       em_.close();
@@ -1701,16 +1811,25 @@ class StageCodegen {
         em_.close();
       }
       em_.close();
+      if (split > 1) {
+        em_.open("");
+        em_.line(tileDecl);
+        exchange("cacc_[0]");
+        em_.close();
+      }
       em_.line("#pragma unroll");
       em_.open("for (int j_ = 0; j_ < " + std::to_string(tilesPerWave) + "; ++j_)");
       ++opened;
-      em_.line("const int tl_ = wv_ + j_ * " + std::to_string(st_.waves) + ";");
-      em_.open("if (tl_ < " + std::to_string(tiles) + ")");
+      em_.line(tileDecl);
+      em_.open("if (" + ownsTile + ")");
       ++opened;
       decodeTile();
+      if (split > 1) gather("cacc_[j_]");
       finish("cacc_[j_]");
     }
     closeN(opened);
+    // inside loops the partial tiles are written again: not before every owner has read them
+    if (split > 1 && (kc_.kernelLoops || stageTileLoops_)) em_.line("__syncthreads();");
     hoistedLoads_.clear();
     for (const auto& p : st_.promotions) activePromotions_.erase(p.tensor);
   }
@@ -1814,6 +1933,7 @@ class StageCodegen {
   std::map<std::string, std::string> hoistedLoads_; // printed global load -> register holding it
   bool inCachedReduction_ = false;
   bool stageTileLoops_ = false; // the stage's code sits inside tile loops of its own
+  bool kSplitAllowed_ = true;   // LDS has room for the partial tiles of a split reduction
   bool copiedBefore_ = false;   // this stage has already written LDS once
   bool stagedAheadOfPointLoops_ = false; // the footprints were staged before the per-thread loops opened
   const StageStmt* promotedPointwise_ = nullptr; // statement of a reduction-free stage that reads staged footprints

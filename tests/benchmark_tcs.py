@@ -194,17 +194,18 @@ TUNED_AT_REFERENCE_SIZES = {
     # 54 threads along w; hand-set: the search's thread counts do not contain 54 x 9
     "group_convolution": "naive;tile=1,1,4,27,0;mapToThreads=54,9;mapToBlocks=32,32,8;useSharedMemory=1;unroll=16;"
                          "useReadOnlyCache=1",
-    "tmm": "naive;tile=1,32,0;unroll=128;matchLibraryCalls=1;mapToThreads=64,4,4;mapToBlocks=256,256;"
-           "useSharedMemory=1;unrollCopyShared=1;useReadOnlyCache=1;sharedDepth=2;vectorWidth=2;useMfma=1;"
-           "prefetchShared=1",
-    "matmul": "naive;intraTileScheduleFusionStrategy=Max;tile=16,32;unroll=256;matchLibraryCalls=1;mapToThreads=512,2;"
-              "mapToBlocks=125,1000;unrollCopyShared=1;useReadOnlyCache=1;useMfma=1;prefetchShared=1",
+    "tmm": "naive;tile=8,8;unroll=128;matchLibraryCalls=1;mapToThreads=256;mapToBlocks=256,32;useSharedMemory=1;"
+           "useReadOnlyCache=1;sharedDepth=7;collapseContiguous=0;useMfma=1;"
+           "outerScheduleFusionStrategy=Preserve3Coincident;intraTileScheduleFusionStrategy=Min",
+    # two 16x16 tiles per block of 8 wavefronts, 250 reduction steps of a tile split over 4 of them
+    "matmul": "naive;tile=16,32;unroll=256;matchLibraryCalls=1;mapToThreads=256,2;mapToBlocks=125,1000;useSharedMemory=1;"
+              "useReadOnlyCache=1;vectorWidth=2;useMfma=1",
     "convolution": "naive;intraTileScheduleFusionStrategy=Min;fixParametersBeforeScheduling=1;tile=1,27,1,0;unroll=128;"
                    "tileImperfectlyNested=1;mapToThreads=256,1;mapToBlocks=256,64,1;useSharedMemory=1;useReadOnlyCache=1;"
                    "collapseContiguous=0",
-    "2fcrelu": "naive;intraTileScheduleFusionStrategy=Max;fixParametersBeforeScheduling=1;tile=1,64;unroll=256;"
-               "mapToThreads=250,4;mapToBlocks=512,256;useSharedMemory=1;usePrivateMemory=1;unrollCopyShared=1;"
-               "sharedDepth=1",
+    # one 16x16 tile per block, the 500 reduction steps of the first layer split over 16 wavefronts
+    "2fcrelu": "naive;tile=16,16,128;unroll=256;mapToThreads=512,2;mapToBlocks=512,256;useMfma=1;useReadOnlyCache=1;"
+               "useSharedMemory=1",
     "lut": "naive;outerScheduleFusionStrategy=Min;tile=4,32,32;unroll=64;usePrivateMemory=1;unrollCopyShared=1;"
            "collapseContiguous=0",
     "moments2": "naive;outerScheduleFusionStrategy=Max;fixParametersBeforeScheduling=1;tile=1;unroll=128;"

@@ -167,3 +167,46 @@ def test_reduction_tiling_stages_operands_per_tile(opts):
     tc.run(ex, ins, [C])
     torch.cuda.synchronize()
     assert np.array_equal(C.cpu().numpy(), C0 + A @ B)
+
+
+FC = """def fc(float(B, K) I, float(N, K) W1, float(N) B1) -> (O1) {
+    O1(b, n) +=! I(b, k) * W1(n, k)
+    O1(b, n) = O1(b, n) + B1(n)
+    O1(b, n) = fmax(O1(b, n), 0) }"""
+
+
+@pytest.mark.parametrize("k,opts,split", [
+    # one tile, 16 wavefronts, 128 steps: 16 slices of 8
+    (512, "naive;tile=16,16;mapToThreads=512,2;mapToBlocks=64,64;useMfma=1", 16),
+    # 250 steps over 8 wavefronts per tile: 7 slices of 32 and one of 26
+    (1000, "naive;tile=16,32;mapToThreads=512,2;mapToBlocks=64,64;useMfma=1", 8),
+    # operands staged in LDS per reduction tile, the slices inside every tile
+    (1000, "naive;tile=16,32,200;mapToThreads=512,2;mapToBlocks=64,64;useMfma=1;useSharedMemory=1", 6),
+    (1000, "naive;tile=16,16,200;mapToThreads=256,1;mapToBlocks=64,64;useMfma=1;useSharedMemory=1;prefetchShared=1", 4),
+    # blocks loop over tiles: the partial tiles in LDS are reused from one iteration to the next
+    (512, "naive;tile=16,16;mapToThreads=256,2;mapToBlocks=2,3;useMfma=1", 8),
+    # a reduction whose length is no multiple of 4 lanes groups x steps
+    (203, "naive;tile=16,16;mapToThreads=256;mapToBlocks=64,64;useMfma=1", 4),
+])
+def test_reduction_split_over_wavefronts(k, opts, split):
+    """Fewer output tiles than wavefronts: the reduction steps of a tile are divided among several
+    wavefronts whose partial tiles meet in LDS."""
+    A, B = ints((40, k), k), ints((k, 70), k + 1)
+    ins = [torch.from_numpy(a).cuda() for a in (A, B)]
+    src = tc.compile(MM, "matmul", ins, opts).compiled_source
+    assert "ksplit0_" in src and f"sl_ < {split})" in src, src
+    (C,) = run(MM, "matmul", [A, B], opts)
+    assert np.array_equal(C, A @ B)
+
+
+def test_split_reduction_accumulates_into_existing_output_and_runs_the_epilogue():
+    src = "def mmacc(float(M, K) A, float(K, N) B) -> (C) { C(m, n) += A(m, r_k) * B(r_k, n) }"
+    A, B, C0 = ints((20, 400), 3), ints((400, 18), 4), ints((20, 18), 5)
+    opts = "naive;tile=16,16;mapToThreads=256,2;mapToBlocks=8,8;useMfma=1"
+    (C,) = run(src, "mmacc", [A, B], opts, outs_init=[C0])
+    assert np.array_equal(C, C0 + A @ B)
+    I, W1, B1 = ints((30, 600), 6), ints((50, 600), 7), ints((50,), 8)
+    (O,) = run(FC, "fc", [I, W1, B1], opts)
+    assert np.array_equal(O, np.maximum(I @ W1.T + B1, 0))
+    (ref,) = tc_oracle.run(FC, "fc", [I, W1, B1])
+    assert np.array_equal(O, ref)
