@@ -109,6 +109,37 @@ def define(tc, mapping_options_factory):
     return TC(tc, mapping_options_factory)
 
 
+def make_autograd(forward_fun, backward_fun):
+    """A callable with torch.autograd support from two functions on tensors (typically methods of
+    a `define`d TC): `forward_fun(*inputs)` computes the outputs, `backward_fun(*inputs,
+    *output_gradients)` the gradients of the inputs, in input order.  Counterpart of the reference's
+    helper (tensor_comprehensions/__init__.py:513-576): the inputs are saved for the backward
+    pass, incoming gradients are made contiguous, `backward_fun=None` gives no gradients."""
+    import torch
+
+    class _Op(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, *inputs):
+            ctx.save_for_backward(*inputs)
+            out = forward_fun(*inputs)
+            return tuple(out) if isinstance(out, (list, tuple)) else out
+
+        @staticmethod
+        def backward(ctx, *gradients):
+            saved = ctx.saved_tensors
+            if backward_fun is None:
+                return (None,) * len(saved)
+            grads = backward_fun(*saved, *[g.contiguous() for g in gradients])
+            grads = tuple(grads) if isinstance(grads, (list, tuple)) else (grads,)
+            if len(grads) != len(saved):
+                raise _tc.TcError(f"backward function returned {len(grads)} gradients for {len(saved)} inputs")
+            return grads
+
+    def apply(*inputs):
+        return _Op.apply(*inputs)
+    return apply
+
+
 def assert_almost_equal(actual, expected, *inputs, operations=1, precision=1e-7):
     """|actual - expected| <= precision * operations * max|input| elementwise bound of the reference's
     helper (tensor_comprehensions/__init__.py:47-71)."""

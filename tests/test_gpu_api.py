@@ -268,3 +268,42 @@ def test_autotune_from_the_naive_options_reaches_the_stored_options(name):
     torch.cuda.synchronize()
     for o, r in zip(outs, tc_oracle.run(src, entry, ins_np)):
         assert np.abs(o.cpu().numpy() - r).max() <= W.tolerance(k, r)
+
+
+def test_make_autograd_runs_forward_and_backward_comprehensions():
+    """The example of tensor_comprehensions/__init__.py:556-600 (a 1x1 convolution and its two
+    gradient TCs behind torch.autograd), checked against conv2d's own gradients."""
+    conv = """
+def convolution(float(N,C,H,W) I, float(M,C,KH,KW) W1) -> (O) {
+    O(n, m, h, w) +=! I(n, r_c, h + r_kh, w + r_kw) * W1(m, r_c, r_kh, r_kw)
+}
+def convolution_igrad(float(M,C,KH,KW) W1, float(N,M,H,W) d_O) -> (d_I) {
+    d_I(n, c, h, w) +=! d_O(n, r_m, h - r_kh, w - r_kw) * W1(r_m, c, r_kh, r_kw)
+}
+def convolution_wgrad(float(N,C,H,W) I, float(N,M,H,W) d_O) -> (d_W1) {
+    d_W1(m, c, kh, kw) +=! d_O(r_n, m, r_h - kh, r_w - kw) * I(r_n, c, r_h, r_w)
+}
+"""
+    T = tc.define(conv, tc.make_naive_options_factory())
+
+    def backward(I, W1, d_O):
+        return T.convolution_igrad(W1, d_O), T.convolution_wgrad(I, d_O)
+
+    op = tc.make_autograd(T.convolution, backward)
+    g = torch.Generator().manual_seed(3)
+    I = torch.randint(-3, 4, (2, 3, 9, 8), generator=g).float().cuda().requires_grad_()
+    W1 = torch.randint(-3, 4, (4, 3, 1, 1), generator=g).float().cuda().requires_grad_()
+    for _ in range(2):                                  # the second pass reuses the compiled kernels
+        I.grad = W1.grad = None
+        O = op(I, W1)
+        seed = torch.randint(-2, 3, O.shape, generator=g).float().cuda()
+        O.backward(seed)
+        I2, W2 = I.detach().clone().requires_grad_(), W1.detach().clone().requires_grad_()
+        O2 = torch.nn.functional.conv2d(I2, W2)
+        O2.backward(seed)
+        assert torch.equal(O, O2)                       # small integers: exact in any order
+        assert torch.equal(I.grad, I2.grad) and torch.equal(W1.grad, W2.grad)
+    # no backward function: no gradients flow to the inputs
+    I3 = I.detach().clone().requires_grad_()
+    tc.make_autograd(T.convolution, None)(I3, W1.detach()).sum().backward()
+    assert I3.grad is None

@@ -1,4 +1,6 @@
 """Host-side behaviour of the convenience layer (define / factories / TunerConfig / cache lookup)."""
+import pytest
+
 import tensorcomprehensions_amd as tc
 
 TWO_DEFS = """
@@ -51,3 +53,36 @@ def test_compile_is_reentrant_across_threads():
     with concurrent.futures.ThreadPoolExecutor(max_workers=8) as pool:
         parallel = list(pool.map(build, jobs * 3))
     assert parallel == serial * 3
+
+
+def test_make_autograd_wires_forward_and_backward_functions():
+    """The autograd helper itself needs no GPU: any two functions on tensors will do."""
+    import torch
+    calls = []
+
+    def forward(a, b):
+        calls.append("f")
+        return a * b
+
+    def backward(a, b, g):
+        calls.append(("b", g.is_contiguous()))
+        return g * b, g * a
+
+    op = tc.make_autograd(forward, backward)
+    a = torch.tensor([1.0, 2.0, 3.0], requires_grad=True)
+    b = torch.tensor([4.0, 5.0, 6.0], requires_grad=True)
+    out = op(a, b)
+    out.backward(torch.tensor([1.0, 10.0, 100.0]))
+    assert torch.equal(a.grad, torch.tensor([4.0, 50.0, 600.0])) and torch.equal(b.grad, torch.tensor([1.0, 20.0, 300.0]))
+    assert calls == ["f", ("b", True)]
+    # several outputs, as a list
+    two = tc.make_autograd(lambda x: [x + 1, x * 2], lambda x, g1, g2: g1 + 2 * g2)
+    x = torch.tensor([1.0, 2.0], requires_grad=True)
+    y1, y2 = two(x)
+    (y1.sum() + y2.sum()).backward()
+    assert torch.equal(x.grad, torch.tensor([3.0, 3.0]))
+    # a backward function must answer for every input
+    bad = tc.make_autograd(lambda p, q: p + q, lambda p, q, g: g)
+    p, q = torch.ones(2, requires_grad=True), torch.ones(2, requires_grad=True)
+    with pytest.raises(tc.TcError):
+        bad(p, q).sum().backward()
