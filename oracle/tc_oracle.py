@@ -21,7 +21,11 @@ Reference files followed (paths relative to the reference checkout):
 The loop nest is emitted as C (same text shape as the golden nests in
 test/test_core.cc:93-232), compiled with gcc -O3 without fast-math or FMA
 contraction, and called through ctypes on numpy arrays.  A pure-Python
-interpreter of the same nest (`run_python`) exists for tiny shapes.
+interpreter of the same nest (`run_python`) exists for tiny shapes.  Nests
+with float16 tensors (a type the reference's front end refuses, tc/lang/sema.h:62-66,
+so nothing of the reference pins them: "parity unpinned", checked against IEEE
+half arithmetic in numpy and closed forms instead) are compiled with the ROCm
+clang, `-fexcess-precision=16`: every operation is rounded to half.
 
 Pinned by tests/test_oracle_*.py against: the reference's range-inference
 known answers (test/test_inference.cc:70-540), its golden loop nests
@@ -31,8 +35,8 @@ and integer-valued inputs (exact sums).
 
 Known restriction: non-affine subscripts (indirection, %, /) contribute no range
 constraint here (the reference drops them with a warning once their variables
-are solved, tc2halide.cc:448-465); output tensors whose inferred minimum is not 0
-can be inferred but not executed.
+are solved, tc2halide.cc:448-465).  The storage of an output starts at its inferred
+lower bound (element k of a dimension holds the point min + k).
 """
 from __future__ import annotations
 
@@ -358,10 +362,10 @@ def match_types(a: str, b: str) -> str:
     return f"int{max(ba, bb)}"
 
 
-_CTYPE = {"float": "float", "double": "double", "int8": "int8_t", "int16": "int16_t", "int32": "int32_t",
+_CTYPE = {"float16": "_Float16", "float": "float", "double": "double", "int8": "int8_t", "int16": "int16_t", "int32": "int32_t",
           "int64": "int64_t", "uint8": "uint8_t", "uint16": "uint16_t", "uint32": "uint32_t",
           "uint64": "uint64_t", "bool": "uint8_t"}
-_NPTYPE = {"float": np.float32, "double": np.float64, "int8": np.int8, "int16": np.int16, "int32": np.int32,
+_NPTYPE = {"float16": np.float16, "float": np.float32, "double": np.float64, "int8": np.int8, "int16": np.int16, "int32": np.int32,
            "int64": np.int64, "uint8": np.uint8, "uint16": np.uint16, "uint32": np.uint32,
            "uint64": np.uint64, "bool": np.uint8}
 
@@ -735,6 +739,9 @@ _IDENT = {"+": "0", "*": "1"}
 def _identity(op: str, scalar: str) -> str:
     """Reduction identities (tc2halide.cc:574-601): 0, 1, type max, type min."""
     base = op.rstrip("!").rstrip("=")
+    if scalar == "float16":                         # the largest finite half is 65504
+        return {"+": "((_Float16)0.0f)", "*": "((_Float16)1.0f)", "min": "((_Float16)65504.0f)",
+                "max": "((_Float16)-65504.0f)"}[base]
     fl = scalar in ("float", "double")
     if base == "+":
         return "0.000000f" if scalar == "float" else ("0.0" if fl else "0")
@@ -788,6 +795,8 @@ class _CEmitter:
             args = [self.expr(a, rename, pretty) for a in e.args]
             return self.pretty_index(e.op, args) if pretty else self.index(e.op, args)
         if k == "builtin":
+            if e.type == "float16" and not pretty:   # no half math library: evaluated in float, rounded once
+                return f"((_Float16){e.op}f(" + ", ".join(self.cast(a, "float", rename) for a in e.args) + "))"
             fn = e.op + ("f" if e.type == "float" and not pretty else "")
             return f"{fn}(" + ", ".join(self.cast(a, e.type, rename, pretty) for a in e.args) + ")"
         if k == "cast":
@@ -807,10 +816,14 @@ class _CEmitter:
             if e.op in ("min", "max"):
                 if pretty:
                     return f"{e.op}({sa}, {sb})"
+                if mt == "float16":
+                    return f"((_Float16)f{e.op}f((float)({sa}), (float)({sb})))"
                 if mt in ("float", "double"):
                     return f"{'fminf' if e.op == 'min' else 'fmaxf'}({sa}, {sb})" if mt == "float" else f"f{e.op}({sa}, {sb})"
                 return f"(({sa}) {'<' if e.op == 'min' else '>'} ({sb}) ? ({sa}) : ({sb}))"
-            if e.op in ("/", "%") and mt not in ("float", "double") and not pretty:
+            if e.op == "%" and mt == "float16" and not pretty:
+                return f"((_Float16)fmodf((float)({sa}), (float)({sb})))"
+            if e.op in ("/", "%") and mt not in ("float16", "float", "double") and not pretty:
                 if mt.startswith("uint") or mt == "bool":
                     return f"({sa} {e.op} {sb})"     # unsigned: rounding down is truncation (and 2^63.. must not pass through int64)
                 return f"tc_floor{'div' if e.op == '/' else 'mod'}({sa}, {sb})"   # Halide integer semantics
@@ -871,6 +884,8 @@ class _CEmitter:
             fn = "min" if base == "min=" else "max"
             if pretty:
                 return f"{l} = {fn}({l}, {rhs});"
+            if s.scalar == "float16":
+                return f"{l} = (_Float16)f{fn}f((float)({l}), (float)({rhs}));"
             if s.scalar in ("float", "double"):
                 f = ("fminf" if fn == "min" else "fmaxf") if s.scalar == "float" else "f" + fn
                 return f"{l} = {f}({l}, {rhs});"
@@ -922,6 +937,7 @@ def emit_c(an: Analysis, fname: str = "tc_oracle_kernel") -> str:
 # Build + run
 # ----------------------------------------------------------------------------------------------
 _BUILD_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "_build")
+_CLANG = os.environ.get("TC_ORACLE_CLANG", "/opt/rocm/llvm/bin/clang")
 _CFLAGS = ["-O3", "-ffp-contract=off", "-fno-fast-math", "-shared", "-fPIC"]
 _cache: Dict[str, ctypes.CDLL] = {}
 
@@ -945,7 +961,11 @@ def build(an: Analysis, native: bool = False, in_tree: bool = False) -> ctypes.C
         with open(c, "w") as f:
             f.write(src)
         tmp = so + f".tmp{os.getpid()}"
-        subprocess.run(["gcc", *flags, "-o", tmp, c, "-lm"], check=True)
+        # gcc 11 has no _Float16 on x86-64: nests with half tensors go through the ROCm clang, every
+        # operation rounded to half (no excess precision carried from one operation to the next)
+        half = any(t.scalar == "float16" for t in an.tensors.values())
+        cc = [_CLANG, "-fexcess-precision=16"] if half else ["gcc"]
+        subprocess.run([*cc, *flags, "-o", tmp, c, "-lm"], check=True)
         os.replace(tmp, so)
     lib = ctypes.CDLL(so)
     _cache[key] = lib
@@ -993,19 +1013,19 @@ def run_python(tc: str, entry: str, inputs: Sequence[np.ndarray], acc_dtype=None
             return idx[e.op]
         if k == "access":
             v = env[e.op][tuple(int(ev(a, idx)) - m for a, m in zip(e.args, an.tensors[e.op].mins))]
-            return acc_dtype(v) if acc_dtype and e.type in ("float", "double") else v
+            return acc_dtype(v) if acc_dtype and e.type in ("float16", "float", "double") else v
         if k == "bin":
             a, b = ev(e.args[0], idx), ev(e.args[1], idx)
             mt = match_types(e.args[0].type, e.args[1].type)
-            if mt in ("float", "double"):
+            if mt in ("float16", "float", "double"):
                 ty = acc_dtype or _NPTYPE[mt]
                 a, b = ty(a), ty(b)
             op = e.op
             if op == "+": return a + b
             if op == "-": return a - b
             if op == "*": return a * b
-            if op == "/": return a / b if mt in ("float", "double") else a // b
-            if op == "%": return math.fmod(a, b) if mt in ("float", "double") else a % b
+            if op == "/": return a / b if mt in ("float16", "float", "double") else a // b
+            if op == "%": return math.fmod(a, b) if mt in ("float16", "float", "double") else a % b
             if op == "min": return min(a, b)
             if op == "max": return max(a, b)
             return {"==": a == b, "!=": a != b, "<": a < b, ">": a > b, "<=": a <= b, ">=": a >= b,

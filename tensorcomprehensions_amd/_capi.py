@@ -119,7 +119,7 @@ def take_string(ptr):
 
 # dtype code/bits per numpy/torch dtype name
 DTYPES = {
-    "float32": (2, 32), "float64": (2, 64), "int8": (0, 8), "int16": (0, 16), "int32": (0, 32),
+    "float16": (2, 16), "float32": (2, 32), "float64": (2, 64), "int8": (0, 8), "int16": (0, 16), "int32": (0, 32),
     "int64": (0, 64), "uint8": (1, 8), "uint16": (1, 16), "uint32": (1, 32), "uint64": (1, 64), "bool": (1, 8),
 }
 

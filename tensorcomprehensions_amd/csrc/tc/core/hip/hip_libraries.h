@@ -49,6 +49,8 @@ template <typename T> __device__ __forceinline__ T tmin(T a, T b) { return a < b
 template <typename T> __device__ __forceinline__ T tmax(T a, T b) { return a > b ? a : b; }
 __device__ __forceinline__ float tmin(float a, float b) { return fminf(a, b); }
 __device__ __forceinline__ float tmax(float a, float b) { return fmaxf(a, b); }
+__device__ __forceinline__ _Float16 tmin(_Float16 a, _Float16 b) { return (_Float16)fminf((float)a, (float)b); }
+__device__ __forceinline__ _Float16 tmax(_Float16 a, _Float16 b) { return (_Float16)fmaxf((float)a, (float)b); }
 __device__ __forceinline__ double tmin(double a, double b) { return fmin(a, b); }
 __device__ __forceinline__ double tmax(double a, double b) { return fmax(a, b); }
 } // namespace __tc
@@ -85,6 +87,9 @@ template <int CTRL, typename T> __device__ __forceinline__ T dppMov(T v) {
     return __builtin_bit_cast(T, ((unsigned long long)hi << 32) | lo);
   } else if constexpr (sizeof(T) == 4) {
     return __builtin_bit_cast(T, dppMov32<CTRL>(__builtin_bit_cast(int, v)));
+  } else if constexpr (sizeof(T) == 2) {
+    // by bit pattern: the element may be a half
+    return __builtin_bit_cast(T, (unsigned short)dppMov32<CTRL>((int)__builtin_bit_cast(unsigned short, v)));
   } else {
     return (T)dppMov32<CTRL>((int)v);
   }
@@ -95,6 +100,8 @@ template <int MASK, typename T> __device__ __forceinline__ T laneXor(T v) {
     return __builtin_bit_cast(T, __shfl_xor(__builtin_bit_cast(unsigned long long, v), MASK, 64));
   } else if constexpr (sizeof(T) == 4) {
     return __builtin_bit_cast(T, __shfl_xor(__builtin_bit_cast(int, v), MASK, 64));
+  } else if constexpr (sizeof(T) == 2) {
+    return __builtin_bit_cast(T, (unsigned short)__shfl_xor((int)__builtin_bit_cast(unsigned short, v), MASK, 64));
   } else {
     return (T)__shfl_xor((int)v, MASK, 64);
   }

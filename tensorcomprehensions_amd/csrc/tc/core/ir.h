@@ -30,7 +30,7 @@ struct ScalarType {
   // spelling in generated device / host C
   std::string cName() const {
     if (code == Float) {
-      return bits == 64 ? "double" : "float";
+      return bits == 64 ? "double" : bits == 16 ? "_Float16" : "float";
     }
     if (isBool()) {
       return "bool";

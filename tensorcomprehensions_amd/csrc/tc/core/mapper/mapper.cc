@@ -122,7 +122,7 @@ std::string floatLiteral(double v, const ScalarType& t) {
   if (s.find("inf") != std::string::npos || s.find("nan") != std::string::npos) {
     return v > 0 ? "(1.0f/0.0f)" : "(-1.0f/0.0f)";
   }
-  return t.bits == 64 ? s : s + "f";
+  return t.bits == 64 ? s : t.bits == 16 ? "((_Float16)" + s + "f)" : s + "f";
 }
 
 int64_t ceilDiv(int64_t a, int64_t b) {

@@ -242,11 +242,14 @@ class StageCodegen {
         return "(" + expr(e->args[0], accRef) + " ? " + castTo(e->args[1], e->type, accRef) + " : " +
             castTo(e->args[2], e->type, accRef) + ")";
       case Expr::Call: {
+        // half has no math library of its own: evaluated in float, rounded once
+        const bool half = e->type.isFloat() && e->type.bits == 16;
+        const ScalarType argType = half ? ScalarType{ScalarType::Float, 32} : e->type;
         std::string s = e->name + "(";
         for (size_t i = 0; i < e->args.size(); ++i) {
-          s += (i ? ", " : "") + castTo(e->args[i], e->type, accRef);
+          s += (i ? ", " : "") + castTo(e->args[i], argType, accRef);
         }
-        return s + ")";
+        return half ? "((_Float16)" + s + "))" : s + ")";
       }
       case Expr::Binary: {
         ScalarType mt = matchType(e->args[0]->type, e->args[1]->type);
@@ -258,6 +261,7 @@ class StageCodegen {
         if (e->name == "max") return "__tc::tmax(" + a + ", " + b + ")";
         if (e->name == "/" && !mt.isFloat()) return "__tc::floordiv(" + a + ", " + b + ")";
         if (e->name == "%" && !mt.isFloat()) return "__tc::floormod(" + a + ", " + b + ")";
+        if (e->name == "%" && mt.bits == 16) return "((_Float16)fmodf((float)" + a + ", (float)" + b + "))";
         if (e->name == "%") return std::string(mt.bits == 64 ? "fmod(" : "fmodf(") + a + ", " + b + ")";
         return "(" + a + " " + e->name + " " + b + ")";
       }

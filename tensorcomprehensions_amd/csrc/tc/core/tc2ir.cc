@@ -83,6 +83,15 @@ Affine toAffine(const ExprRef& e) {
 }
 
 std::string identityLiteral(ReduceOp op, const ScalarType& t) {
+  if (t.isFloat() && t.bits == 16) {
+    // largest finite half is 65504
+    switch (op) {
+      case ReduceOp::Times: return "((_Float16)1.0f)";
+      case ReduceOp::Min: return "((_Float16)65504.0f)";
+      case ReduceOp::Max: return "((_Float16)-65504.0f)";
+      default: return "((_Float16)0.0f)";
+    }
+  }
   auto lit = [&](double v) -> std::string {
     std::ostringstream ss;
     if (t.isFloat()) {

@@ -355,3 +355,16 @@ def test_promotion_for_coalescing_alone():
     assert "lds0_A[1056]" in src                        # 32 x 32 tile, pitch 33
     src, _ = mapped("def cp(float(N, M) A) -> (O) { O(i, j) = A(i, j) }", "cp", [(4096, 4096)], o)
     assert "lds0_A" not in src
+
+
+def test_every_scalar_type_maps_including_half():
+    """The type sweep of test/test_tc2halide.cc:201-222, with the float16 it leaves out (the
+    reference's front end refuses the type, tc/lang/sema.h:62-66; hipRTC needs no header for it)."""
+    spelled = {"bool": "bool", "uint8": "unsigned char", "uint16": "unsigned short", "uint32": "unsigned int",
+               "uint64": "unsigned long long", "int8": "signed char", "int16": "short", "int32": "int", "int64": "long long",
+               "float16": "_Float16", "float32": "float", "float64": "double", "float": "float", "double": "double"}
+    for name, c in spelled.items():
+        dtype = {"float": "float32", "double": "float64"}.get(name, name)
+        src, _ = tc.map_only(f"def test_type({name}(N) A) -> (B) {{ B(k) +=! A(i) where k in 0:1 }}", "test_type",
+                             [ShapeOnly((100,), dtype)], "naive")
+        assert f"const {c}* __restrict__ pA" in src, name

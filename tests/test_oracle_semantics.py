@@ -211,3 +211,20 @@ def test_storage_of_an_output_starts_at_its_inferred_lower_bound():
         O, P = runner(src, "f", [A])
         assert np.array_equal(O, 2 * A[3:, 1:5])
         assert np.array_equal(P, (2 * A[3:, 1:5] + A[:9, 1:5]).sum(1))
+
+
+def test_half_is_rounded_after_every_operation():
+    """float16 nests are compiled by clang without excess precision: a product is rounded to half
+    before it is added, sums accumulate in half."""
+    src = "def f(float16(N) a, float16(N) b, float16(N) c) -> (o, s, t) { o(i) = a(i) * b(i) + c(i)\n s(k) +=! a(i) where k in 0:1\n t(k) +=! float(a(i)) where k in 0:1 }"
+    a = np.array([1.0009765625, 3.0, 2049.0 - 1.0], np.float16)      # 1 + 2^-10, 3, 2048
+    b = np.array([1.0009765625, 0.5, 1.0], np.float16)
+    c = np.array([-1.0, 0.25, 1.0], np.float16)
+    o, s, t = tc_oracle.run(src, "f", [a, b, c])
+    assert o.dtype == np.float16 and s.dtype == np.float16 and t.dtype == np.float32
+    # (1 + 2^-10)^2 = 1 + 2^-9 + 2^-20 rounds to 1 + 2^-9 before the subtraction; 2048 + 1 rounds to 2048
+    assert np.array_equal(o, np.array([2.0 ** -9, 1.75, 2048.0], np.float16))
+    half_sum = np.float16(0)
+    for v in a:
+        half_sum = np.float16(half_sum + v)
+    assert s[0] == half_sum and t[0] == np.float32(a.astype(np.float32).sum())
