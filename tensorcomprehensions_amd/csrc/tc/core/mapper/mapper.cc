@@ -412,6 +412,52 @@ void emitKernel(KernelCtx& kc, const DeviceLimits& limits, Emitter& em) {
       }
     }
   }
+  // Producer -> consumer through LDS (useSharedMemory): a tensor exactly one stage of the kernel
+  // writes and later stages read, when every reader's box of one kernel-level iteration lies inside
+  // the producer's and that box fits what is left of LDS.  Stages see the tensor through views that
+  // may merge dimensions differently: only identical views are matched.
+  if (kc.opts.useSharedMemoryValue) {
+    for (size_t i = 0; i + 1 < gens.size(); ++i) {
+      const StagePlan& prod = k.stages[i];
+      const std::string& t = prod.tensor;
+      bool sole = true;
+      for (size_t j = 0; j < k.stages.size(); ++j) sole &= j == i || k.stages[j].tensor != t;
+      if (!sole || tensorsRead(prod).count(t)) continue;
+      auto wbox = gens[i].writeBox();
+      if (!wbox.valid) continue;
+      bool anyReader = false, ok = true;
+      for (size_t j = i + 1; j < gens.size() && ok; ++j) {
+        if (!tensorsRead(k.stages[j]).count(t)) continue;
+        anyReader = true;
+        ok = k.stages[j].views.at(t).extents == prod.views.at(t).extents;
+        auto rbox = ok ? gens[j].readBox(t) : StageCodegen::IterationBox();
+        ok = ok && rbox.valid && rbox.low.size() == wbox.low.size();
+        for (size_t d = 0; ok && d < wbox.low.size(); ++d) {
+          int64_t delta = rbox.low[d].constant - wbox.low[d].constant;
+          ok = rbox.low[d].coef == wbox.low[d].coef && delta >= 0 && delta + rbox.extents[d] <= wbox.extents[d];
+        }
+      }
+      if (!anyReader || !ok) continue;
+      KernelCtx::Forward f;
+      f.producer = static_cast<int>(i);
+      f.ldsName = "fwd" + std::to_string(i) + "_" + t;
+      f.extents = wbox.extents;
+      // pitches: one that is a multiple of the 32 banks puts the lanes (or the four lane groups
+      // of a matrix-core operand read) that step along its dimension onto the same banks; four
+      // elements more spread them and keep rows 16-byte aligned
+      f.strides.assign(wbox.extents.size(), 1);
+      for (size_t d = wbox.extents.size(); d-- > 1;) {
+        f.strides[d - 1] = f.strides[d] * wbox.extents[d];
+        if (f.strides[d - 1] % 32 == 0 && wbox.extents[d - 1] > 1) f.strides[d - 1] += 4;
+      }
+      f.elems = wbox.extents.empty() ? 1 : f.strides[0] * wbox.extents[0];
+      int64_t bytes = f.elems * prod.views.at(t).type.bytes();
+      if (bytes > ldsBudget) continue;
+      ldsBudget -= bytes;
+      for (const auto& low : wbox.low) f.lows.push_back(StageCodegen::tileAffineStr(low));
+      kc.forwards[t] = f;
+    }
+  }
   k.ldsBytes = (before - ldsBudget) + scratchElems * 8;
 
   // Register promotion across stages (usePrivateMemory): an input that several stages read with
@@ -514,6 +560,10 @@ void emitKernel(KernelCtx& kc, const DeviceLimits& limits, Emitter& em) {
     em.line("__shared__ double red_scratch_raw_[" + std::to_string(scratchElems) + "];");
   }
   for (auto& g : gens) g.emitLdsDecls();
+  for (const auto& fw : kc.forwards) {
+    em.line("__shared__ __attribute__((aligned(16))) " + k.stages[fw.second.producer].views.at(fw.first).type.cName() + " " +
+            fw.second.ldsName + "[" + std::to_string(fw.second.elems) + "];");
+  }
   // kernel-level tile loops over the shared parallel variables (taken from the first stage):
   // first the tile indices that are plain block ids, then the loops, outermost first
   int opened = 0;
@@ -606,6 +656,9 @@ void emitKernel(KernelCtx& kc, const DeviceLimits& limits, Emitter& em) {
       }
     }
     for (const auto& sy : findBestSyncs(need, opened > 0)) syncAfter[sy.first] = static_cast<int>(sy.second);
+    // a producer's copy in LDS is overwritten by the next kernel-level iteration: not before the
+    // readers of this one are done
+    if (opened > 0 && !kc.forwards.empty()) syncAfter.back() = std::max(syncAfter.back(), level);
   }
   auto emitSync = [&](int level) {
     if (level == static_cast<int>(SyncLevel::Block)) {

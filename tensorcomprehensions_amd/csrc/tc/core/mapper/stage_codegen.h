@@ -41,6 +41,17 @@ struct KernelCtx {
   // bits (loop variables stay int: every extent is below 2^31).
   bool wide = false;
   bool kernelLoops = false; // the stages sit inside loops over tiles that the blocks share out
+  // A tensor one stage of the kernel produces and later stages of the same kernel read: the part
+  // a block produces during one kernel-level iteration is kept in LDS as well (the producer stores
+  // every element to both places) and the readers take it from there instead of from memory.
+  struct Forward {
+    std::string ldsName;
+    int producer = 0;
+    std::vector<std::string> lows;   // origin of the block's box per view dimension, as C
+    std::vector<int64_t> extents, strides;
+    int64_t elems = 0;
+  };
+  std::map<std::string, Forward> forwards;
   int64_t NT() const { return k.block[0] * k.block[1] * k.block[2]; }
 };
 
@@ -171,6 +182,95 @@ class StageCodegen {
     return true;
   }
 
+  // Box of elements of a tensor this stage touches through subscripts of one shape during one
+  // kernel-level iteration: kernel-level variables span their tile, every other variable its
+  // whole extent.  Origins are affine in the kernel-level tile indices (symbols "t_<var>").
+  struct IterationBox {
+    bool valid = false;
+    std::vector<Affine> low;
+    std::vector<int64_t> extents;
+  };
+  IterationBox iterationBox(const std::vector<std::vector<Affine>>& accesses) const {
+    IterationBox box;
+    if (accesses.empty()) return box;
+    const auto& ref = accesses.front();
+    for (const auto& a : accesses) {
+      if (a.size() != ref.size()) return box;
+      for (size_t j = 0; j < a.size(); ++j) {
+        if (!a[j].valid || a[j].coef != ref[j].coef) return box;
+      }
+    }
+    for (size_t j = 0; j < ref.size(); ++j) {
+      int64_t lo = ref[j].constant, hi = ref[j].constant;
+      for (const auto& a : accesses) {
+        lo = std::min(lo, a[j].constant);
+        hi = std::max(hi, a[j].constant);
+      }
+      Affine low;
+      low.valid = true;
+      low.constant = lo;
+      int64_t ext = 1 + hi - lo;
+      for (const auto& c : ref[j].coef) {
+        if (c.second == 0) continue;
+        const LoopVar& v = var(c.first);
+        int pos = 0;
+        for (size_t i = 0; i < st_.vars.size(); ++i) {
+          if (st_.vars[i].name == v.name) pos = static_cast<int>(i);
+        }
+        const bool kernelLevel = !v.reduction && pos < kc_.k.sharedDepth;
+        const int64_t span = kernelLevel ? v.tile : v.extent;
+        int64_t base = v.min;
+        if (c.second < 0) base += span - 1;
+        low.constant += c.second * base;
+        if (kernelLevel && v.numTiles > 1) low.coef["t_" + v.name] += c.second * v.tile;
+        ext += std::abs(c.second) * (span - 1);
+      }
+      box.low.push_back(low);
+      box.extents.push_back(ext);
+    }
+    box.valid = true;
+    return box;
+  }
+  IterationBox writeBox() const {
+    std::vector<Affine> subs;
+    for (const auto& e : st_.lhsSubs) subs.push_back(ir::toAffine(e));
+    return iterationBox({subs});
+  }
+  // every load of `tensor` in the stage; invalid when one of them is not affine
+  IterationBox readBox(const std::string& tensor) const {
+    std::vector<std::vector<Affine>> accesses;
+    for (const auto& stmt : st_.stmts) {
+      visit(stmt.rhs, [&](const ExprRef& e) {
+        if (e->kind != Expr::Load || e->name != tensor) return;
+        std::vector<Affine> subs;
+        for (const auto& a : e->args) subs.push_back(ir::toAffine(a));
+        accesses.push_back(subs);
+      });
+    }
+    return iterationBox(accesses);
+  }
+  static std::string tileAffineStr(const Affine& a) {
+    std::ostringstream ss;
+    ss << a.constant;
+    for (const auto& c : a.coef) {
+      if (c.second != 0) ss << (c.second < 0 ? " - " : " + ") << std::abs(c.second) << " * " << c.first;
+    }
+    return ss.str();
+  }
+  const KernelCtx::Forward* forwardOf(const std::string& tensor) const {
+    auto it = kc_.forwards.find(tensor);
+    return it == kc_.forwards.end() ? nullptr : &it->second;
+  }
+  std::string forwardIndex(const KernelCtx::Forward& f, const std::vector<ExprRef>& subs) {
+    std::ostringstream ss;
+    for (size_t j = 0; j < subs.size(); ++j) {
+      if (j) ss << " + ";
+      ss << "((" << affineStr(ir::toAffine(subs[j])) << ") - (" << f.lows[j] << "))";
+      if (f.strides[j] != 1) ss << " * " << f.strides[j];
+    }
+    return ss.str();
+  }
+
   // The stage's result when nothing later in this kernel reads it back: it is stored with
   // device-scope write-through (buffer stores with the sc1 bit).  A plain or non-temporal store
   // leaves the line dirty in the L2 of its XCD, and everything still dirty when the last wavefront
@@ -179,6 +279,7 @@ class StageCodegen {
   // Byte offsets of a buffer access are 32 bits wide, which bounds the tensors this applies to.
   bool streamedStore() const {
     if (!kc_.opts.useReadOnlyCacheValue || viewBytes(st_.tensor) >= (int64_t(1) << 31)) return false;
+    if (forwardOf(st_.tensor)) return true; // the later stages read the copy in LDS
     for (size_t j = stageIdx_ + 1; j < kc_.k.stages.size(); ++j) {
       if (tensorsRead(kc_.k.stages[j]).count(st_.tensor)) return false;
     }
@@ -188,10 +289,14 @@ class StageCodegen {
 
   std::string storeStmt(const std::string& cond, const std::string& value) {
     std::string index = flatIndex(st_.tensor, st_.lhsSubs, "");
-    if (streamedStore()) {
-      return "if (" + cond + ") __tc::storeThrough(" + bufferName(st_.tensor) + ", " + index + ", " + value + ");";
+    std::string store = streamedStore()
+        ? "__tc::storeThrough(" + bufferName(st_.tensor) + ", " + index + ", " + value + ");"
+        : "p" + st_.tensor + "[" + index + "] = " + value + ";";
+    const KernelCtx::Forward* f = forwardOf(st_.tensor);
+    if (f && f->producer == stageIdx_) {
+      return "if (" + cond + ") { " + store + " " + f->ldsName + "[" + forwardIndex(*f, st_.lhsSubs) + "] = " + value + "; }";
     }
-    return "if (" + cond + ") p" + st_.tensor + "[" + index + "] = " + value + ";";
+    return "if (" + cond + ") " + store;
   }
 
   std::string loadStr(const ExprRef& e, const std::string& accRef) {
@@ -205,6 +310,9 @@ class StageCodegen {
       if (p.tensor == e->name && activePromotions_.count(p.tensor)) {
         return p.ldsName + "[" + ldsIndex(p, e->args) + "]";
       }
+    }
+    if (const KernelCtx::Forward* f = forwardOf(e->name)) {
+      if (f->producer < stageIdx_) return f->ldsName + "[" + forwardIndex(*f, e->args) + "]";
     }
     std::string global = "p" + e->name + "[" + flatIndex(e->name, e->args, accRef) + "]";
     {
@@ -468,6 +576,10 @@ class StageCodegen {
       // (promotionImprovesCoalescing, tc/core/polyhedral/cuda/memory_promotion_heuristic.cc:211-244).
       const bool coalesces = lanesWalkOuterDim(ref) && c.p.extents.back() >= 8;
       if (c.p.reuse < 2 && !coalesces) continue;
+      // A footprint of fewer elements than the block has threads is read where it lies: the copy
+      // would put two block barriers around less than one load per thread (the 16x16 factors of
+      // the Kronecker product, staged inside its tile loops, cost 3 us of 17).
+      if (elems < kc_.NT()) continue;
       // Pitches.  pad[j] = elements added to the distance between consecutive indices of dimension j.
       const size_t nd = ref.size();
       std::vector<int64_t> pad(nd, 0);
@@ -1460,7 +1572,7 @@ class StageCodegen {
       decodeGroup(st_.mfmaM, "mposa_", true);
       // consecutive steps of a lane read consecutive elements when the operand's reduction
       // subscripts are jointly contiguous: four steps are then fetched with one 16-byte load
-      bool contiguous = !residentFromLds && aligned && quarter * 4 == KT && ksteps % 4 == 0;
+      bool contiguous = !residentFromLds && !forwardOf(loadA->name) && aligned && quarter * 4 == KT && ksteps % 4 == 0;
       {
         Affine fa = flatAffine(loadA->name, loadA->args);
         contiguous &= fa.valid;

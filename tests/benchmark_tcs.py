@@ -217,7 +217,7 @@ TUNED_AT_REFERENCE_SIZES = {
                                          "mapToBlocks=256,256;usePrivateMemory=1;useReadOnlyCache=1;vectorWidth=4",
     "kronecker3": "naive;outerScheduleFusionStrategy=Max;intraTileScheduleFusionStrategy=Max;tile=1,32,16;unroll=8;"
                   "tileImperfectlyNested=1;mapToThreads=32,32;mapToBlocks=256,32;useReadOnlyCache=1;privateDepth=5;"
-                  "collapseContiguous=0;useMfma=1;prefetchShared=1",
+                  "collapseContiguous=0;useMfma=1;prefetchShared=1;useSharedMemory=1",
     "wavenet1": "naive;intraTileScheduleFusionStrategy=Max;fixParametersBeforeScheduling=1;tile=2,2000,16,1;mapToThreads=16,64;"
                 "mapToBlocks=2000,256;useSharedMemory=1;usePrivateMemory=1;privateDepth=8;sharedDepth=3;vectorWidth=4;"
                 "collapseContiguous=0;prefetchShared=1",

@@ -106,3 +106,54 @@ def test_transposed_read_is_staged_for_coalescing(options):
     assert np.array_equal(got, A.T)
     (ref,) = tc_oracle.run(src, "tr", [A])
     assert np.array_equal(got, ref)
+
+
+CHAIN = """def chain(float(M, K) A, float(K, N) W) -> (B, C, D) {
+    B(m, k) = A(m, k) * 2.0 + 1.0
+    C(m, n) +=! B(m, r_k) * W(r_k, n)
+    D(m) +=! C(m, r_n) + B(m, 0)
+}"""
+
+
+@pytest.mark.parametrize("options,forwarded", [
+    ("naive;tile=4,32;mapToThreads=32,4;mapToBlocks=64;useSharedMemory=1;outerScheduleFusionStrategy=Max;unroll=4", True),
+    # blocks loop over row tiles: the copies in LDS are rewritten every iteration
+    ("naive;tile=4,32;mapToThreads=32,4;mapToBlocks=3;useSharedMemory=1;outerScheduleFusionStrategy=Max;unroll=4", True),
+    ("naive;tile=8,16;mapToThreads=64,2;mapToBlocks=5;useSharedMemory=1;outerScheduleFusionStrategy=Max;useMfma=1", True),
+    ("naive;tile=4,32;mapToThreads=32,4;mapToBlocks=64;useSharedMemory=0;outerScheduleFusionStrategy=Max;unroll=4", False),
+    # a budget the producer's box does not fit: the readers go to memory
+    ("naive;tile=4,32;mapToThreads=32,4;mapToBlocks=64;useSharedMemory=1;maxSharedMemory=512;outerScheduleFusionStrategy=Max", False),
+])
+def test_producer_to_consumer_through_lds(options, forwarded):
+    """A tensor one stage of a kernel writes and later stages read is kept in LDS as well for the
+    block's part of it: the readers never go to memory for it."""
+    rng = np.random.Generator(np.random.Philox(46))
+    A = rng.integers(-3, 4, size=(40, 48)).astype(np.float32)
+    Wt = rng.integers(-3, 4, size=(48, 70)).astype(np.float32)
+    got, ex = run(CHAIN, "chain", [A, Wt], options)
+    assert ("fwd0_B[" in ex.compiled_source) == forwarded, options
+    B = A * 2 + 1
+    C = B @ Wt
+    D = C.sum(1) + 70 * B[:, 0]
+    ref = tc_oracle.run(CHAIN, "chain", [A, Wt])
+    for r, closed in zip(ref, (B, C, D)):
+        assert np.array_equal(r, closed)                   # small integers: exact in any order
+    for g, r in zip(got, ref):
+        assert np.array_equal(g, r), options
+
+
+def test_reader_of_other_blocks_rows_stays_in_a_kernel_of_its_own():
+    """Rows another block produces are read through memory, after the producing kernel: such a
+    reader is not fused with its producer, and nothing is forwarded."""
+    src = """def shifted(float(M, K) A) -> (B, C) {
+        B(m, k) = A(m, k) + 1.0
+        C(m, k) = B(m + 1, k) + B(m, k) where m in 0:M-1
+    }"""
+    A = np.random.Generator(np.random.Philox(47)).integers(-9, 10, size=(33, 40)).astype(np.float32)
+    opts = "naive;tile=4,40;mapToThreads=40,4;mapToBlocks=64;useSharedMemory=1;outerScheduleFusionStrategy=Max"
+    got, ex = run(src, "shifted", [A], opts)
+    assert "fwd0_B" not in ex.compiled_source and ex.num_kernels == 2
+    ref = tc_oracle.run(src, "shifted", [A])
+    assert np.array_equal(ref[1], (A[1:] + 1) + (A[:-1] + 1))
+    for g, r in zip(got, ref):
+        assert np.array_equal(g, r)
