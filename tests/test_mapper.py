@@ -368,3 +368,21 @@ def test_every_scalar_type_maps_including_half():
         src, _ = tc.map_only(f"def test_type({name}(N) A) -> (B) {{ B(k) +=! A(i) where k in 0:1 }}", "test_type",
                              [ShapeOnly((100,), dtype)], "naive")
         assert f"const {c}* __restrict__ pA" in src, name
+
+
+def test_written_tensor_is_forwarded_to_later_stages_through_lds():
+    """Producer -> consumer through LDS (the reference promotes written references and copies them
+    out, memory_promotion.cc:507-524): the producer stores to memory and to the block's copy, the
+    reader indexes the copy; a barrier closes each iteration of a kernel-level loop."""
+    chain = """def chain(float(M, K) A, float(K, N) W) -> (B, C) {
+        B(m, k) = A(m, k) * 2.0 + 1.0
+        C(m, n) +=! B(m, r_k) * W(r_k, n) }"""
+    base = "naive;tile=4,32;mapToThreads=32,4;outerScheduleFusionStrategy=Max;unroll=4"
+    src, launches = mapped(chain, "chain", [(40, 48), (48, 70)], base + ";mapToBlocks=64;useSharedMemory=1")
+    assert len(launches) == 1 and "float fwd0_B[192];" in src                    # 4 rows x 48
+    assert "pB[i_k + 48 * i_m] = acc_[a_]; fwd0_B[((i_m) - (0 + 4 * t_m)) * 48 + ((i_k) - (0))] = acc_[a_];" in src
+    assert "(fwd0_B[((i_m) - (0 + 4 * t_m)) * 48 + ((i_r_k_s1) - (0))] * " in src and "pB[" not in src.split("// stage 1")[1]
+    looped, _ = mapped(chain, "chain", [(40, 48), (48, 70)], base + ";mapToBlocks=3;useSharedMemory=1")
+    assert looped.count("__syncthreads();") == src.count("__syncthreads();") + 1
+    plain, _ = mapped(chain, "chain", [(40, 48), (48, 70)], base + ";mapToBlocks=64;useSharedMemory=0")
+    assert "fwd0_B" not in plain
