@@ -212,12 +212,14 @@ TUNED_AT_REFERENCE_SIZES = {
                 "tileImperfectlyNested=1;matchLibraryCalls=1;mapToThreads=256;mapToBlocks=1152;usePrivateMemory=1;"
                 "unrollCopyShared=1;vectorWidth=2;collapseContiguous=0;useMfma=1",
     # 576 threads x float4 = one 48x48 plane per pass: the normalising stage then finds every
-    # element in the register cache the two reductions filled (one read of the input)
-    "group_normalization_single_kernel": "naive;outerScheduleFusionStrategy=Max;tile=1,1;unroll=64;matchLibraryCalls=1;mapToThreads=576;"
-                                         "mapToBlocks=256,256;usePrivateMemory=1;useReadOnlyCache=1;vectorWidth=4",
-    "kronecker3": "naive;outerScheduleFusionStrategy=Max;intraTileScheduleFusionStrategy=Max;tile=1,32,16;unroll=8;"
-                  "tileImperfectlyNested=1;mapToThreads=32,32;mapToBlocks=256,32;useReadOnlyCache=1;privateDepth=5;"
-                  "collapseContiguous=0;useMfma=1;prefetchShared=1;useSharedMemory=1",
+    # element in the register cache the two reductions filled (one read of the input); two groups
+    # per block
+    "group_normalization_single_kernel": "naive;outerScheduleFusionStrategy=Max;intraTileScheduleFusionStrategy=Preserve3Coincident;"
+                                         "tile=1,2,0;unroll=128;matchLibraryCalls=1;mapToThreads=576;mapToBlocks=256,256;"
+                                         "useSharedMemory=1;usePrivateMemory=1;useReadOnlyCache=1;vectorWidth=4",
+    "kronecker3": "naive;outerScheduleFusionStrategy=Max;intraTileScheduleFusionStrategy=Max;tile=1,32,32;unroll=8;"
+                  "tileImperfectlyNested=1;mapToThreads=64,16;mapToBlocks=256,256;useSharedMemory=1;useReadOnlyCache=1;"
+                  "privateDepth=5;collapseContiguous=0;useMfma=1;prefetchShared=1",
     "wavenet1": "naive;intraTileScheduleFusionStrategy=Max;fixParametersBeforeScheduling=1;tile=2,2000,16,1;mapToThreads=16,64;"
                 "mapToBlocks=2000,256;useSharedMemory=1;usePrivateMemory=1;privateDepth=8;sharedDepth=3;vectorWidth=4;"
                 "collapseContiguous=0;prefetchShared=1",
