@@ -508,8 +508,22 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
             cand->invalid = true;
             continue;
           }
+          // Ten samples, the median is the fitness (tc/autotuner/autotuner-inl.h:140-170).  The
+          // events around a single launch of a few microseconds see the dispatch path more than the
+          // kernel, and the order of short candidates then comes out at random: a sample of a short
+          // kernel is the mean over as many back-to-back launches as fill about 200 us (at most 64).
           std::vector<int64_t> runs;
-          for (int r = 0; r < 10; ++r) runs.push_back(ex.profile(ins, outs).kernelRuntime.toNanoSeconds());
+          const int64_t warmNs = std::max<int64_t>(1, warm.kernelRuntime.toNanoSeconds());
+          const int repeats = warmNs >= 50000 ? 1 : static_cast<int>(std::min<int64_t>(64, std::max<int64_t>(1, 200000 / warmNs)));
+          if (repeats == 1) {
+            for (int r = 0; r < 10; ++r) runs.push_back(ex.profile(ins, outs).kernelRuntime.toNanoSeconds());
+          } else {
+            std::vector<const void*> in;
+            std::vector<void*> out;
+            for (auto t : ins) in.push_back(static_cast<const char*>(t->data) + t->byte_offset);
+            for (auto t : outs) out.push_back(static_cast<char*>(t->data) + t->byte_offset);
+            for (int r = 0; r < 10; ++r) runs.push_back(ex.profileRepeated(in, out, repeats).toNanoSeconds() / repeats);
+          }
           Duration med = Duration::fromNanoSeconds(median(runs));
           if (med == Duration::zero()) {
             cand->invalid = true;
