@@ -25,7 +25,8 @@ extern "C" {
 #ifndef TC_DLPACK_TYPES_DEFINED
 #define TC_DLPACK_TYPES_DEFINED
 typedef struct { int32_t device_type; int32_t device_id; } tc_dl_context;
-typedef struct { uint8_t code; uint8_t bits; uint16_t lanes; } tc_dl_datatype; /* code: 0 int, 1 uint, 2 float */
+/* code: 0 int (8, 16, 32, 64 bits), 1 uint (8 = uint8 or bool, 16, 32, 64), 2 float (16, 32, 64) */
+typedef struct { uint8_t code; uint8_t bits; uint16_t lanes; } tc_dl_datatype;
 typedef struct {
   void* data;
   tc_dl_context ctx;
