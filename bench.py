@@ -250,6 +250,8 @@ def suite_library_routines():
         "group_convolution": lambda i, w, b: F.conv2d(
             i.reshape(i.shape[0], -1, i.shape[3], i.shape[4]), w.reshape(-1, *w.shape[2:]), b.reshape(-1), groups=i.shape[1]),
         "2fcrelu": lambda i, w1, b1, w2, b2: F.relu(F.linear(F.relu(F.linear(i, w1, b1)), w2, b2)),
+        "mlp1": lambda i, w1, b1: F.relu(i @ w1 + b1),
+        "mlp3": lambda i, w2, b2, w3, b3, w4, b4: F.relu(F.linear(F.relu(F.linear(F.relu(F.linear(i, w2, b2)), w3, b3)), w4, b4)),
         "lut": lambda t, i: t[i.long()].sum(1),
         "moments2": lambda x: (x.mean(1), x.var(1, unbiased=False)),
         "group_normalization_single_kernel": lambda i, g, b: F.group_norm(

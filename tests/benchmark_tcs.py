@@ -38,6 +38,30 @@ def func_2fcrelu(float(B, M) I, float(N, M) W1, float(N) B1, float(O, N) W2, flo
 }
 """
 
+# tc/benchmarks/MLP_model.cc:479-483 and :548-559
+MLP1 = """
+def mlp1(float(B, M) I, float(M, N) W1, float(N) B1) -> (O1) {
+    O1(b, n) +=! I(b, r_m) * W1(r_m, n)
+    O1(b, n) = O1(b, n) + B1(n)
+    O1(b, n) = fmax(O1(b, n), 0)
+}
+"""
+
+MLP3 = """
+def mlp3(float(B, N) I, float(O, N) W2, float(O) B2, float(P, O) W3, float(P) B3, float(Q, P) W4, float(Q) B4)
+-> (O2, O3, O4) {
+    O2(b, o) +=! I(b, n) * W2(o, n)
+    O2(b, o) = O2(b, o) + B2(o)
+    O2(b, o) = fmax(O2(b, o), 0)
+    O3(b, p) +=! O2(b, o) * W3(p, o)
+    O3(b, p) = O3(b, p) + B3(p)
+    O3(b, p) = fmax(O3(b, p), 0)
+    O4(b, q) +=! O3(b, p) * W4(q, p)
+    O4(b, q) = O4(b, q) + B4(q)
+    O4(b, q) = fmax(O4(b, q), 0)
+}
+"""
+
 LUT = """
 def lut(float(E, D) LUT, int32(B, L) I) -> (O) {
     O(i, j) +=! LUT(I(i, k), j)
@@ -157,6 +181,8 @@ CASES = {
     "matmul": (MATMUL, "matmul", [(72, 60), (60, 50)], 60),
     "convolution": (CONVOLUTION, "convolution", [(3, 4, 12, 11), (8, 4, 3, 3), (8,)], 36),
     "2fcrelu": (FCRELU2, "func_2fcrelu", [(20, 48), (36, 48), (36,), (24, 36), (24,)], 48),
+    "mlp1": (MLP1, "mlp1", [(20, 48), (48, 36), (36,)], 48),
+    "mlp3": (MLP3, "mlp3", [(20, 24), (18, 24), (18,), (10, 18), (10,), (2, 10), (2,)], 24),
     "lut": (LUT, "lut", [(50, 24), ("int", (9, 7), 0, 50)], 7),
     "2lut": (LUT2, "func_2lut", [(50, 24), ("int", (9, 7), 0, 50), (30, 24), ("int", (9, 5), 0, 30)], 7),
     "batchnorm": (BATCHNORM, "spatialBatchNorm",
@@ -173,8 +199,8 @@ CASES = {
 
 
 # The same comprehensions at the default sizes of the reference's benchmark programs
-# (tc/benchmarks/tmm.cc:42-44, MLP_model.cc:43-59 for the 1000x1024 matmul, the fc-relu chain and
-# the look-up table, convolution.cc:40-46, group_convolution.cc:42-49, moments.cc:42-43, group_normalization.cc:42-46,
+# (tc/benchmarks/tmm.cc:42-44, MLP_model.cc:43-59 for the 1000x1024 matmul, the fc-relu chain, the one- and
+# three-layer perceptrons and the look-up table, convolution.cc:40-46, group_convolution.cc:42-49, moments.cc:42-43, group_normalization.cc:42-46,
 # kronecker.cc:41-47, wavenet.cc:42-60), and the mapping options the autotuner found for them on an
 # MI355X (a few generations from the naive options; written relative to the naive options).
 REFERENCE_SIZES = {
@@ -183,6 +209,8 @@ REFERENCE_SIZES = {
     "matmul": [(128, 1000), (1000, 1024)],
     "convolution": [(32, 4, 56, 56), (4, 4, 3, 3), (4,)],
     "2fcrelu": [(128, 2000), (128, 2000), (128,), (64, 128), (64,)],
+    "mlp1": [(128, 2000), (2000, 128), (128,)],
+    "mlp3": [(128, 128), (64, 128), (64,), (32, 64), (32,), (2, 32), (2,)],
     "lut": [(100000, 64), ("int", (128, 50), 0, 100000)],
     "moments2": [(1024, 36864)],
     "group_normalization_single_kernel": [(32, 32, 16, 48, 48), (32, 16), (32, 16)],
@@ -206,6 +234,10 @@ TUNED_AT_REFERENCE_SIZES = {
     # one 16x16 tile per block, the 500 reduction steps of the first layer split over 16 wavefronts
     "2fcrelu": "naive;tile=16,16,128;unroll=256;mapToThreads=512,2;mapToBlocks=512,256;useMfma=1;useReadOnlyCache=1;"
                "useSharedMemory=1",
+    "mlp1": "naive;tile=16,16,128;unroll=256;mapToThreads=64,4;mapToBlocks=512,256;useMfma=1;useReadOnlyCache=1",
+    # the three layers in one kernel, 16 batch rows per block, each layer's result handed on in LDS
+    "mlp3": "naive;outerScheduleFusionStrategy=Max;intraTileScheduleFusionStrategy=Max;tile=16,256;unroll=16;mapToThreads=256;"
+            "mapToBlocks=256,128;useSharedMemory=1;unrollCopyShared=1;sharedDepth=4;useMfma=1;prefetchShared=1",
     "lut": "naive;outerScheduleFusionStrategy=Min;tile=4,32,32;unroll=64;usePrivateMemory=1;unrollCopyShared=1;"
            "collapseContiguous=0",
     "moments2": "naive;outerScheduleFusionStrategy=Max;fixParametersBeforeScheduling=1;tile=1;unroll=128;"

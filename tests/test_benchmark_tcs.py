@@ -46,6 +46,15 @@ def test_oracle_matches_library_routines():
     got = tc_oracle.run(B.FCRELU2, "func_2fcrelu", [I, W1, B1, W2, B2])
     close(got[0], o1, 48)
     close(got[1], o2, 48 * 36)
+    I, W1, B1 = B.make_inputs("mlp1")
+    close(tc_oracle.run(B.MLP1, "mlp1", [I, W1, B1])[0], torch.relu(f64(I) @ f64(W1) + f64(B1)), 48)
+    ins = B.make_inputs("mlp3")
+    I, W2, B2, W3, B3, W4, B4 = [f64(a) for a in ins]
+    o2 = torch.relu(I @ W2.T + B2)
+    o3 = torch.relu(o2 @ W3.T + B3)
+    o4 = torch.relu(o3 @ W4.T + B4)
+    for got, want, k in zip(tc_oracle.run(B.MLP3, "mlp3", ins), (o2, o3, o4), (24, 24 * 18, 24 * 18 * 10)):
+        close(got, want, k)
     lut, idx = B.make_inputs("lut")
     close(tc_oracle.run(B.LUT, "lut", [lut, idx])[0], f64(lut)[torch.from_numpy(idx).long()].sum(1), 7)
     X, = B.make_inputs("moments2")

@@ -22,7 +22,7 @@ def chain(*lengths):
     return float(sum(np.sqrt(k) for k in lengths)) ** 2
 
 
-CHAINED = {"2fcrelu": chain(48, 36), "kronecker3": chain(5, 4, 3), "batchnorm": 140, "wavenet1": chain(16, 8, 8),
+CHAINED = {"2fcrelu": chain(48, 36), "mlp3": chain(24, 18, 10), "kronecker3": chain(5, 4, 3), "batchnorm": 140, "wavenet1": chain(16, 8, 8),
            "group_normalization_single_kernel": 210}
 
 
@@ -62,7 +62,7 @@ def test_parity_at_the_reference_sizes_with_the_tuned_options(name):
     tc.run(ex, ins, outs)
     torch.cuda.synchronize()
     # reduction lengths at these sizes (chains: see chain())
-    k = {"tmm": 256, "matmul": 1000, "convolution": 36, "group_convolution": 36, "2fcrelu": chain(2000, 128), "lut": 50,
+    k = {"tmm": 256, "matmul": 1000, "convolution": 36, "group_convolution": 36, "2fcrelu": chain(2000, 128), "mlp1": 2000, "mlp3": chain(128, 64, 32), "lut": 50,
          "moments2": 36864, "group_normalization_single_kernel": 36864, "kronecker3": chain(16, 16, 16),
          "wavenet1": chain(64, 32, 32)}[name]
     for o, r in zip(outs, ref):
@@ -87,7 +87,7 @@ def test_lookup_indices_are_exact():
 
 
 @pytest.mark.parametrize("options", sorted(OPTION_SETS))
-@pytest.mark.parametrize("name", ["2fcrelu", "kronecker3", "matmul", "tmm_odd", "convolution"])
+@pytest.mark.parametrize("name", ["2fcrelu", "mlp1", "mlp3", "kronecker3", "matmul", "tmm_odd", "convolution"])
 def test_chains_and_contractions_are_exact_on_small_integers(name, options):
     """Inputs in {-2..2}: every product, partial sum and intermediate result is an integer far
     below 2^24, so any order of summation gives the same bits and a dropped or doubled partial
