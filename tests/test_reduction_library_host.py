@@ -6,7 +6,7 @@ import pytest
 
 import tensorcomprehensions_amd as tc
 
-TYPES = ["int8", "int16", "int32", "int64", "uint8", "uint16", "uint32", "uint64", "float", "double"]
+TYPES = ["int8", "int16", "int32", "int64", "uint8", "uint16", "uint32", "uint64", "float16", "float", "double"]
 # 32: lane groups inside one wavefront; 48: rows through LDS; 128: wavefront reduce + LDS partials
 WIDTHS = [32, 48, 128]
 
@@ -29,7 +29,7 @@ def test_block_reduction_compiles_for_every_type_operator_and_width(dtype, width
     ex = tc.compile(ALL_OPS.format(T=dtype), "red", ins, options)      # raises on a hipRTC error
     src = ex.compiled_source
     c_type = {"int8": "signed char", "uint8": "unsigned char", "int16": "short", "uint16": "unsigned short", "int32": "int",
-              "uint32": "unsigned int", "int64": "long long", "uint64": "unsigned long long"}.get(dtype, dtype)
+              "uint32": "unsigned int", "int64": "long long", "uint64": "unsigned long long", "float16": "_Float16"}.get(dtype, dtype)
     for op in ("OpSum", "OpProd", "OpMin", "OpMax"):
         assert f"__tc::blockAllReduceX<__tc::{op}<{c_type}>, {width}, 1, 1>" in src, (op, c_type)
     assert ex.num_kernels == 4
