@@ -63,7 +63,8 @@ TuningConfiguration::TuningConfiguration()
       vectorWidth({1, 2, 4}, "vector width"),
       collapseContiguous(RangeParameter::boolean("collapse contiguous")),
       useMfma(RangeParameter::boolean("use mfma")),
-      prefetchShared(RangeParameter::boolean("prefetch shared")) {
+      prefetchShared(RangeParameter::boolean("prefetch shared")),
+      reductionBlocks({1, 2, 4, 8, 16, 32, 64}, "reduction blocks") {
   tilingParams.setRange(1, 1, "t", {0}, "t");
   blockParams.setRange(1, 3, "b", {1}, "b");
   gridParams.setRange(1, 3, "g", {1}, "g");
@@ -90,7 +91,7 @@ std::vector<RangeParameter*> TuningConfiguration::collectParameters() {
   multi(gridParams);
   for (auto* x : {&unrollFactor, &tileImperfectlyNested, &useSharedMemory, &usePrivateMemory, &unrollCopyShared,
                   &useReadOnlyCache, &matchLibraryCalls, &privateDepth, &sharedDepth, &vectorWidth,
-                  &collapseContiguous, &useMfma, &prefetchShared}) {
+                  &collapseContiguous, &useMfma, &prefetchShared, &reductionBlocks}) {
     p.push_back(x);
   }
   return p;
@@ -128,6 +129,11 @@ void TuningConfiguration::fromHipMappingOptions(const HipMappingOptions& o) {
   collapseContiguous.selectFromValue(o.collapseContiguousValue);
   useMfma.selectFromValue(o.useMfmaValue);
   prefetchShared.selectFromValue(o.prefetchSharedValue);
+  size_t blocks = 1; // the largest searched value not above the given one
+  for (size_t v : reductionBlocks.values()) {
+    if (v <= o.reductionBlocksValue) blocks = std::max(blocks, v);
+  }
+  reductionBlocks.selectFromValue(blocks);
 }
 
 void TuningConfiguration::applyToHipMappingOptions(HipMappingOptions& o) const {
@@ -151,6 +157,7 @@ void TuningConfiguration::applyToHipMappingOptions(HipMappingOptions& o) const {
   o.collapseContiguous(collapseContiguous.value());
   o.useMfma(useMfma.value());
   o.prefetchShared(prefetchShared.value());
+  o.reductionBlocks(static_cast<uint32_t>(reductionBlocks.value()));
 }
 
 void TuningConfiguration::fixParameters(const TuningParameterFixer& f) {

@@ -84,7 +84,7 @@ class TuningConfiguration {
   RangeParameter tileImperfectlyNested;
   RangeParameter useSharedMemory, usePrivateMemory, unrollCopyShared, useReadOnlyCache, matchLibraryCalls;
   RangeParameter privateDepth, sharedDepth;
-  RangeParameter vectorWidth, collapseContiguous, useMfma, prefetchShared;
+  RangeParameter vectorWidth, collapseContiguous, useMfma, prefetchShared, reductionBlocks;
 
  private:
   std::vector<std::function<bool(const TuningConfiguration&)>> validators_;

@@ -45,6 +45,10 @@ template <typename T> __device__ __forceinline__ void storeThrough(__amdgpu_buff
     __builtin_amdgcn_raw_buffer_store_b8(__builtin_bit_cast(unsigned char, v), rs, index, 0, 16);
   }
 }
+// Partial sum of one block into an element other blocks add to as well (device scope, no order).
+template <typename T> __device__ __forceinline__ void atomicAccumulate(T* p, T v) {
+  __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 template <typename T> __device__ __forceinline__ T tmin(T a, T b) { return a < b ? a : b; }
 template <typename T> __device__ __forceinline__ T tmax(T a, T b) { return a > b ? a : b; }
 __device__ __forceinline__ float tmin(float a, float b) { return fminf(a, b); }

@@ -36,6 +36,7 @@ std::string HipMappingOptions::toText() const {
   if (hasSharedDepth) ss << ";sharedDepth=" << sharedDepthValue;
   ss << ";vectorWidth=" << vectorWidthValue << ";collapseContiguous=" << collapseContiguousValue
      << ";useMfma=" << useMfmaValue << ";prefetchShared=" << prefetchSharedValue;
+  if (reductionBlocksValue != 1) ss << ";reductionBlocks=" << reductionBlocksValue;
   return ss.str();
 }
 
@@ -87,6 +88,7 @@ HipMappingOptions HipMappingOptions::fromText(const std::string& text) {
     else if (k == "collapseContiguous") o.collapseContiguous(b());
     else if (k == "useMfma") o.useMfma(b());
     else if (k == "prefetchShared") o.prefetchShared(b());
+    else if (k == "reductionBlocks") o.reductionBlocks(static_cast<uint32_t>(std::stoul(v)));
     else TC_CHECK(false) << "unknown mapping option '" << k << "'";
   }
   return o;
@@ -129,6 +131,7 @@ std::ostream& operator<<(std::ostream& os, const HipMappingOptionsAsCpp& p) {
      << in << ".collapseContiguous(" << bs(o.collapseContiguousValue) << ")\n"
      << in << ".useMfma(" << bs(o.useMfmaValue) << ")\n"
      << in << ".prefetchShared(" << bs(o.prefetchSharedValue) << ")";
+  if (o.reductionBlocksValue != 1) os << "\n" << in << ".reductionBlocks(" << o.reductionBlocksValue << ")";
   return os;
 }
 

@@ -9,7 +9,9 @@
 //     contiguous dimension), collapseContiguous (merge loop dimensions that are jointly contiguous
 //     in every tensor before mapping), useMfma (matrix-core tiles for dense contractions),
 //     prefetchShared (software-pipelined LDS staging: the next block tile's global loads are
-//     in flight while the current one is computed).
+//     in flight while the current one is computed), reductionBlocks (a sum whose outermost
+//     reduction index is divided among that many blocks, which add their partial results into
+//     the output with atomics; 1 = the reference's behaviour, a reduction stays inside a block).
 #pragma once
 #include <algorithm>
 #include <array>
@@ -83,6 +85,7 @@ class HipMappingOptions : public GenericOptionsFluent<HipMappingOptions> {
   bool collapseContiguousValue = true;
   bool useMfmaValue = false;
   bool prefetchSharedValue = false;
+  uint32_t reductionBlocksValue = 1;
 
   HipMappingOptions() = default;
   // from a serialized HipMappingOptionsProto
@@ -96,7 +99,7 @@ class HipMappingOptions : public GenericOptionsFluent<HipMappingOptions> {
         useReadOnlyCacheValue == o.useReadOnlyCacheValue && privateDepthValue == o.privateDepthValue &&
         sharedDepthValue == o.sharedDepthValue && vectorWidthValue == o.vectorWidthValue &&
         collapseContiguousValue == o.collapseContiguousValue && useMfmaValue == o.useMfmaValue &&
-        prefetchSharedValue == o.prefetchSharedValue;
+        prefetchSharedValue == o.prefetchSharedValue && reductionBlocksValue == o.reductionBlocksValue;
   }
   bool operator!=(const HipMappingOptions& o) const { return !(*this == o); }
 
@@ -145,6 +148,11 @@ class HipMappingOptions : public GenericOptionsFluent<HipMappingOptions> {
   HipMappingOptions& collapseContiguous(bool b) { collapseContiguousValue = b; return *this; }
   HipMappingOptions& useMfma(bool b) { useMfmaValue = b; return *this; }
   HipMappingOptions& prefetchShared(bool b) { prefetchSharedValue = b; return *this; }
+  HipMappingOptions& reductionBlocks(uint32_t n) {
+    TC_CHECK(n >= 1 && n <= 1024) << "reductionBlocks must be between 1 and 1024, got " << n;
+    reductionBlocksValue = n;
+    return *this;
+  }
 
   std::string toProtobufSerializedString() const {
     protowire::Writer w;
@@ -162,6 +170,7 @@ class HipMappingOptions : public GenericOptionsFluent<HipMappingOptions> {
     w.boolean(12, collapseContiguousValue);
     w.boolean(13, useMfmaValue);
     w.boolean(14, prefetchSharedValue);
+    if (reductionBlocksValue != 1) w.varint(15, reductionBlocksValue);
     return w.str();
   }
   void fromProto(const std::string& s) {
@@ -182,6 +191,7 @@ class HipMappingOptions : public GenericOptionsFluent<HipMappingOptions> {
         case 12: collapseContiguousValue = r.value() != 0; break;
         case 13: useMfmaValue = r.value() != 0; break;
         case 14: prefetchSharedValue = r.value() != 0; break;
+        case 15: reductionBlocksValue = static_cast<uint32_t>(r.value()); break;
         default: break;
       }
     }

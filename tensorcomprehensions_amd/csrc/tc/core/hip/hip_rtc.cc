@@ -55,7 +55,10 @@ std::unique_ptr<HipRTCFunction> HipRTCFunction::Compile(const std::string& name,
   res->name_ = name;
   std::string arch = HipGPUInfo::GPUInfo().GetArch();
   // Packed-FP32 instruction selection is switched off for all device code of this library.
-  std::vector<const char*> opts = {"-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+  // (-munsafe-fp-atomics: floating-point atomic adds become the hardware instruction; tensors live
+  // in ordinary device memory, for which it is exact)
+  std::vector<const char*> opts = {"-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                                   "-munsafe-fp-atomics"};
   if (tc::flags().fast_math) opts.push_back("-ffast-math");
   char* code = nullptr;
   char* log = nullptr;

@@ -87,6 +87,11 @@ struct Statement {
   ExprRef rhs;
   ScalarType type;
   lang::TreeRef tree;                   // for error reports
+  // Set by the mapper when it divides a sum among blocks: `sliceVar` (the first of lhsVars, not a
+  // subscript of the tensor) numbers the slices of the outermost reduction index, and the
+  // partial result of a slice is added into the tensor atomically.
+  bool atomic = false;
+  std::string sliceVar;
 };
 
 struct Tensor {

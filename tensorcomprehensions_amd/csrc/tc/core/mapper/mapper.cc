@@ -748,6 +748,68 @@ ir::Function withZeroBasedOutputs(const ir::Function& in) {
   }
   return f;
 }
+// reductionBlocks: a sum `O(p...) +=(!) rhs` is divided among blocks along its outermost reduction
+// index r (extent E, `split` = the largest divisor of E not above `blocks`):
+//     O(p...) = 0                                   only for "+=!", a kernel of its own
+//     O(p...) += rhs[r := r + (E / split) * slice]   slice in 0:split, r in 0:E/split
+// where `slice` becomes the outermost parallel variable of the second statement and its partial
+// sums are added into O atomically.  Floating-point sums then depend on the order in which the
+// blocks arrive (within the rounding of any other summation order); integer sums do not.
+ir::Function withSplitReductions(const ir::Function& in, int64_t blocks) {
+  ir::Function f = in;
+  f.statements.clear();
+  int counter = 0;
+  for (const auto& s : in.statements) {
+    const ir::Tensor* t = in.find(s.tensor);
+    bool ok = t && s.op == ReduceOp::Plus && !s.redVars.empty() && accessesTo(s, s.tensor).empty() &&
+        (t->type.bits == 32 || t->type.bits == 64);
+    int64_t split = 1, extent = 0;
+    if (ok) {
+      extent = s.ranges.at(s.redVars[0]).extent();
+      for (int64_t d = std::min<int64_t>(blocks, extent); d >= 2; --d) {
+        if (extent % d == 0) {
+          split = d;
+          break;
+        }
+      }
+    }
+    if (split < 2) {
+      f.statements.push_back(s);
+      continue;
+    }
+    if (s.init) {
+      ir::Statement zero;
+      zero.tensor = s.tensor;
+      zero.lhsVars = s.lhsVars;
+      for (const auto& v : s.lhsVars) zero.ranges[v] = s.ranges.at(v);
+      zero.type = t->type;
+      zero.tree = s.tree;
+      auto z = std::make_shared<Expr>();
+      z->kind = t->type.isFloat() ? Expr::FloatImm : Expr::IntImm;
+      z->type = t->type;
+      zero.rhs = z;
+      f.statements.push_back(zero);
+    }
+    ir::Statement part = s;
+    part.init = false;
+    part.atomic = true;
+    do {
+      part.sliceVar = "slice" + std::to_string(counter++);
+    } while (part.ranges.count(part.sliceVar));
+    part.lhsVars.insert(part.lhsVars.begin(), part.sliceVar);
+    part.ranges[part.sliceVar] = ir::Range{0, split - 1};
+    const std::string r = s.redVars[0];
+    const int64_t chunk = extent / split;
+    ir::Range& rr = part.ranges.at(r);
+    rr.max = rr.min + chunk - 1;
+    part.rhs = rewrite(s.rhs, [&](const ExprRef& e) -> ExprRef {
+      if (e->kind != Expr::Var || e->name != r) return nullptr;
+      return mkBin("+", e, mkBin("*", mkVar(part.sliceVar), mkInt(chunk)));
+    });
+    f.statements.push_back(part);
+  }
+  return f;
+}
 } // namespace
 
 MappedProgram mapToHip(
@@ -760,7 +822,10 @@ MappedProgram mapToHip(
     for (auto m : t.mins) shifted |= m != 0;
   }
   const ir::Function zeroBased = shifted ? withZeroBasedOutputs(given) : ir::Function();
-  const ir::Function& f = shifted ? zeroBased : given;
+  const bool divided = options.reductionBlocksValue > 1;
+  const ir::Function dividedSums =
+      divided ? withSplitReductions(shifted ? zeroBased : given, options.reductionBlocksValue) : ir::Function();
+  const ir::Function& f = divided ? dividedSums : shifted ? zeroBased : given;
   // 1. stages
   std::vector<RawStage> raw;
   bool allowStageFusion = options.generic.intraTileScheduleOptions.fusionStrategy != FusionStrategy::Min ||

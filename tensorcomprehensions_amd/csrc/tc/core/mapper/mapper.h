@@ -94,6 +94,9 @@ struct StagePlan {
   std::vector<std::string> mfmaM, mfmaN, mfmaBatch, mfmaK;
   bool mfmaSwapOperands = false;     // the first factor of the product is the N-side operand
   int64_t waves = 1;
+  // The stage adds partial sums into its tensor with atomics: its first parallel variable numbers
+  // slices of the reduction and is no subscript of the tensor.
+  bool atomic = false;
 };
 
 struct KernelPlan {

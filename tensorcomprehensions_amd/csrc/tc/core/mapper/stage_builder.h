@@ -64,6 +64,9 @@ std::set<std::string> tensorsRead(const ir::Statement& s) {
 // first d left-hand-side positions of both, or -1 when they cannot share a kernel.
 int sharedPrefix(const RawStage& A, const RawStage& B) {
   const ir::Statement &a0 = A.first(), &b0 = B.first();
+  // partial sums of all blocks must be complete before anything reads them, and the zeroing must
+  // be complete before the first of them arrives: a kernel of its own
+  if (a0.atomic || b0.atomic) return -1;
   size_t d = std::min(a0.lhsVars.size(), b0.lhsVars.size());
   for (size_t p = 0; p < d; ++p) {
     const ir::Range &ra = a0.ranges.at(a0.lhsVars[p]), &rb = b0.ranges.at(b0.lhsVars[p]);
@@ -116,8 +119,9 @@ struct StageBuilder {
   void init(const RawStage& raw) {
     const ir::Statement& s0 = raw.first();
     st.tensor = s0.tensor;
+    st.atomic = s0.atomic;
     for (const auto& v : s0.lhsVars) {
-      st.lhsSubs.push_back(mkVar(v));
+      if (!(s0.atomic && v == s0.sliceVar)) st.lhsSubs.push_back(mkVar(v));
       LoopVar lv;
       lv.name = v;
       lv.min = s0.ranges.at(v).min;
@@ -129,7 +133,8 @@ struct StageBuilder {
     for (const auto* s : raw.stmts) {
       StageStmt ss;
       ss.op = s->op;
-      ss.init = s->init;
+      ss.init = s->init || s->atomic; // a partial sum starts from zero, the tensor is never read
+
       ss.type = s->type;
       ExprRef rhs = s->rhs;
       // reduction variables get stage-unique names (two statements may both use "k")
@@ -345,7 +350,7 @@ struct StageBuilder {
 bool classifyContraction(StagePlan& st) {
   if (st.stmts.empty()) return false;
   const StageStmt& s = st.stmts[0];
-  if (s.redVars.empty() || s.op != ReduceOp::Plus) return false;
+  if (s.redVars.empty() || s.op != ReduceOp::Plus || st.atomic) return false;
   for (size_t i = 1; i < st.stmts.size(); ++i) {
     if (!st.stmts[i].redVars.empty()) return false;
   }

@@ -278,6 +278,7 @@ class StageCodegen {
   // write-back time to the kernel (12.8 MB: 2.4 us) instead of overlapping it with the computation.
   // Byte offsets of a buffer access are 32 bits wide, which bounds the tensors this applies to.
   bool streamedStore() const {
+    if (st_.atomic) return false;
     if (!kc_.opts.useReadOnlyCacheValue || viewBytes(st_.tensor) >= (int64_t(1) << 31)) return false;
     if (forwardOf(st_.tensor)) return true; // the later stages read the copy in LDS
     for (size_t j = stageIdx_ + 1; j < kc_.k.stages.size(); ++j) {
@@ -289,6 +290,7 @@ class StageCodegen {
 
   std::string storeStmt(const std::string& cond, const std::string& value) {
     std::string index = flatIndex(st_.tensor, st_.lhsSubs, "");
+    if (st_.atomic) return "if (" + cond + ") __tc::atomicAccumulate(&p" + st_.tensor + "[" + index + "], " + value + ");";
     std::string store = streamedStore()
         ? "__tc::storeThrough(" + bufferName(st_.tensor) + ", " + index + ", " + value + ");"
         : "p" + st_.tensor + "[" + index + "] = " + value + ";";

@@ -76,6 +76,7 @@ class MappingOptions:
     def collapseContiguous(self, b): return self._set("collapseContiguous", _b(b))
     def useMfma(self, b): return self._set("useMfma", _b(b))
     def prefetchShared(self, b): return self._set("prefetchShared", _b(b))
+    def reductionBlocks(self, n): return self._set("reductionBlocks", int(n))
 
     def to_text(self):
         return ";".join(self._parts)

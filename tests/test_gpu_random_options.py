@@ -43,6 +43,8 @@ def random_options(rng, band):
     parts.append(f"vectorWidth={rng.choice([1, 1, 2, 4])}")
     parts.append(f"outerScheduleFusionStrategy={rng.choice(['Max', 'Preserve3Coincident', 'Min'])}")
     parts.append(f"intraTileScheduleFusionStrategy={rng.choice(['Max', 'Preserve3Coincident', 'Min'])}")
+    if rng.random() < 0.25:
+        parts.append(f"reductionBlocks={rng.choice([2, 3, 4, 8, 16])}")
     return ";".join(parts)
 
 

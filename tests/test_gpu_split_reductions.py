@@ -1,0 +1,77 @@
+"""reductionBlocks: a sum whose outermost reduction index is divided among blocks that add their
+partial results into the output with atomics (the reference keeps a reduction inside one block,
+mapped_scop.cc:253-383).  Integer sums are exact in any order; floating-point sums are held to the
+tolerance every other summation order is held to."""
+import numpy as np
+import pytest
+import torch
+
+import tensorcomprehensions_amd as tc
+from oracle import tc_oracle
+from tests import workloads as W
+
+pytestmark = pytest.mark.gpu
+
+BIAS_GRAD = "def bias_grad(float(N, M, H, W) d_O) -> (d_B) { d_B(m) +=! d_O(r_n, m, r_h, r_w) }"
+STATS = """def stats(float(N, C, H, W) I) -> (sum, mean, centered) {
+    sum(c) +=! I(r_n, c, r_h, r_w)
+    mean(c) = sum(c) / (N * H * W)
+    centered(n, c, h, w) = I(n, c, h, w) - mean(c)
+}"""
+OPTION_SETS = [
+    "naive;tile=1,1;mapToThreads=256;mapToBlocks=64,64;matchLibraryCalls=1;reductionBlocks=16",
+    "naive;tile=1,4;mapToThreads=64,4;mapToBlocks=8,4;matchLibraryCalls=1;reductionBlocks=8;unroll=4",
+    "naive;tile=2,8;mapToThreads=8,16;mapToBlocks=256,256;matchLibraryCalls=0;reductionBlocks=64;vectorWidth=2",
+    "naive;tile=1,32;mapToThreads=32;mapToBlocks=3;reductionBlocks=5;outerScheduleFusionStrategy=Max",
+]
+
+
+def run(src, entry, ins_np, options, outs_init=None):
+    ins = [torch.from_numpy(a).cuda() for a in ins_np]
+    ex = tc.compile(src, entry, ins, options)
+    outs = tc.prepare_outputs(src, entry, ins)
+    for i, o in enumerate(outs):
+        if outs_init is not None:
+            o.copy_(torch.from_numpy(outs_init[i]))
+        else:
+            o.fill_(float("nan") if o.dtype.is_floating_point else -77)
+    tc.run(ex, ins, outs)
+    torch.cuda.synchronize()
+    return [o.cpu().numpy() for o in outs], ex
+
+
+@pytest.mark.parametrize("options", OPTION_SETS)
+def test_bias_gradient_split_over_blocks(options):
+    d_O = np.random.Generator(np.random.Philox(61)).integers(-3, 4, size=(20, 24, 9, 7)).astype(np.float32)
+    (got,), ex = run(BIAS_GRAD, "bias_grad", [d_O], options)
+    assert "__tc::atomicAccumulate(&pd_B[" in ex.compiled_source and ex.num_kernels == 2
+    (ref,) = tc_oracle.run(BIAS_GRAD, "bias_grad", [d_O])
+    assert np.array_equal(ref, d_O.sum((0, 2, 3)))
+    assert np.array_equal(got, ref)                        # small integers: exact in any order
+    # run it again on the same outputs: the zeroing kernel precedes the partial sums every time
+    ins = [torch.from_numpy(d_O).cuda()]
+    outs = [torch.from_numpy(got.copy()).cuda()]
+    tc.run(ex, ins, outs)
+    torch.cuda.synchronize()
+    assert np.array_equal(outs[0].cpu().numpy(), ref)
+
+
+@pytest.mark.parametrize("options", OPTION_SETS)
+def test_readers_of_a_split_sum_wait_for_all_of_it(options):
+    I = np.random.Generator(np.random.Philox(62)).standard_normal((20, 6, 9, 7), dtype=np.float32)
+    got, ex = run(STATS, "stats", [I], options)
+    ref = tc_oracle.run(STATS, "stats", [I])
+    assert ex.num_kernels >= 3
+    for g, r in zip(got, ref):
+        assert np.abs(g - r).max() <= W.tolerance(20 * 9 * 7, r)
+
+
+@pytest.mark.parametrize("dtype,tc_type", [(np.int32, "int32"), (np.int64, "int64"), (np.uint32, "uint32"), (np.float64, "double")])
+def test_accumulating_into_existing_values_and_other_types(dtype, tc_type):
+    src = f"def acc({tc_type}(M, K) X) -> (s) {{ s(m) += X(m, r_k) * X(m, r_k) }}"
+    X = np.random.Generator(np.random.Philox(63)).integers(0, 9, size=(33, 600)).astype(dtype)
+    prior = np.arange(33).astype(dtype)
+    (got,), ex = run(src, "acc", [X], "naive;tile=1,1;mapToThreads=64;mapToBlocks=64,64;matchLibraryCalls=1;reductionBlocks=8",
+                     outs_init=[prior])
+    assert ex.num_kernels == 1 and "atomicAccumulate" in ex.compiled_source       # "+=": nothing to zero
+    assert np.array_equal(got, prior + (X.astype(np.int64) ** 2).sum(1).astype(dtype))

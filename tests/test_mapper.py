@@ -386,3 +386,25 @@ def test_written_tensor_is_forwarded_to_later_stages_through_lds():
     assert looped.count("__syncthreads();") == src.count("__syncthreads();") + 1
     plain, _ = mapped(chain, "chain", [(40, 48), (48, 70)], base + ";mapToBlocks=64;useSharedMemory=0")
     assert "fwd0_B" not in plain
+
+
+def test_reduction_blocks_divides_a_sum_among_blocks():
+    """reductionBlocks: `O +=! f` becomes a zeroing kernel and a kernel whose outermost parallel
+    variable numbers slices of the outermost reduction index; partial sums meet in atomics."""
+    src = "def bias_grad(float(N, M, H, W) d_O) -> (d_B) { d_B(m) +=! d_O(r_n, m, r_h, r_w) }"
+    opts = "naive;tile=1,1;mapToThreads=256;mapToBlocks=64,64;matchLibraryCalls=1"
+    plain, launches = mapped(src, "bias_grad", [(32, 64, 56, 56)], opts)
+    assert launches == [((64, 1, 1), (256, 1, 1))] and "atomicAccumulate(&p" not in plain
+    split, launches = mapped(src, "bias_grad", [(32, 64, 56, 56)], opts + ";reductionBlocks=16")
+    assert [g for g, _ in launches] == [(64, 1, 1), (16, 64, 1)]              # zeroing, then 16 slices x 64 outputs
+    assert "__tc::atomicAccumulate(&pd_B[i_m], acc_[a_]);" in split
+    assert "401408 * i_slice0" in split                                       # slice = 2 of the 32 images
+    # an extent without a divisor in range, a narrow element type, a maximum: mapped as without the option
+    for text, shape, dtype, blocks in [("def f(float(M, K) X) -> (s) { s(m) +=! X(m, r_k) }", (8, 127), "float32", 64),
+                                       ("def f(int8(M, K) X) -> (s) { s(m) +=! X(m, r_k) }", (8, 128), "int8", 16),
+                                       ("def f(float(M, K) X) -> (s) { s(m) max=! X(m, r_k) }", (8, 128), "float32", 16)]:
+        s, _ = tc.map_only(text, "f", [ShapeOnly(shape, dtype)], f"naive;reductionBlocks={blocks}")
+        assert "atomicAccumulate(&p" not in s
+    # the option survives text and wire form
+    o = MappingOptions("naive;reductionBlocks=8")
+    assert "reductionBlocks=8" in o.normalized() and "reductionBlocks" not in MappingOptions("naive").normalized()
