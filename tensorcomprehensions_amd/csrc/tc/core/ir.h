@@ -89,8 +89,11 @@ struct Statement {
   lang::TreeRef tree;                   // for error reports
   // Set by the mapper when it divides a sum among blocks: `sliceVar` (the first of lhsVars, not a
   // subscript of the tensor) numbers the slices of the outermost reduction index, and the
-  // partial result of a slice is added into the tensor atomically.
+  // partial result of a slice is added into the tensor atomically.  `zeroing` marks the statement
+  // that clears the tensor beforehand: it is mapped as a plain fill, whatever the options say
+  // about tiles and blocks (their positions mean the variables of the sliced statement).
   bool atomic = false;
+  bool zeroing = false;
   std::string sliceVar;
 };
 

@@ -777,10 +777,15 @@ ir::Function withSplitReductions(const ir::Function& in, int64_t blocks) {
       f.statements.push_back(s);
       continue;
     }
+    std::string slice;
+    do {
+      slice = "slice" + std::to_string(counter++);
+    } while (s.ranges.count(slice));
     if (s.init) {
       ir::Statement zero;
       zero.tensor = s.tensor;
       zero.lhsVars = s.lhsVars;
+      zero.zeroing = true;
       for (const auto& v : s.lhsVars) zero.ranges[v] = s.ranges.at(v);
       zero.type = t->type;
       zero.tree = s.tree;
@@ -793,9 +798,7 @@ ir::Function withSplitReductions(const ir::Function& in, int64_t blocks) {
     ir::Statement part = s;
     part.init = false;
     part.atomic = true;
-    do {
-      part.sliceVar = "slice" + std::to_string(counter++);
-    } while (part.ranges.count(part.sliceVar));
+    part.sliceVar = slice;
     part.lhsVars.insert(part.lhsVars.begin(), part.sliceVar);
     part.ranges[part.sliceVar] = ir::Range{0, split - 1};
     const std::string r = s.redVars[0];
@@ -812,9 +815,19 @@ ir::Function withSplitReductions(const ir::Function& in, int64_t blocks) {
 }
 } // namespace
 
+namespace {
+HipMappingOptions given_options_for_fill(const HipMappingOptions& given) {
+  HipMappingOptions o = given;
+  o.tile(std::vector<uint64_t>{1024}).unroll(4).matchLibraryCalls(false);
+  o.mapToThreads(256).mapToBlocks(1 << 20).useSharedMemory(false).usePrivateMemory(false);
+  o.vectorWidth(4).collapseContiguous(true).useMfma(false).prefetchShared(false);
+  return o;
+}
+} // namespace
+
 MappedProgram mapToHip(
     const ir::Function& given,
-    const HipMappingOptions& options,
+    const HipMappingOptions& optionsIn,
     const std::string& specializedName,
     const DeviceLimits& limits) {
   bool shifted = false;
@@ -822,14 +835,14 @@ MappedProgram mapToHip(
     for (auto m : t.mins) shifted |= m != 0;
   }
   const ir::Function zeroBased = shifted ? withZeroBasedOutputs(given) : ir::Function();
-  const bool divided = options.reductionBlocksValue > 1;
+  const bool divided = optionsIn.reductionBlocksValue > 1;
   const ir::Function dividedSums =
-      divided ? withSplitReductions(shifted ? zeroBased : given, options.reductionBlocksValue) : ir::Function();
+      divided ? withSplitReductions(shifted ? zeroBased : given, optionsIn.reductionBlocksValue) : ir::Function();
   const ir::Function& f = divided ? dividedSums : shifted ? zeroBased : given;
   // 1. stages
   std::vector<RawStage> raw;
-  bool allowStageFusion = options.generic.intraTileScheduleOptions.fusionStrategy != FusionStrategy::Min ||
-      options.generic.outerScheduleOptions.fusionStrategy != FusionStrategy::Min;
+  bool allowStageFusion = optionsIn.generic.intraTileScheduleOptions.fusionStrategy != FusionStrategy::Min ||
+      optionsIn.generic.outerScheduleOptions.fusionStrategy != FusionStrategy::Min;
   for (const auto& s : f.statements) {
     for (const auto& subs : accessesTo(s, s.tensor)) {
       TC_CHECK(isIdentityAccess(subs, s.lhsVars))
@@ -852,7 +865,7 @@ MappedProgram mapToHip(
     int depth;
   };
   std::vector<Group> groups;
-  FusionStrategy fs = options.generic.outerScheduleOptions.fusionStrategy;
+  FusionStrategy fs = optionsIn.generic.outerScheduleOptions.fusionStrategy;
   for (size_t i = 0; i < raw.size(); ++i) {
     bool joined = false;
     if (!groups.empty() && fs != FusionStrategy::Min) {
@@ -896,9 +909,16 @@ MappedProgram mapToHip(
   }
   const bool wide = maxNumel >= (1LL << 31);
 
+  // The fill that precedes a divided sum: all dimensions merged, four elements per thread, 256
+  // threads, as many blocks as that takes.
+  HipMappingOptions fillOptions = given_options_for_fill(optionsIn);
+  std::vector<const HipMappingOptions*> kernelOptions;
   bool anyThreadReduction = false;
   std::vector<std::unique_ptr<Emitter>> bodies;
   for (size_t gi = 0; gi < groups.size(); ++gi) {
+    const bool fill = groups[gi].stages.size() == 1 && raw[groups[gi].stages[0]].first().zeroing;
+    const HipMappingOptions& options = fill ? fillOptions : optionsIn;
+    kernelOptions.push_back(&options);
     KernelPlan k;
     k.name = specializedName + (gi == 0 ? "" : "_k" + std::to_string(gi));
     bool single = groups[gi].stages.size() == 1;
@@ -960,8 +980,9 @@ MappedProgram mapToHip(
     prog.kernels.push_back(std::move(k));
   }
   std::ostringstream src;
-  for (auto& k : prog.kernels) {
-    KernelCtx kc{f, options, k};
+  for (size_t ki = 0; ki < prog.kernels.size(); ++ki) {
+    KernelPlan& k = prog.kernels[ki];
+    KernelCtx kc{f, *kernelOptions[ki], k};
     kc.wide = wide;
     if (wide) kc.idx = "int64";
     mapKernel(kc, limits);

@@ -121,7 +121,7 @@ struct StageBuilder {
     st.tensor = s0.tensor;
     st.atomic = s0.atomic;
     for (const auto& v : s0.lhsVars) {
-      if (!(s0.atomic && v == s0.sliceVar)) st.lhsSubs.push_back(mkVar(v));
+      if (s0.sliceVar.empty() || v != s0.sliceVar) st.lhsSubs.push_back(mkVar(v));
       LoopVar lv;
       lv.name = v;
       lv.min = s0.ranges.at(v).min;
@@ -350,7 +350,7 @@ struct StageBuilder {
 bool classifyContraction(StagePlan& st) {
   if (st.stmts.empty()) return false;
   const StageStmt& s = st.stmts[0];
-  if (s.redVars.empty() || s.op != ReduceOp::Plus || st.atomic) return false;
+  if (s.redVars.empty() || s.op != ReduceOp::Plus) return false;
   for (size_t i = 1; i < st.stmts.size(); ++i) {
     if (!st.stmts[i].redVars.empty()) return false;
   }

@@ -20,6 +20,7 @@ STATS = """def stats(float(N, C, H, W) I) -> (sum, mean, centered) {
 }"""
 OPTION_SETS = [
     "naive;tile=1,1;mapToThreads=256;mapToBlocks=64,64;matchLibraryCalls=1;reductionBlocks=16",
+    "naive;tile=1,16,16;mapToThreads=64,4;mapToBlocks=8,8,8;useMfma=1;reductionBlocks=4",
     "naive;tile=1,4;mapToThreads=64,4;mapToBlocks=8,4;matchLibraryCalls=1;reductionBlocks=8;unroll=4",
     "naive;tile=2,8;mapToThreads=8,16;mapToBlocks=256,256;matchLibraryCalls=0;reductionBlocks=64;vectorWidth=2",
     "naive;tile=1,32;mapToThreads=32;mapToBlocks=3;reductionBlocks=5;outerScheduleFusionStrategy=Max",
@@ -75,3 +76,15 @@ def test_accumulating_into_existing_values_and_other_types(dtype, tc_type):
                      outs_init=[prior])
     assert ex.num_kernels == 1 and "atomicAccumulate" in ex.compiled_source       # "+=": nothing to zero
     assert np.array_equal(got, prior + (X.astype(np.int64) ** 2).sum(1).astype(dtype))
+
+
+def test_matrix_product_divided_among_blocks_on_the_matrix_cores():
+    src = "def mm(float(M, K) A, float(K, N) B) -> (C) { C(m, n) +=! A(m, r_k) * B(r_k, n) }"
+    rng = np.random.Generator(np.random.Philox(64))
+    A = rng.integers(-3, 4, size=(40, 640)).astype(np.float32)
+    Bm = rng.integers(-3, 4, size=(640, 50)).astype(np.float32)
+    opts = "naive;tile=1,16,16;mapToThreads=64,4;mapToBlocks=8,8,8;useMfma=1;reductionBlocks=8"
+    (got,), ex = run(src, "mm", [A, Bm], opts)
+    s = ex.compiled_source
+    assert "__builtin_amdgcn_mfma_f32_16x16x4f32" in s and "__tc::atomicAccumulate(&pC[" in s and "ksplit0_" in s
+    assert np.array_equal(got, A @ Bm)

@@ -396,7 +396,7 @@ def test_reduction_blocks_divides_a_sum_among_blocks():
     plain, launches = mapped(src, "bias_grad", [(32, 64, 56, 56)], opts)
     assert launches == [((64, 1, 1), (256, 1, 1))] and "atomicAccumulate(&p" not in plain
     split, launches = mapped(src, "bias_grad", [(32, 64, 56, 56)], opts + ";reductionBlocks=16")
-    assert [g for g, _ in launches] == [(64, 1, 1), (16, 64, 1)]              # zeroing, then 16 slices x 64 outputs
+    assert launches == [((1, 1, 1), (16, 1, 1)), ((16, 64, 1), (256, 1, 1))]  # a fill of 64 floats, then 16 slices x 64 outputs
     assert "__tc::atomicAccumulate(&pd_B[i_m], acc_[a_]);" in split
     assert "401408 * i_slice0" in split                                       # slice = 2 of the 32 images
     # an extent without a divisor in range, a narrow element type, a maximum: mapped as without the option
