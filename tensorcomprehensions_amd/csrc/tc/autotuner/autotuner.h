@@ -7,6 +7,7 @@
 // OptionsCache and on the candidate; the search strategy then breeds the next generation.
 // SIGINT finishes the current generation and returns the best so far; SIGTERM aborts.
 #pragma once
+#include <limits>
 #include <atomic>
 #include <chrono>
 #include <condition_variable>
@@ -123,7 +124,7 @@ inline std::vector<size_t> mergedDimensionThreadCounts(const std::vector<const D
 // a member of the search space (0, powers of two up to 256, merged-dimension thread counts).
 inline std::vector<HipMappingOptions> heuristicSeeds(
     const HipMappingOptions& base, const std::vector<const DLConstTensor*>& inputs, size_t smallestOutputRank,
-    size_t innermostOutputExtent = 0) {
+    size_t innermostOutputExtent = 0, bool fewOutputs = false) {
   std::vector<HipMappingOptions> seeds;
   size_t maxRank = 0;
   uint64_t largest = 256; // largest extent: a grid limit that never forces a block to loop over tiles
@@ -167,6 +168,23 @@ inline std::vector<HipMappingOptions> heuristicSeeds(
       seeds.push_back(o);
     }
   }
+  // few outputs, long sums: the rows as above, the outermost reduction index divided among blocks
+  // (the slice number is the first variable of the divided statement)
+  if (fewOutputs) {
+    for (uint32_t slices : {16u, 64u}) {
+      HipMappingOptions o = base;
+      std::vector<uint64_t> rows(1 + std::max<size_t>(1, smallestOutputRank), 1);
+      rows.push_back(0);
+      o.generic.tile(rows);
+      o.generic.unroll(8);
+      o.generic.matchLibraryCallsValue = true;
+      o.mapToThreads(256).mapToBlocks(largest, largest, 256).useReadOnlyCache(true);
+      o.vectorWidthValue = 4;
+      o.collapseContiguousValue = true;
+      o.reductionBlocksValue = slices;
+      seeds.push_back(o);
+    }
+  }
   // windows (convolutions with few channels): one image per block with its input window in LDS,
   // the innermost output dimension along threadIdx.x and as many rows as fit along threadIdx.y
   if (innermostOutputExtent >= 8 && innermostOutputExtent <= 256 && smallestOutputRank >= 3) {
@@ -205,7 +223,7 @@ inline TuningConfiguration setupTuningParameters(
   std::vector<size_t> blockRange = range, gridRange = range;
   // Deviation: thread counts that cover merged trailing dimensions exactly.
   blockRange = mergeVectors(std::move(blockRange), mergedDimensionThreadCounts(inputs));
-  size_t tileDims = maxRank + 1;
+  size_t tileDims = maxRank + 2; // (+1 as in the reference, +1 for the slice number of a divided sum)
   for (const auto& b : baseMappings) {
     blockRange = mergeVectors(std::move(blockRange), std::vector<size_t>(b.block.extractVector().begin(), b.block.extractVector().end()));
     gridRange = mergeVectors(std::move(gridRange), std::vector<size_t>(b.grid.extractVector().begin(), b.grid.extractVector().end()));
@@ -299,6 +317,19 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
     space.tileImperfectlyNested.fixValue(b0.generic.tileImperfectlyNestedValue);
     space.privateDepth.fixValue(b0.privateDepthValue);
   }
+  // Dividing a sum among blocks can only pay where the outputs are too few to fill the device by
+  // themselves; elsewhere the gene keeps the base value instead of thinning the search.
+  bool fewOutputs = false;
+  {
+    int64_t fewest = std::numeric_limits<int64_t>::max();
+    for (const auto& o : outputsInfo) {
+      int64_t n = 1;
+      for (auto e : o.shape) n *= e;
+      fewest = std::min(fewest, n);
+    }
+    fewOutputs = fewest < (int64_t(1) << 16);
+    if (!fewOutputs) space.reductionBlocks.fixValue(bases.front().reductionBlocksValue);
+  }
   std::vector<TuningConfiguration> configs;
   for (const auto& b : bases) {
     TuningConfiguration c = space;
@@ -315,7 +346,7 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
       if (!info.shape.empty()) innermostOutputExtent = std::max<size_t>(innermostOutputExtent, info.shape.back());
     }
     for (const auto& seed :
-         detail::heuristicSeeds(baseMappings.front(), firstInputs, smallestOutputRank, innermostOutputExtent)) {
+         detail::heuristicSeeds(baseMappings.front(), firstInputs, smallestOutputRank, innermostOutputExtent, fewOutputs)) {
       if (std::find(bases.begin(), bases.end(), seed) != bases.end()) continue;
       try {
         TuningConfiguration c = space;
@@ -483,9 +514,12 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
         }
         try {
           // prune launches that cannot fill even one compute unit
-          auto g = ex.grid().extractDefaultedArray();
-          auto b = ex.block().extractDefaultedArray();
-          if (g[0] * g[1] * g[2] * b[0] * b[1] * b[2] < settings.minLaunchTotalThreads) {
+          // (the largest launch of the TC counts: a small fill may precede the kernel that matters)
+          uint64_t launched = 0;
+          for (const auto& kl : ex.compilationResult().kernels) {
+            launched = std::max<uint64_t>(launched, uint64_t(kl.grid[0]) * kl.grid[1] * kl.grid[2] * kl.block[0] * kl.block[1] * kl.block[2]);
+          }
+          if (launched < settings.minLaunchTotalThreads) {
             cand->invalid = true;
             continue;
           }

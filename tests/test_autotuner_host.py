@@ -29,7 +29,7 @@ def test_search_space_from_shapes():
     fields = dict(kv.split("=") for kv in tc.host_query("search_space", "500x26x72;500x72x26").split(";"))
     tile = [int(x) for x in fields["tile"].split(",")]
     block = [int(x) for x in fields["block"].split(",")]
-    assert fields["tile_dims"] == "4"                       # largest rank + 1
+    assert fields["tile_dims"] == "5"                       # largest rank + 1, + 1 for the slice number of a divided sum
     assert 0 in tile and 0 not in block                     # 0 = "do not tile"; never a block size
     for v in (26, 72, 500, 13, 36, 250, 256, 64):           # divisors of the dims, and of 256
         assert v in tile and v in block

@@ -88,3 +88,25 @@ def test_matrix_product_divided_among_blocks_on_the_matrix_cores():
     s = ex.compiled_source
     assert "__builtin_amdgcn_mfma_f32_16x16x4f32" in s and "__tc::atomicAccumulate(&pC[" in s and "ksplit0_" in s
     assert np.array_equal(got, A @ Bm)
+
+
+def test_the_tuner_divides_a_sum_with_few_outputs():
+    """From the naive options: with 64 outputs the search may divide the sum among blocks (the gene
+    is searched only where outputs are few) and has a structured starting point that does."""
+    d_O = torch.randn(32, 64, 56, 56, generator=torch.Generator().manual_seed(3)).cuda()
+    outs = tc.prepare_outputs(BIAS_GRAD, "bias_grad", [d_O])
+    best = tc.autotune(BIAS_GRAD, "bias_grad", [d_O], "naive", outputs=outs, generations=3, pop_size=30, threads=16, seed=5, top_k=1)
+    ex = tc.compile(BIAS_GRAD, "bias_grad", [d_O], best[0])
+    tc.run(ex, [d_O], outs)
+    torch.cuda.synchronize()
+    ref = d_O.double().sum((0, 2, 3)).float()
+    assert (outs[0] - ref).abs().max().item() <= W.tolerance(32 * 56 * 56, ref.cpu().numpy())
+
+    def time_of(e):
+        tc.profile_repeated(e, [d_O], outs, 50)
+        return min(tc.profile_repeated(e, [d_O], outs, 20) for _ in range(5))
+    plain = tc.compile(BIAS_GRAD, "bias_grad", [d_O],
+                       "naive;tile=1;mapToThreads=1024;mapToBlocks=64;matchLibraryCalls=1;vectorWidth=4;useReadOnlyCache=1")
+    # 64 blocks cannot fill 256 compute units: whatever the search settles on beats the best
+    # mapping that keeps each sum inside one block (25.8 us against about 10)
+    assert time_of(ex) < time_of(plain), best[0].to_text()
