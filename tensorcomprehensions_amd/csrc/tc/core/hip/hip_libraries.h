@@ -49,6 +49,28 @@ template <typename T> __device__ __forceinline__ void storeThrough(__amdgpu_buff
 template <typename T> __device__ __forceinline__ void atomicAccumulate(T* p, T v) {
   __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// The same for any other combining operator (product, minimum, maximum) of a 32- or 64-bit
+// element: compare-and-swap on the bit pattern until the combined value is in place.
+template <typename Op, typename T> __device__ __forceinline__ void atomicCombine(T* p, T v) {
+  static_assert(sizeof(T) == 4 || sizeof(T) == 8, "32- or 64-bit elements");
+  if constexpr (sizeof(T) == 4) {
+    unsigned* q = reinterpret_cast<unsigned*>(p);
+    unsigned seen = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    while (true) {
+      const unsigned want = __builtin_bit_cast(unsigned, Op::apply(__builtin_bit_cast(T, seen), v));
+      if (want == seen) break;
+      if (__hip_atomic_compare_exchange_strong(q, &seen, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) break;
+    }
+  } else {
+    unsigned long long* q = reinterpret_cast<unsigned long long*>(p);
+    unsigned long long seen = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    while (true) {
+      const unsigned long long want = __builtin_bit_cast(unsigned long long, Op::apply(__builtin_bit_cast(T, seen), v));
+      if (want == seen) break;
+      if (__hip_atomic_compare_exchange_strong(q, &seen, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) break;
+    }
+  }
+}
 template <typename T> __device__ __forceinline__ T tmin(T a, T b) { return a < b ? a : b; }
 template <typename T> __device__ __forceinline__ T tmax(T a, T b) { return a > b ? a : b; }
 __device__ __forceinline__ float tmin(float a, float b) { return fminf(a, b); }

@@ -1,6 +1,7 @@
 #include "tc/core/mapper/mapper.h"
 #include "tc/core/mapper/sync_placement.h"
 
+#include <limits>
 #include <algorithm>
 #include <cctype>
 #include <cstdio>
@@ -748,20 +749,47 @@ ir::Function withZeroBasedOutputs(const ir::Function& in) {
   }
   return f;
 }
-// reductionBlocks: a sum `O(p...) +=(!) rhs` is divided among blocks along its outermost reduction
-// index r (extent E, `split` = the largest divisor of E not above `blocks`):
-//     O(p...) = 0                                   only for "+=!", a kernel of its own
-//     O(p...) += rhs[r := r + (E / split) * slice]   slice in 0:split, r in 0:E/split
+// reductionBlocks: a reduction `O(p...) op=(!) rhs` is divided among blocks along its outermost
+// reduction index r (extent E, `split` = the largest divisor of E not above `blocks`):
+//     O(p...) = identity of op                       only for "op=!", a kernel of its own
+//     O(p...) op= rhs[r := r + (E / split) * slice]   slice in 0:split, r in 0:E/split
 // where `slice` becomes the outermost parallel variable of the second statement and its partial
-// sums are added into O atomically.  Floating-point sums then depend on the order in which the
+// results are combined into O atomically.  Floating-point sums then depend on the order in which the
 // blocks arrive (within the rounding of any other summation order); integer sums do not.
+// The identity of a reduction operator as an expression of the given 32- or 64-bit type (values
+// an integer literal cannot spell are formed by an operation: 0 - 1 for the largest uint64).
+ExprRef identityExpr(ReduceOp op, const ScalarType& t) {
+  auto imm = [&](double f, int64_t i) {
+    auto e = std::make_shared<Expr>();
+    e->kind = t.isFloat() ? Expr::FloatImm : Expr::IntImm;
+    e->type = t;
+    e->fval = f;
+    e->ival = i;
+    return ExprRef(e);
+  };
+  auto minus = [&](const ExprRef& a, const ExprRef& b) { return mkExpr(Expr::Binary, t, "-", {a, b}); };
+  if (op == ReduceOp::Plus) return imm(0.0, 0);
+  if (op == ReduceOp::Times) return imm(1.0, 1);
+  const bool largest = op == ReduceOp::Min; // a minimum starts from the largest value of the type
+  if (t.isFloat()) {
+    double m = t.bits == 64 ? std::numeric_limits<double>::max() : static_cast<double>(std::numeric_limits<float>::max());
+    return imm(largest ? m : -m, 0);
+  }
+  if (t.code == ScalarType::UInt) {
+    if (!largest) return imm(0.0, 0);
+    return t.bits == 64 ? minus(imm(0.0, 0), imm(0.0, 1)) : imm(0.0, (int64_t(1) << t.bits) - 1);
+  }
+  const int64_t top = t.bits == 64 ? std::numeric_limits<int64_t>::max() : (int64_t(1) << (t.bits - 1)) - 1;
+  return largest ? imm(0.0, top) : minus(imm(0.0, -top), imm(0.0, 1));
+}
+
 ir::Function withSplitReductions(const ir::Function& in, int64_t blocks) {
   ir::Function f = in;
   f.statements.clear();
   int counter = 0;
   for (const auto& s : in.statements) {
     const ir::Tensor* t = in.find(s.tensor);
-    bool ok = t && s.op == ReduceOp::Plus && !s.redVars.empty() && accessesTo(s, s.tensor).empty() &&
+    bool ok = t && s.op != ReduceOp::None && !s.redVars.empty() && accessesTo(s, s.tensor).empty() &&
         (t->type.bits == 32 || t->type.bits == 64);
     int64_t split = 1, extent = 0;
     if (ok) {
@@ -789,10 +817,7 @@ ir::Function withSplitReductions(const ir::Function& in, int64_t blocks) {
       for (const auto& v : s.lhsVars) zero.ranges[v] = s.ranges.at(v);
       zero.type = t->type;
       zero.tree = s.tree;
-      auto z = std::make_shared<Expr>();
-      z->kind = t->type.isFloat() ? Expr::FloatImm : Expr::IntImm;
-      z->type = t->type;
-      zero.rhs = z;
+      zero.rhs = identityExpr(s.op, t->type);
       f.statements.push_back(zero);
     }
     ir::Statement part = s;
@@ -986,7 +1011,7 @@ MappedProgram mapToHip(
     kc.wide = wide;
     if (wide) kc.idx = "int64";
     mapKernel(kc, limits);
-    for (const auto& st : k.stages) anyThreadReduction |= st.threadReduction;
+    for (const auto& st : k.stages) anyThreadReduction |= st.threadReduction || st.atomic;
     bodies.emplace_back(new Emitter());
     emitKernel(kc, limits, *bodies.back());
   }

@@ -290,7 +290,12 @@ class StageCodegen {
 
   std::string storeStmt(const std::string& cond, const std::string& value) {
     std::string index = flatIndex(st_.tensor, st_.lhsSubs, "");
-    if (st_.atomic) return "if (" + cond + ") __tc::atomicAccumulate(&p" + st_.tensor + "[" + index + "], " + value + ");";
+    if (st_.atomic) {
+      const ReduceOp op = st_.stmts[0].op;
+      const std::string fn =
+          op == ReduceOp::Plus ? "__tc::atomicAccumulate" : "__tc::atomicCombine<" + opStruct(op, accType_) + ">";
+      return "if (" + cond + ") " + fn + "(&p" + st_.tensor + "[" + index + "], " + value + ");";
+    }
     std::string store = streamedStore()
         ? "__tc::storeThrough(" + bufferName(st_.tensor) + ", " + index + ", " + value + ");"
         : "p" + st_.tensor + "[" + index + "] = " + value + ";";

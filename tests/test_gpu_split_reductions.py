@@ -110,3 +110,25 @@ def test_the_tuner_divides_a_sum_with_few_outputs():
     # 64 blocks cannot fill 256 compute units: whatever the search settles on beats the best
     # mapping that keeps each sum inside one block (25.8 us against about 10)
     assert time_of(ex) < time_of(plain), best[0].to_text()
+
+
+@pytest.mark.parametrize("dtype,tc_type", [(np.float32, "float"), (np.float64, "double"), (np.int32, "int32"),
+                                           (np.int64, "int64"), (np.uint32, "uint32"), (np.uint64, "uint64")])
+def test_minimum_maximum_and_product_divided_among_blocks(dtype, tc_type):
+    src = f"""def red({tc_type}(M, K) X) -> (lo, hi, p, cnt) {{
+        lo(m) min=! X(m, k)
+        hi(m) max=! X(m, k)
+        p(m) *=! ((X(m, k) > 5) ? 2 : 1)
+        cnt(m) +=! ((X(m, k) > 5) ? 1 : 0)
+    }}"""
+    X = np.random.Generator(np.random.Philox(65)).integers(0, 200, size=(19, 1200)).astype(dtype)
+    X[3] = 150                                       # a row without any small value
+    X[:, ::40] = 7                                   # about thirty factors of two per row
+    if np.issubdtype(dtype, np.signedinteger) or np.issubdtype(dtype, np.floating):
+        X[5] = -X[5] - 1                             # an all-negative row: the maximum must not start at zero
+    got, ex = run(src, "red", [X], "naive;tile=1,1;mapToThreads=64;mapToBlocks=64,64;matchLibraryCalls=1;reductionBlocks=8")
+    assert ex.num_kernels == 8 and "atomicCombine<__tc::OpMin<" in ex.compiled_source
+    ref = tc_oracle.run(src, "red", [X])
+    assert np.array_equal(ref[0], X.min(1)) and np.array_equal(ref[1], X.max(1))
+    for g, r in zip(got, ref):
+        assert g.dtype == r.dtype and np.array_equal(g, r)

@@ -33,3 +33,18 @@ def test_block_reduction_compiles_for_every_type_operator_and_width(dtype, width
     for op in ("OpSum", "OpProd", "OpMin", "OpMax"):
         assert f"__tc::blockAllReduceX<__tc::{op}<{c_type}>, {width}, 1, 1>" in src, (op, c_type)
     assert ex.num_kernels == 4
+
+
+@pytest.mark.parametrize("dtype", ["int32", "int64", "uint32", "uint64", "float", "double"])
+def test_reductions_divided_among_blocks_compile_for_every_operator(dtype):
+    """reductionBlocks: sums meet in an atomic add, the other operators in a compare-and-swap loop
+    on the bit pattern; 32- and 64-bit element types."""
+    torch_name = {"float": "float32", "double": "float64"}.get(dtype, dtype)
+    ins = [tc.ShapeOnly((8, 1024), torch_name)]
+    options = "naive;tile=1,1;mapToThreads=64;mapToBlocks=64,64;matchLibraryCalls=1;reductionBlocks=8"
+    ex = tc.compile(ALL_OPS.format(T=dtype), "red", ins, options)      # raises on a hipRTC error
+    src = ex.compiled_source
+    assert ex.num_kernels == 8                                          # a fill and a sliced kernel per statement
+    assert "__tc::atomicAccumulate(&ps[" in src
+    for op, out in (("OpProd", "pp"), ("OpMin", "plo"), ("OpMax", "phi")):
+        assert f"__tc::atomicCombine<__tc::{op}<" in src and f">>(&{out}[" in src
