@@ -841,7 +841,7 @@ ir::Function withSplitReductions(const ir::Function& in, int64_t blocks) {
 } // namespace
 
 namespace {
-HipMappingOptions given_options_for_fill(const HipMappingOptions& given) {
+HipMappingOptions fillMappingOptions(const HipMappingOptions& given) {
   HipMappingOptions o = given;
   o.tile(std::vector<uint64_t>{1024}).unroll(4).matchLibraryCalls(false);
   o.mapToThreads(256).mapToBlocks(1 << 20).useSharedMemory(false).usePrivateMemory(false);
@@ -936,7 +936,7 @@ MappedProgram mapToHip(
 
   // The fill that precedes a divided sum: all dimensions merged, four elements per thread, 256
   // threads, as many blocks as that takes.
-  HipMappingOptions fillOptions = given_options_for_fill(optionsIn);
+  HipMappingOptions fillOptions = fillMappingOptions(optionsIn);
   std::vector<const HipMappingOptions*> kernelOptions;
   bool anyThreadReduction = false;
   std::vector<std::unique_ptr<Emitter>> bodies;
