@@ -88,7 +88,7 @@ def device_sync():
         torch.cuda.synchronize()          # (profile_repeated has synchronised the stream already)
 
 
-def measure(name, steps, warmup, options=None):
+def measure(name, steps, warmup, options=None, bursts=1):
     import tensorcomprehensions_amd as tc
     from tests import workloads as W
 
@@ -106,6 +106,11 @@ def measure(name, steps, warmup, options=None):
     device_us = tc.profile_repeated(ex, ins, outs, steps)
     device_sync()
     wall = time.perf_counter() - t0
+    if bursts > 1:
+        # (the workloads beside the headline one: the median of several such bursts, since K launches
+        # of a kernel of a few microseconds are over before the figure has settled)
+        more = [device_us] + [tc.profile_repeated(ex, ins, outs, steps) for _ in range(bursts - 1)]
+        device_us = sorted(more)[len(more) // 2]
     kernel_ms = device_us / 1e3 / steps
     nbytes = algorithmic_bytes(src, entry, ins)
     return {
@@ -371,7 +376,7 @@ def main():
         for name in W.CONFIGS:
             if name == a.config:
                 continue
-            o = measure(name, a.steps, a.warmup)
+            o = measure(name, a.steps, a.warmup, bursts=7)
             others[name] = {"kernel_us": round(o["kernel_ms"] * 1e3, 3), "roofline": roofline(o),
                             "gflops": round(o["flops"] / (o["kernel_ms"] * 1e-3) / 1e9, 1), "launch": o["launch"]}
         line["others"] = others
