@@ -59,6 +59,10 @@ struct Promotion {
   std::string tensor;
   std::string ldsName;
   std::vector<int64_t> extents;      // footprint box, per view dimension
+  // Distance in the tensor between neighbouring footprint elements of a dimension: above 1 when
+  // every access steps through the dimension in multiples of it (I(j, 2 * i + 1)); elements the
+  // computation jumps over are not staged.
+  std::vector<int64_t> steps;
   std::vector<int64_t> ldsStrides;   // row-major, pitches padded against bank conflicts
   int64_t elems = 0;                 // LDS elements including padding
   int64_t reuse = 1;                 // accesses per staged element

@@ -437,6 +437,7 @@ class StageCodegen {
     for (size_t j = 0; j < subs.size(); ++j) {
       if (j) ss << " + ";
       ss << "((" << affineStr(ir::toAffine(subs[j])) << ") - lo" << stageIdx_ << "_" << p.tensor << "_" << j << ")";
+      if (p.steps[j] != 1) ss << " / " << p.steps[j]; // exact: every access is a whole number of steps from the origin
       if (p.ldsStrides[j] != 1) ss << " * " << p.ldsStrides[j];
     }
     if (subs.empty()) ss << "0";
@@ -570,11 +571,17 @@ class StageCodegen {
           hi = std::max(hi, a[j].constant);
         }
         int64_t ext = 1 + (hi - lo);
+        int64_t step = 0; // gcd of everything that moves an access along this dimension
         for (const auto& cv : ref[j].coef) {
-          ext += std::abs(cv.second) * (spanOf(var(cv.first), inside) - 1);
+          const int64_t span = spanOf(var(cv.first), inside);
+          ext += std::abs(cv.second) * (span - 1);
+          if (span > 1) step = gcd(step, cv.second);
         }
+        for (const auto& a : acc.second) step = gcd(step, a[j].constant - lo);
+        if (step > 1) ext = (ext - 1) / step + 1;
         c.fp.minConst.push_back(lo);
         c.p.extents.push_back(ext);
+        c.p.steps.push_back(std::max<int64_t>(1, step));
         elems *= ext;
       }
       c.p.reuse = static_cast<int64_t>(iterations * acc.second.size() / static_cast<double>(elems));
@@ -702,6 +709,7 @@ class StageCodegen {
   // sides and every row starts on a multiple of four elements, threads move 16-byte vectors.
   struct CopyDim {
     int64_t extent, tensorExtent, gStride, lStride;
+    int64_t step; // tensor elements between neighbouring footprint elements
     std::string lo;
     int64_t loGcd; // every value of `lo` is a multiple of this (0: lo is always 0)
     bool inside;   // the footprint never leaves the tensor in this dimension: no bounds test
@@ -756,7 +764,7 @@ class StageCodegen {
       lo += std::min(a, b);
       hi += std::max(a, b);
     }
-    return lo >= 0 && hi + p.extents[j] <= st_.views.at(p.tensor).extents[j];
+    return lo >= 0 && hi + (p.extents[j] - 1) * p.steps[j] + 1 <= st_.views.at(p.tensor).extents[j];
   }
 
   CopyPlan copyPlan(const Promotion& p) const {
@@ -765,14 +773,14 @@ class StageCodegen {
     CopyPlan plan;
     for (auto e : p.extents) plan.count *= e;
     for (size_t j = 0; j < p.extents.size(); ++j) {
-      plan.dims.push_back(CopyDim{p.extents[j], view.extents[j], gStridesFull[j], p.ldsStrides[j],
+      plan.dims.push_back(CopyDim{p.extents[j], view.extents[j], gStridesFull[j], p.ldsStrides[j], p.steps[j],
                                   loPrefix(p) + std::to_string(j), footprintLowGcd(p, j), footprintAlwaysInside(p, j)});
     }
     auto& dims = plan.dims;
     while (dims.size() >= 2) {
       CopyDim& in = dims.back();
       CopyDim& out = dims[dims.size() - 2];
-      bool full = in.extent == in.tensorExtent && out.lStride == in.lStride * in.extent &&
+      bool full = in.extent == in.tensorExtent && in.step == 1 && out.step == 1 && out.lStride == in.lStride * in.extent &&
           out.gStride == in.gStride * in.tensorExtent;
       if (!full) break;
       // (out, in) -> one dimension of extent out*in starting at out.lo * in.extent (in.lo is 0)
@@ -789,7 +797,7 @@ class StageCodegen {
     plan.regType = plan.elemType;
     if (view.type.isFloat() && view.type.bits == 32 && !dims.empty()) {
       const CopyDim& in = dims.back();
-      bool ok = in.gStride == 1 && in.lStride == 1 && in.extent % 4 == 0 && in.tensorExtent % 4 == 0 &&
+      bool ok = in.gStride == 1 && in.lStride == 1 && in.step == 1 && in.extent % 4 == 0 && in.tensorExtent % 4 == 0 &&
           in.loGcd % 4 == 0;
       for (size_t j = 0; j + 1 < dims.size(); ++j) ok &= dims[j].gStride % 4 == 0 && dims[j].lStride % 4 == 0;
       if (ok) {
@@ -845,7 +853,7 @@ class StageCodegen {
       }
       if (loads) {
         std::string g = "g" + std::to_string(j) + "_";
-        em_.line("const int " + g + " = " + dims[j].lo + " + " + l + ";");
+        em_.line("const int " + g + " = " + dims[j].lo + " + " + l + (dims[j].step != 1 ? " * " + std::to_string(dims[j].step) : "") + ";");
         if (!dims[j].inside) {
           cond += (cond.empty() ? "" : " && ") + std::string("(unsigned)") + g + " < " + std::to_string(dims[j].tensorExtent) + "u";
         }
@@ -1428,7 +1436,9 @@ class StageCodegen {
   std::string footprintKey(const Promotion& p) const {
     std::ostringstream ss;
     ss << p.tensor << (p.insideReductionTiles ? "|inside" : "|outside");
-    for (size_t j = 0; j < p.extents.size(); ++j) ss << "|" << p.extents[j] << ":" << p.ldsStrides[j] << ":" << footprintLow(p, j);
+    for (size_t j = 0; j < p.extents.size(); ++j) {
+      ss << "|" << p.extents[j] << ":" << p.steps[j] << ":" << p.ldsStrides[j] << ":" << footprintLow(p, j);
+    }
     return ss.str();
   }
   // Whether every footprint origin is fixed by the block ids and the kernel-level tile loops: the

@@ -157,3 +157,34 @@ def test_reader_of_other_blocks_rows_stays_in_a_kernel_of_its_own():
     assert np.array_equal(ref[1], (A[1:] + 1) + (A[:-1] + 1))
     for g, r in zip(got, ref):
         assert np.array_equal(g, r)
+
+
+@pytest.mark.parametrize("sub,shape", [("2 * i + 1", (42, 420)), ("5 * i", (42, 420)), ("3 * i + 2", (70, 200))])
+@pytest.mark.parametrize("options", [
+    "naive;tile=32,32;mapToThreads=32,8;mapToBlocks=64,64;useSharedMemory=1;unroll=4",
+    "naive;tile=16,64;mapToThreads=64,4;mapToBlocks=2,2;useSharedMemory=1;unroll=1",
+])
+def test_strided_footprints(sub, shape, options):
+    """Only the elements the computation touches are staged (test_cuda_mapper_memory_promotion.cc:709-751)."""
+    src = "def strided(float(N, M) I) -> (O) { O(i, j) = I(j, %s) }" % sub
+    I = np.random.Generator(np.random.Philox(48)).standard_normal(shape, dtype=np.float32)
+    (got,), ex = run(src, "strided", [I], options)
+    assert "lds0_I" in ex.compiled_source
+    (ref,) = tc_oracle.run(src, "strided", [I])
+    a, b = [int(x) for x in sub.replace("* i", "").replace("+", " ").split()] if "+" in sub else (int(sub.split()[0]), 0)
+    n = (shape[1] - 1 - b) // a + 1
+    assert np.array_equal(ref, I[:, b:b + a * (n - 1) + 1:a].T)
+    assert np.array_equal(got, ref)
+
+
+def test_strided_convolution_keeps_every_element():
+    # 2 * w + k with k in 0..4 touches every column: nothing to leave out
+    src = "def sconv(float(N, W) I, float(K) F) -> (O) { O(n, w) +=! I(n, 2 * w + k) * F(k) }"
+    rng = np.random.Generator(np.random.Philox(49))
+    I = rng.integers(-3, 4, size=(30, 131)).astype(np.float32)
+    F = rng.integers(-3, 4, size=(5,)).astype(np.float32)
+    (got,), ex = run(src, "sconv", [I, F], "naive;tile=4,32;mapToThreads=32,4;mapToBlocks=64,64;useSharedMemory=1;unroll=4")
+    assert "lds0_I" in ex.compiled_source and " / 2]" not in ex.compiled_source
+    (ref,) = tc_oracle.run(src, "sconv", [I, F])
+    closed = sum(I[:, k:k + 2 * 63 + 1:2] * F[k] for k in range(5))
+    assert np.array_equal(ref, closed) and np.array_equal(got, ref)

@@ -408,3 +408,15 @@ def test_reduction_blocks_divides_a_sum_among_blocks():
     # the option survives text and wire form
     o = MappingOptions("naive;reductionBlocks=8")
     assert "reductionBlocks=8" in o.normalized() and "reductionBlocks" not in MappingOptions("naive").normalized()
+
+
+def test_strided_accesses_are_staged_without_the_elements_jumped_over():
+    """test/test_cuda_mapper_memory_promotion.cc:709-751: O(i, j) = I(j, 2 * i + 1) promotes a
+    32 x 32 footprint with stride 2 along the second dimension (stride 5 for I(j, 5 * i)); the copy
+    reads the tensor with that stride, the computation reads the staged array without it."""
+    opts = "naive;tile=32,32;mapToThreads=32,8;mapToBlocks=64,64;useSharedMemory=1;unroll=4"
+    for sub, step in (("2 * i + 1", 2), ("5 * i", 5)):
+        src, _ = mapped("def strided(float(N, M) I) -> (O) { O(i, j) = I(j, %s) }" % sub, "strided", [(42, 420)], opts)
+        assert "float lds0_I[1056];" in src                                   # 32 rows of 32 (+1: odd pitch)
+        assert f"const int g1_ = lo0_I_1 + l1_ * {step};" in src              # strided read of the tensor
+        assert f" - lo0_I_1) / {step}];" in src                                # unit stride in the staged array
