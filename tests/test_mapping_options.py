@@ -30,7 +30,7 @@ def test_preset_values():
 def test_serialisation_round_trip():
     o = (MappingOptions.naive().tile(1, 2, 2, 0).mapToThreads(256).mapToBlocks(32, 256).unroll(64).vectorWidth(4)
          .useSharedMemory(True).maxSharedMemory(40000).scheduleFusionStrategy("Max").sharedDepth(3).privateDepth(2)
-         .matchLibraryCalls(True).collapseContiguous(False))
+         .matchLibraryCalls(True).collapseContiguous(False).reductionBlocks(16))
     data = o.serialize()
     back = MappingOptions.deserialize(data)
     assert back == o

@@ -50,7 +50,8 @@ def _file():
         ("private_depth", 9, OPT, U32, None), ("shared_depth", 10, OPT, U32, None),
         # beyond the reference's message: the CDNA4 mapper's own knobs
         ("vector_width", 11, OPT, U32, None), ("collapse_contiguous", 12, OPT, BOOL, None),
-        ("use_mfma", 13, OPT, BOOL, None), ("prefetch_shared", 14, OPT, BOOL, None)])
+        ("use_mfma", 13, OPT, BOOL, None), ("prefetch_shared", 14, OPT, BOOL, None),
+        ("reduction_blocks", 15, OPT, U32, None)])
     message("DLDataTypeProto", [("code", 1, REQ, U32, None), ("bits", 2, REQ, U32, None), ("lanes", 3, REQ, U32, None)])
     message("TensorInfoProto", [("shape", 1, REP, U64, None), ("strides", 2, REP, U64, None), ("alignment", 3, REQ, U64, None),
                                 ("dtype", 4, REQ, MSG, "DLDataTypeProto")])
@@ -93,7 +94,7 @@ OPTIONS = ("naive;outerScheduleFusionStrategy=Max;intraTileScheduleFusionStrateg
            "fixParametersBeforeScheduling=1;tile=1,8,2,0;unroll=128;tileImperfectlyNested=1;matchLibraryCalls=1;"
            "mapToThreads=196,2;mapToBlocks=32,64,3;useSharedMemory=1;usePrivateMemory=1;unrollCopyShared=1;"
            "maxSharedMemory=40000;useReadOnlyCache=1;privateDepth=3;sharedDepth=2;vectorWidth=4;collapseContiguous=0;"
-           "useMfma=1;prefetchShared=1")
+           "useMfma=1;prefetchShared=1;reductionBlocks=8")
 
 
 def test_protobuf_reads_the_serialized_options_field_by_field(messages):
@@ -111,12 +112,14 @@ def test_protobuf_reads_the_serialized_options_field_by_field(messages):
     assert m.use_shared_memory and m.use_private_memory and m.unroll_copy_shared and m.use_readonly_cache
     assert (m.max_shared_memory, m.private_depth, m.shared_depth) == (40000, 3, 2)
     assert (m.vector_width, m.collapse_contiguous, m.use_mfma, m.prefetch_shared) == (4, False, True, True)
+    assert m.reduction_blocks == 8
     # nothing on the wire that the schema does not name: re-serialising gives the same bytes
     assert m.SerializeToString() == serialized(OPTIONS)
     # optional fields that were never set stay absent on the wire
     plain = messages["HipMappingOptionsProto"]()
     plain.ParseFromString(serialized("naive"))
     assert not plain.HasField("max_shared_memory") and not plain.HasField("private_depth") and not plain.HasField("shared_depth")
+    assert not plain.HasField("reduction_blocks")
     assert list(plain.generic_mapping_options.tiling.sizes) == [32, 32, 32] and plain.generic_mapping_options.unroll == 1
 
 
@@ -140,10 +143,12 @@ def test_the_library_reads_options_that_protobuf_serialized(messages):
     n.use_shared_memory, n.use_private_memory, n.unroll_copy_shared, n.use_readonly_cache = True, False, False, True
     n.shared_depth = 1
     n.vector_width, n.collapse_contiguous, n.use_mfma, n.prefetch_shared = 2, True, False, False
+    n.reduction_blocks = 16
     text = from_serialized(n.SerializeToString())
     for fragment in ("outerScheduleFusionStrategy=Preserve3Coincident", "intraTileScheduleFusionStrategy=Max", "tile=4,16", "unroll=16",
                      "matchLibraryCalls=1", "mapToThreads=64,4", "mapToBlocks=500", "useSharedMemory=1", "usePrivateMemory=0",
-                     "useReadOnlyCache=1", "sharedDepth=1", "vectorWidth=2", "collapseContiguous=1", "useMfma=0"):
+                     "useReadOnlyCache=1", "sharedDepth=1", "vectorWidth=2", "collapseContiguous=1", "useMfma=0",
+                     "reductionBlocks=16"):
         assert fragment in text.split(";"), (fragment, text)
     assert "privateDepth" not in text and "maxSharedMemory" not in text
 
