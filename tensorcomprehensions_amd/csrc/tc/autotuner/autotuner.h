@@ -124,7 +124,7 @@ inline std::vector<size_t> mergedDimensionThreadCounts(const std::vector<const D
 // a member of the search space (0, powers of two up to 256, merged-dimension thread counts).
 inline std::vector<HipMappingOptions> heuristicSeeds(
     const HipMappingOptions& base, const std::vector<const DLConstTensor*>& inputs, size_t smallestOutputRank,
-    size_t innermostOutputExtent = 0, bool fewOutputs = false) {
+    size_t innermostOutputExtent = 0, bool fewOutputs = false, const std::vector<int64_t>& firstOutputShape = {}) {
   std::vector<HipMappingOptions> seeds;
   size_t maxRank = 0;
   uint64_t largest = 256; // largest extent: a grid limit that never forces a block to loop over tiles
@@ -196,6 +196,23 @@ inline std::vector<HipMappingOptions> heuristicSeeds(
       o.generic.unroll(unroll);
       o.mapToThreads(innermostOutputExtent, rows).mapToBlocks(largest, 256).useSharedMemory(true).useReadOnlyCache(true);
       o.collapseContiguousValue = false;
+      seeds.push_back(o);
+    }
+  }
+  // convolutions with many channels on the matrix cores: output (n, m, h, w); one image, 32 (16)
+  // output channels and a band of rows per block, the reduction over input channels in tiles of
+  // 8 (16) whose input window and weights are staged in LDS
+  if (firstOutputShape.size() == 4 && firstOutputShape[2] >= 4) {
+    uint64_t band = 1;
+    for (uint64_t d = 1; d <= 16; ++d) {
+      if (static_cast<uint64_t>(firstOutputShape[2]) % d == 0) band = d;
+    }
+    for (bool wide : {true, false}) {
+      HipMappingOptions o = base;
+      o.generic.tile(std::vector<uint64_t>{1, wide ? 32u : 16u, band, 0, wide ? 8u : 16u});
+      o.mapToThreads(64, wide ? 8 : 4).mapToBlocks(largest, 256, 256).useSharedMemory(true).useReadOnlyCache(true);
+      o.useMfmaValue = true;
+      o.prefetchSharedValue = wide;
       seeds.push_back(o);
     }
   }
@@ -346,7 +363,8 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
       if (!info.shape.empty()) innermostOutputExtent = std::max<size_t>(innermostOutputExtent, info.shape.back());
     }
     for (const auto& seed :
-         detail::heuristicSeeds(baseMappings.front(), firstInputs, smallestOutputRank, innermostOutputExtent, fewOutputs)) {
+         detail::heuristicSeeds(baseMappings.front(), firstInputs, smallestOutputRank, innermostOutputExtent, fewOutputs,
+                                outputsInfo.empty() ? std::vector<int64_t>() : outputsInfo.front().shape)) {
       if (std::find(bases.begin(), bases.end(), seed) != bases.end()) continue;
       try {
         TuningConfiguration c = space;
