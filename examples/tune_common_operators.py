@@ -1,4 +1,4 @@
-"""Autotunes a handful of everyday operators written as Tensor Comprehensions, each from the naive
+"""Autotunes ten everyday operators written as Tensor Comprehensions, each from the naive
 mapping options, and times the winner next to PyTorch's own routine on the same GPU.
 
     python examples/tune_common_operators.py [name,name,...] [generations x population, default 5x40]
@@ -54,6 +54,21 @@ OPERATORS = {
                   lambda: [rand(32, 256, 56, 56)], lambda i: i.permute(0, 2, 3, 1).contiguous(), 2 * 32 * 256 * 56 * 56 * 4),
     "gemv": ("def gemv(float(M, K) A, float(K) x) -> (y) { y(m) +=! A(m, k) * x(k) }",
              lambda: [rand(16384, 8192), rand(8192)], lambda a, x: a @ x, 16384 * 8192 * 4),
+    "softmax": ("""def softmax(float(M, N) X) -> (mx, s, Y) {
+        mx(m) max=! X(m, n)
+        s(m) +=! exp(X(m, n) - mx(m))
+        Y(m, n) = exp(X(m, n) - mx(m)) / s(m) }""",
+                lambda: [rand(8192, 4096)], lambda x: torch.softmax(x, 1), 2 * 8192 * 4096 * 4),
+    "maxpool2x2": ("""def maxpool(float(N, C, H, W) I) -> (O) {
+        O(n, c, h, w) max=! I(n, c, 2 * h + kh, 2 * w + kw) where kh in 0:2, kw in 0:2 }""",
+                   lambda: [rand(32, 64, 112, 112)], lambda i: F.max_pool2d(i, 2), 5 * 32 * 64 * 56 * 56 * 4),
+    "depthwise3x3": ("""def depthwise(float(N, C, H, W) I, float(C, KH, KW) W1) -> (O) {
+        O(n, c, h, w) +=! I(n, c, h + kh, w + kw) * W1(c, kh, kw) }""",
+                     lambda: [rand(32, 128, 58, 58), rand(128, 3, 3)],
+                     lambda i, w: F.conv2d(i, w.unsqueeze(1), groups=128), 32 * 128 * (58 * 58 + 56 * 56) * 4),
+    "embedding": ("def embedding(float(V, E) T, int32(B) idx) -> (O) { O(b, e) = T(idx(b), e) }",
+                  lambda: [rand(50000, 1024), torch.randint(0, 50000, (16384,), device="cuda", dtype=torch.int32)],
+                  lambda t, i: F.embedding(i, t), 2 * 16384 * 1024 * 4),
     "bias_gradient": ("def bias_gradient(float(N, M, H, W) d_O) -> (d_B) { d_B(m) +=! d_O(n, m, h, w) }",
                       lambda: [rand(32, 64, 56, 56)], lambda d: d.sum((0, 2, 3)), 32 * 64 * 56 * 56 * 4),
 }

@@ -413,6 +413,42 @@ void emitKernel(KernelCtx& kc, const DeviceLimits& limits, Emitter& em) {
       }
     }
   }
+  // Producer -> consumer through a register (usePrivateMemory): a block-wide reduction over a
+  // one-dimensional block leaves its result in every thread.  When the block produces one element
+  // per kernel-level iteration and the later stages read exactly that element, they use the
+  // register (the reference promotes such written scalars to registers,
+  // memory_promotion_heuristic.cc:581-616).
+  std::vector<std::string> forwardDecls;
+  if (kc.opts.usePrivateMemoryValue && k.block[1] == 1 && k.block[2] == 1) {
+    for (size_t i = 0; i + 1 < gens.size(); ++i) {
+      const StagePlan& prod = k.stages[i];
+      const std::string& t = prod.tensor;
+      if (!prod.threadReduction || prod.atomic || prod.mfma) continue;
+      bool sole = true;
+      for (size_t j = 0; j < k.stages.size(); ++j) sole &= j == i || k.stages[j].tensor != t;
+      if (!sole || tensorsRead(prod).count(t)) continue;
+      auto wbox = gens[i].writeBox();
+      bool ok = wbox.valid;
+      for (size_t d = 0; ok && d < wbox.extents.size(); ++d) ok = wbox.extents[d] == 1;
+      bool anyReader = false;
+      for (size_t j = i + 1; j < gens.size() && ok; ++j) {
+        if (!tensorsRead(k.stages[j]).count(t)) continue;
+        anyReader = true;
+        ok = k.stages[j].views.at(t).extents == prod.views.at(t).extents;
+        auto rbox = ok ? gens[j].readBox(t) : StageCodegen::IterationBox();
+        ok = ok && rbox.valid && rbox.low.size() == wbox.low.size();
+        for (size_t d = 0; ok && d < wbox.low.size(); ++d) {
+          ok = rbox.extents[d] == 1 && rbox.low[d].coef == wbox.low[d].coef && rbox.low[d].constant == wbox.low[d].constant;
+        }
+      }
+      if (!anyReader || !ok) continue;
+      KernelCtx::RegisterForward f;
+      f.producer = static_cast<int>(i);
+      f.name = "rfwd" + std::to_string(i) + "_" + t;
+      forwardDecls.push_back(prod.views.at(t).type.cName() + " " + f.name + ";");
+      kc.registerForwards[t] = f;
+    }
+  }
   // Producer -> consumer through LDS (useSharedMemory): a tensor exactly one stage of the kernel
   // writes and later stages read, when every reader's box of one kernel-level iteration lies inside
   // the producer's and that box fits what is left of LDS.  Stages see the tensor through views that
@@ -423,7 +459,7 @@ void emitKernel(KernelCtx& kc, const DeviceLimits& limits, Emitter& em) {
       const std::string& t = prod.tensor;
       bool sole = true;
       for (size_t j = 0; j < k.stages.size(); ++j) sole &= j == i || k.stages[j].tensor != t;
-      if (!sole || tensorsRead(prod).count(t)) continue;
+      if (!sole || tensorsRead(prod).count(t) || kc.registerForwards.count(t)) continue;
       auto wbox = gens[i].writeBox();
       if (!wbox.valid) continue;
       bool anyReader = false, ok = true;
@@ -638,6 +674,7 @@ void emitKernel(KernelCtx& kc, const DeviceLimits& limits, Emitter& em) {
     g.suppressCopy = true;
   }
   for (const auto& d : cacheDecls) em.line(d);
+  for (const auto& d : forwardDecls) em.line(d);
   // Barriers between the stages: only where a later stage touches what an earlier one wrote (or
   // overwrites what it read) through different threads, at the weakest sufficient level, placed
   // by the exact search of sync_placement.h.  Every stage writes elements indexed by the
@@ -652,7 +689,9 @@ void emitKernel(KernelCtx& kc, const DeviceLimits& limits, Emitter& em) {
       for (int j = i + 1; j < n; ++j) {
         const StagePlan& a = k.stages[i];
         const StagePlan& b = k.stages[j];
-        bool conflict = a.tensor == b.tensor || tensorsRead(b).count(a.tensor) || tensorsRead(a).count(b.tensor);
+        // (a result the later stage takes from a register is no dependence through memory)
+        bool conflict = a.tensor == b.tensor || tensorsRead(a).count(b.tensor) ||
+            (tensorsRead(b).count(a.tensor) && !kc.registerForwards.count(a.tensor));
         if (conflict && !gens[j].readsPrivatelyFrom(a)) need[i][j - i] = level;
       }
     }

@@ -52,6 +52,14 @@ struct KernelCtx {
     int64_t elems = 0;
   };
   std::map<std::string, Forward> forwards;
+  // The result of a block-wide reduction that later stages of the kernel read at the element the
+  // block has just produced: after the reduction every thread holds the value, so the readers take
+  // it from a register instead of from memory (thread 0 still stores it for later kernels).
+  struct RegisterForward {
+    std::string name;
+    int producer = 0;
+  };
+  std::map<std::string, RegisterForward> registerForwards;
   int64_t NT() const { return k.block[0] * k.block[1] * k.block[2]; }
 };
 
@@ -280,7 +288,7 @@ class StageCodegen {
   bool streamedStore() const {
     if (st_.atomic) return false;
     if (!kc_.opts.useReadOnlyCacheValue || viewBytes(st_.tensor) >= (int64_t(1) << 31)) return false;
-    if (forwardOf(st_.tensor)) return true; // the later stages read the copy in LDS
+    if (forwardOf(st_.tensor) || kc_.registerForwards.count(st_.tensor)) return true; // the later stages read the copy
     for (size_t j = stageIdx_ + 1; j < kc_.k.stages.size(); ++j) {
       if (tensorsRead(kc_.k.stages[j]).count(st_.tensor)) return false;
     }
@@ -299,6 +307,12 @@ class StageCodegen {
     std::string store = streamedStore()
         ? "__tc::storeThrough(" + bufferName(st_.tensor) + ", " + index + ", " + value + ");"
         : "p" + st_.tensor + "[" + index + "] = " + value + ";";
+    {
+      auto rf = kc_.registerForwards.find(st_.tensor);
+      if (rf != kc_.registerForwards.end() && rf->second.producer == stageIdx_) {
+        return rf->second.name + " = " + value + "; if (" + cond + ") " + store;
+      }
+    }
     const KernelCtx::Forward* f = forwardOf(st_.tensor);
     if (f && f->producer == stageIdx_) {
       return "if (" + cond + ") { " + store + " " + f->ldsName + "[" + forwardIndex(*f, st_.lhsSubs) + "] = " + value + "; }";
@@ -317,6 +331,10 @@ class StageCodegen {
       if (p.tensor == e->name && activePromotions_.count(p.tensor)) {
         return p.ldsName + "[" + ldsIndex(p, e->args) + "]";
       }
+    }
+    {
+      auto rf = kc_.registerForwards.find(e->name);
+      if (rf != kc_.registerForwards.end() && rf->second.producer < stageIdx_) return rf->second.name;
     }
     if (const KernelCtx::Forward* f = forwardOf(e->name)) {
       if (f->producer < stageIdx_) return f->ldsName + "[" + forwardIndex(*f, e->args) + "]";

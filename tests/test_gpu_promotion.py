@@ -142,6 +142,36 @@ def test_producer_to_consumer_through_lds(options, forwarded):
         assert np.array_equal(g, r), options
 
 
+SOFTMAX = """def softmax(float(M, N) X) -> (mx, s, Y) {
+    mx(m) max=! X(m, n)
+    s(m) +=! exp(X(m, n) - mx(m))
+    Y(m, n) = exp(X(m, n) - mx(m)) / s(m) }"""
+
+
+@pytest.mark.parametrize("shape,options", [
+    ((37, 1000), "naive;tile=1;mapToThreads=128;mapToBlocks=64;matchLibraryCalls=1;usePrivateMemory=1;outerScheduleFusionStrategy=Max"),
+    # blocks that loop over the rows; a row length no thread count divides
+    ((37, 777), "naive;tile=1;mapToThreads=256;mapToBlocks=8;matchLibraryCalls=1;usePrivateMemory=1;vectorWidth=4;outerScheduleFusionStrategy=Max"),
+    ((5, 4096), "naive;tile=1,0;mapToThreads=512;mapToBlocks=256;matchLibraryCalls=1;usePrivateMemory=1;unroll=64;vectorWidth=2;outerScheduleFusionStrategy=Max"),
+    # a row of threads that is no multiple of the wavefront
+    ((19, 300), "naive;tile=1;mapToThreads=100;mapToBlocks=4;matchLibraryCalls=1;usePrivateMemory=1;useSharedMemory=1;outerScheduleFusionStrategy=Max"),
+])
+def test_reduction_results_forwarded_in_registers(shape, options):
+    """The maximum and the sum of a row are handed to the later stages in a register: same values
+    as through memory (the oracle's order for the maximum, the tolerance of a sum for the rest),
+    and the stored per-row results are those the later stages used."""
+    X = np.random.Generator(np.random.Philox(48)).standard_normal(shape).astype(np.float32) * 3
+    got, ex = run(SOFTMAX, "softmax", [X], options)
+    assert "rfwd0_mx" in ex.compiled_source and "rfwd1_s" in ex.compiled_source and ex.num_kernels == 1
+    ref = tc_oracle.run(SOFTMAX, "softmax", [X])
+    assert np.array_equal(got[0], ref[0])                          # a maximum has no rounding
+    np.testing.assert_allclose(got[1], ref[1], rtol=1e-5 * np.sqrt(shape[1]))
+    np.testing.assert_allclose(got[2], ref[2], rtol=1e-5 * np.sqrt(shape[1]), atol=1e-12)
+    # the forwarded values are the stored ones: recomputing the last stage from them is exact up to exp's rounding
+    np.testing.assert_allclose(got[2], np.exp(X - got[0][:, None]) / got[1][:, None], rtol=2e-6, atol=1e-12)
+    np.testing.assert_allclose(got[2].sum(1), 1.0, rtol=1e-5 * np.sqrt(shape[1]))
+
+
 def test_reader_of_other_blocks_rows_stays_in_a_kernel_of_its_own():
     """Rows another block produces are read through memory, after the producing kernel: such a
     reader is not fused with its producer, and nothing is forwarded."""

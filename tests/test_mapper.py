@@ -241,7 +241,7 @@ def test_pointwise_stage_reads_the_reductions_register_cache():
     text, launches = mapped(src, entry, shapes, common + "576")
     assert launches == [((32, 32, 1), (576, 1, 1))]
     assert text.count("pI[") == 1 and "float rcache0_[64];" in text
-    assert "(rcache0_[a_] - (psum[" in text
+    assert "(rcache0_[a_] - (rfwd0_sum / " in text           # the sums come in registers as well
     text, _ = mapped(src, entry, shapes, common + "512")
     assert text.count("pI[") == 2
 
@@ -386,6 +386,32 @@ def test_written_tensor_is_forwarded_to_later_stages_through_lds():
     assert looped.count("__syncthreads();") == src.count("__syncthreads();") + 1
     plain, _ = mapped(chain, "chain", [(40, 48), (48, 70)], base + ";mapToBlocks=64;useSharedMemory=0")
     assert "fwd0_B" not in plain
+
+
+def test_block_wide_reduction_result_is_forwarded_in_a_register():
+    """usePrivateMemory: what a block-wide reduction leaves in every thread is read by the later
+    stages of the kernel from a register (the reference promotes written scalars to registers,
+    memory_promotion_heuristic.cc:581-616); thread 0 still stores it, and no barrier stands between
+    the stages for its sake."""
+    moments = """def moments(float(M, N) X) -> (mean, var) {
+        mean(m) +=! X(m, r_n) / N
+        var(m) +=! (X(m, r_n) - mean(m)) * (X(m, r_n) - mean(m)) / N }"""
+    base = "naive;tile=1;mapToThreads=128;matchLibraryCalls=1;outerScheduleFusionStrategy=Max"
+    src, launches = mapped(moments, "moments", [(37, 1000)], base + ";mapToBlocks=64;usePrivateMemory=1")
+    assert launches == [((37, 1, 1), (128, 1, 1))]
+    stage1 = src.split("// stage 1")[1]
+    assert "float rfwd0_mean;" in src and "rfwd0_mean = acc_[a_]; if (ok_ && threadIdx.x == 0)" in src
+    assert "- rfwd0_mean)" in stage1 and "pmean[" not in stage1
+    plain, _ = mapped(moments, "moments", [(37, 1000)], base + ";mapToBlocks=64;usePrivateMemory=0")
+    assert "rfwd0_mean" not in plain and "pmean[" in plain.split("// stage 1")[1]
+    assert plain.count("__syncthreads();") == src.count("__syncthreads();") + 1
+    # blocks that loop over rows: the register is set anew in every iteration
+    looped, launches = mapped(moments, "moments", [(37, 1000)], base + ";mapToBlocks=8;usePrivateMemory=1")
+    assert launches[0][0] == (8, 1, 1) and "rfwd0_mean" in looped
+    # two rows per block, or rows along threadIdx.y: the value differs between threads' rows
+    for other in (base.replace("tile=1", "tile=2") + ";mapToBlocks=64;usePrivateMemory=1",
+                  base.replace("tile=1", "tile=2").replace("mapToThreads=128", "mapToThreads=64,2") + ";mapToBlocks=64;usePrivateMemory=1"):
+        assert "rfwd0_mean" not in mapped(moments, "moments", [(37, 1000)], other)[0], other
 
 
 def test_reduction_blocks_divides_a_sum_among_blocks():
