@@ -257,7 +257,12 @@ def suite_library_routines():
         "2fcrelu": lambda i, w1, b1, w2, b2: F.relu(F.linear(F.relu(F.linear(i, w1, b1)), w2, b2)),
         "mlp1": lambda i, w1, b1: F.relu(i @ w1 + b1),
         "mlp3": lambda i, w2, b2, w3, b3, w4, b4: F.relu(F.linear(F.relu(F.linear(F.relu(F.linear(i, w2, b2)), w3, b3)), w4, b4)),
+        "c3": lambda a, b: a @ b.t(),
         "lut": lambda t, i: t[i.long()].sum(1),
+        "2lut": lambda t1, i1, t2, i2: (t1[i1.long()].sum(1), t2[i2.long()].sum(1)),
+        "group_normalization": lambda i, g, b, mean, var: (
+            g[None, :, :, None, None] * (i - mean[:, :, None, None, None]) * torch.rsqrt(var[:, :, None, None, None] + 1e-5)
+            + b[None, :, :, None, None]),
         "moments2": lambda x: (x.mean(1), x.var(1, unbiased=False)),
         "group_normalization_single_kernel": lambda i, g, b: F.group_norm(
             i.reshape(i.shape[0], -1, i.shape[3], i.shape[4]), i.shape[1], g.reshape(-1), b.reshape(-1), 1e-5),
@@ -284,8 +289,9 @@ def measure_suite(steps, warmup):
             tc.unchecked_run(ex, ins, outs)
         us = tc.profile_repeated(ex, ins, outs, steps) / steps
         nbytes = sum(t.numel() * t.element_size() for t in ins + outs)
-        if name == "lut":
-            nbytes += (ins[1].numel() * ins[0].shape[1] - ins[0].numel()) * 4
+        if name in ("lut", "2lut"):
+            for table, index in zip(ins[0::2], ins[1::2]):
+                nbytes += (index.numel() * table.shape[1] - table.numel()) * 4
         entry_out = {"kernel_us": round(us, 2), "kernels": ex.num_kernels, "bytes": nbytes,
                      "gb_per_s": round(nbytes / us / 1e3, 1),
                      "launch": [ex.launch_bounds(k) for k in range(ex.num_kernels)]}

@@ -216,13 +216,38 @@ inline std::vector<HipMappingOptions> heuristicSeeds(
       seeds.push_back(o);
     }
   }
-  // dense contractions: one batch element and a 32x32 output tile per block on the matrix cores
+  // dense contractions on the matrix cores: a 32x32 output tile per block (of one batch element,
+  // when the output has more than two dimensions), operands from memory or through LDS
+  const bool matrix = firstOutputShape.size() == 2;
   for (bool lds : {false, true}) {
     HipMappingOptions o = base;
-    o.generic.tile(std::vector<uint64_t>{1, 32, 32});
+    o.generic.tile(matrix ? std::vector<uint64_t>{32, 32} : std::vector<uint64_t>{1, 32, 32});
     o.mapToThreads(64, 4).mapToBlocks(largest, 256).useSharedMemory(lds).useReadOnlyCache(true);
     o.useMfmaValue = true;
     seeds.push_back(o);
+  }
+  if (matrix) {
+    // many output tiles: 64x64 per block, the reduction in tiles of 32 staged through LDS while
+    // the previous tile multiplies
+    {
+      HipMappingOptions o = base;
+      o.generic.tile(std::vector<uint64_t>{64, 64, 32});
+      o.mapToThreads(64, 4).mapToBlocks(largest, largest).useSharedMemory(true).useReadOnlyCache(true);
+      o.useMfmaValue = true;
+      o.prefetchSharedValue = true;
+      seeds.push_back(o);
+    }
+    // few output tiles: two (one) 16x16 tiles per block of 8 (16) wavefronts, which divide the
+    // reduction steps of a tile among themselves
+    for (bool two : {true, false}) {
+      HipMappingOptions o = base;
+      o.generic.tile(std::vector<uint64_t>{16, two ? 32u : 16u});
+      o.generic.unroll(256);
+      o.mapToThreads(two ? 256 : 512, 2).mapToBlocks(largest, largest).useSharedMemory(true).useReadOnlyCache(true);
+      o.useMfmaValue = true;
+      o.vectorWidthValue = 2;
+      seeds.push_back(o);
+    }
   }
   return seeds;
 }

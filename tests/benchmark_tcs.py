@@ -62,6 +62,12 @@ def mlp3(float(B, N) I, float(O, N) W2, float(O) B2, float(P, O) W3, float(P) B3
 }
 """
 
+C3 = """
+def _C3(float(B, WX) I, float(WY, WX) W) -> (C3) {
+    C3(b, wy) +=! I(b, r_wx) * W(wy, r_wx)
+}
+"""
+
 LUT = """
 def lut(float(E, D) LUT, int32(B, L) I) -> (O) {
     O(i, j) +=! LUT(I(i, k), j)
@@ -183,6 +189,7 @@ CASES = {
     "2fcrelu": (FCRELU2, "func_2fcrelu", [(20, 48), (36, 48), (36,), (24, 36), (24,)], 48),
     "mlp1": (MLP1, "mlp1", [(20, 48), (48, 36), (36,)], 48),
     "mlp3": (MLP3, "mlp3", [(20, 24), (18, 24), (18,), (10, 18), (10,), (2, 10), (2,)], 24),
+    "c3": (C3, "_C3", [(20, 48), (36, 48)], 48),
     "lut": (LUT, "lut", [(50, 24), ("int", (9, 7), 0, 50)], 7),
     "2lut": (LUT2, "func_2lut", [(50, 24), ("int", (9, 7), 0, 50), (30, 24), ("int", (9, 5), 0, 30)], 7),
     "batchnorm": (BATCHNORM, "spatialBatchNorm",
@@ -199,8 +206,8 @@ CASES = {
 
 
 # The same comprehensions at the default sizes of the reference's benchmark programs
-# (tc/benchmarks/tmm.cc:42-44, MLP_model.cc:43-59 for the 1000x1024 matmul, the fc-relu chain, the one- and
-# three-layer perceptrons and the look-up table, convolution.cc:40-46, group_convolution.cc:42-49, moments.cc:42-43, group_normalization.cc:42-46,
+# (tc/benchmarks/tmm.cc:42-44, MLP_model.cc:43-59 for the 1000x1024 matmul and its transposed form C3, the fc-relu chain, the one- and
+# three-layer perceptrons and the one and two look-up tables, convolution.cc:40-46, group_convolution.cc:42-49, moments.cc:42-43, group_normalization.cc:42-46,
 # kronecker.cc:41-47, wavenet.cc:42-60), and the mapping options the autotuner found for them on an
 # MI355X (a few generations from the naive options; written relative to the naive options).
 REFERENCE_SIZES = {
@@ -211,8 +218,11 @@ REFERENCE_SIZES = {
     "2fcrelu": [(128, 2000), (128, 2000), (128,), (64, 128), (64,)],
     "mlp1": [(128, 2000), (2000, 128), (128,)],
     "mlp3": [(128, 128), (64, 128), (64,), (32, 64), (32,), (2, 32), (2,)],
+    "c3": [(128, 1000), (1024, 1000)],
     "lut": [(100000, 64), ("int", (128, 50), 0, 100000)],
+    "2lut": [(100000, 64), ("int", (128, 50), 0, 100000), (100000, 64), ("int", (128, 50), 0, 100000)],
     "moments2": [(1024, 36864)],
+    "group_normalization": [(32, 32, 16, 48, 48), (32, 16), (32, 16), (32, 32), ("positive", (32, 32))],
     "group_normalization_single_kernel": [(32, 32, 16, 48, 48), (32, 16), (32, 16)],
     "kronecker3": [(32, 16), (32, 16), (32, 16), (256, 16, 16, 16)],
     "wavenet1": [(1, 32, 4000), (32, 32, 2), (32,), (32, 32, 2), (32,), (32, 32), (32,), (32, 32), (32,), (1,)],
@@ -238,8 +248,12 @@ TUNED_AT_REFERENCE_SIZES = {
     # the three layers in one kernel, 16 batch rows per block, each layer's result handed on in LDS
     "mlp3": "naive;outerScheduleFusionStrategy=Max;intraTileScheduleFusionStrategy=Max;tile=16,256;unroll=16;mapToThreads=256;"
             "mapToBlocks=256,128;useSharedMemory=1;unrollCopyShared=1;sharedDepth=4;useMfma=1;prefetchShared=1",
+    # two 16x16 tiles per block, the 250 reduction steps of a tile split over two wavefronts each
+    "c3": "naive;tile=16,32;unroll=256;mapToThreads=256;mapToBlocks=1024,1024;useSharedMemory=1;unrollCopyShared=1;"
+          "useReadOnlyCache=1;vectorWidth=2;useMfma=1",
     "lut": "naive;outerScheduleFusionStrategy=Min;tile=4,32,32;unroll=64;usePrivateMemory=1;unrollCopyShared=1;"
            "collapseContiguous=0",
+    "2lut": "naive;tile=2,32,32;unroll=256;mapToThreads=64,4,1;mapToBlocks=100000,256;vectorWidth=4;useMfma=1",
     "moments2": "naive;outerScheduleFusionStrategy=Max;fixParametersBeforeScheduling=1;tile=1;unroll=128;"
                 "tileImperfectlyNested=1;matchLibraryCalls=1;mapToThreads=256;mapToBlocks=1152;usePrivateMemory=1;"
                 "unrollCopyShared=1;vectorWidth=2;collapseContiguous=0;useMfma=1",
@@ -249,6 +263,8 @@ TUNED_AT_REFERENCE_SIZES = {
     "group_normalization_single_kernel": "naive;outerScheduleFusionStrategy=Max;intraTileScheduleFusionStrategy=Preserve3Coincident;"
                                          "tile=1,2,0;unroll=128;matchLibraryCalls=1;mapToThreads=576;mapToBlocks=256,256;"
                                          "useSharedMemory=1;usePrivateMemory=1;useReadOnlyCache=1;vectorWidth=4",
+    "group_normalization": "naive;tile=4,1,0,0,0;unroll=16;mapToThreads=48,16,1;mapToBlocks=256,256;useSharedMemory=1;"
+                           "useReadOnlyCache=1;vectorWidth=4",
     "kronecker3": "naive;outerScheduleFusionStrategy=Max;intraTileScheduleFusionStrategy=Max;tile=1,32,32;unroll=8;"
                   "tileImperfectlyNested=1;mapToThreads=64,16;mapToBlocks=256,256;useSharedMemory=1;useReadOnlyCache=1;"
                   "privateDepth=5;collapseContiguous=0;useMfma=1;prefetchShared=1",

@@ -57,6 +57,16 @@ def test_oracle_matches_library_routines():
         close(got, want, k)
     lut, idx = B.make_inputs("lut")
     close(tc_oracle.run(B.LUT, "lut", [lut, idx])[0], f64(lut)[torch.from_numpy(idx).long()].sum(1), 7)
+    ins = B.make_inputs("c3")
+    close(tc_oracle.run(B.C3, "_C3", ins)[0], f64(ins[0]) @ f64(ins[1]).T, 48)
+    lut1, idx1, lut2, idx2 = B.make_inputs("2lut")
+    got = tc_oracle.run(B.LUT2, "func_2lut", [lut1, idx1, lut2, idx2])
+    close(got[0], f64(lut1)[torch.from_numpy(idx1).long()].sum(1), 7)
+    close(got[1], f64(lut2)[torch.from_numpy(idx2).long()].sum(1), 5)
+    I, gamma, beta, mean, var = B.make_inputs("group_normalization")
+    ref = (f64(gamma)[None, :, :, None, None] * (f64(I) - f64(mean)[:, :, None, None, None])
+           / torch.sqrt(f64(var)[:, :, None, None, None] + float(np.float32(1e-5))) + f64(beta)[None, :, :, None, None])
+    close(tc_oracle.run(B.GROUP_NORMALIZATION, "group_normalization", [I, gamma, beta, mean, var])[0], ref, 1)
     X, = B.make_inputs("moments2")
     mean, var = tc_oracle.run(B.MOMENTS2, "moments2_2D_1D", [X])
     close(mean, f64(X).mean(1), 500)
@@ -116,7 +126,8 @@ def test_tuned_options_compile_at_the_reference_sizes(name):
     """The stored options map and compile (hipRTC, gfx950) at the reference's default sizes: the
     thread block fits the device, LDS stays within 160 KB, every kernel has a launch."""
     src, entry, _, _ = B.CASES[name]
-    shapes = [tc.ShapeOnly(s[1], "int32") if isinstance(s[0], str) else tc.ShapeOnly(s) for s in B.REFERENCE_SIZES[name]]
+    shapes = [tc.ShapeOnly(s[1], "int32" if s[0] == "int" else "float32") if isinstance(s[0], str) else tc.ShapeOnly(s)
+              for s in B.REFERENCE_SIZES[name]]
     ex = tc.compile(src, entry, shapes, B.TUNED_AT_REFERENCE_SIZES[name])
     assert ex.num_kernels >= 1 and ex.lds_bytes() <= 160 * 1024
     for k in range(ex.num_kernels):
