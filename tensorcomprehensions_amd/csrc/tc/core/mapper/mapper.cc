@@ -542,7 +542,7 @@ void emitKernel(KernelCtx& kc, const DeviceLimits& limits, Emitter& em) {
       for (const auto& stmt : cs.stmts) {
         if (stmt.op != ReduceOp::None) continue;
         visitUnconditional(stmt.rhs, [&](const ExprRef& e) {
-          if (e->kind != Expr::Load) return;
+          if (e->kind != Expr::Load || kc.registerForwards.count(e->name)) return; // (already in a register)
           StageCodegen::AddressForm want = gens[j].addressForm(e, nullptr);
           if (!want.valid || want.slots > 256) return;
           std::string mine = "p" + e->name + "[" + gens[j].flatIndex(e->name, e->args, "") + "]";
@@ -553,7 +553,7 @@ void emitKernel(KernelCtx& kc, const DeviceLimits& limits, Emitter& em) {
             if (gens[i].cachedStmt_ && gens[i].cachedStmt_ != red) continue;
             std::string found;
             visitUnconditional(red->rhs, [&](const ExprRef& m) {
-              if (m->kind != Expr::Load || !found.empty()) return;
+              if (m->kind != Expr::Load || !found.empty() || kc.registerForwards.count(m->name)) return;
               if (gens[i].addressForm(m, red) == want) {
                 found = "p" + m->name + "[" + gens[i].flatIndex(m->name, m->args, "") + "]";
               }
