@@ -135,7 +135,7 @@ int tc_lang_dump(const char* text, const char* what, char** out);
  * tc/autotuner/autotuner.h:153-161).  Tensors must live on the current device; outputs are
  * scratch the candidates write into.  `settings` is "key=value;..." over generations, pop_size,
  * crossover_rate, mutation_rate, number_elites, threads, seed, cache_file, top_k,
- * min_launch_total_threads, max_serial_depth_ratio, seed_heuristics, refinement_rounds, fix_inert, fix_* ; NULL = flag
+ * min_launch_total_threads, max_serial_depth_ratio, seed_heuristics, refinement_rounds, resample_duplicates, fix_inert, fix_* ; NULL = flag
  * defaults.  Returns the best option text in *best (top_k best, newline separated). */
 int tc_autotune(
     const char* tc, const char* entry_point,

@@ -55,6 +55,7 @@ extern "C" int tc_autotune(
       else if (k == "seed_heuristics") st.seedHeuristics = num() != 0;
       else if (k == "refinement_rounds") st.refinementRounds = num();
       else if (k == "fix_inert") st.fixInertParameters = num() != 0;
+      else if (k == "resample_duplicates") st.resampleDuplicates = num();
       else if (k == "cache_file") st.cacheFile = v;
       else if (k == "fix_tile") fixer.fixTilingParameters(list());
       else if (k == "fix_block") fixer.fixBlockParameters(list());

@@ -16,6 +16,7 @@
 #include <deque>
 #include <iostream>
 #include <mutex>
+#include <set>
 #include <thread>
 #include <unordered_map>
 
@@ -57,6 +58,12 @@ struct TunerSettings {
   // tileImperfectlyNested, privateDepth: they exist for the reference's isl scheduler and its
   // promotion heuristic) keep the value of the first base mapping instead of being searched.
   bool fixInertParameters = true;
+  // A bred candidate that the mapper refuses, or that maps to kernels this run has already
+  // measured (an unmutated survivor, a child of near-identical parents, a mutation of an option
+  // that does not apply), is mutated again, up to this many times, until it maps to something new; elites are left alone.  0 = the
+  // reference's behaviour: such candidates keep their slot in the population and only a handful of
+  // new kernels are measured per generation (6 of 40 on the large tensordot).
+  size_t resampleDuplicates = 4;
 };
 
 namespace detail {
@@ -438,6 +445,40 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
   tc::detail::checkInputsCompliant(function, firstInputs);
   // compiles (worker threads) and measures (this device) every candidate of `population`;
   // returns the runtimes of the valid ones
+  auto mappingKey = [&](const TuningConfiguration& conf) -> std::string { // empty: the mapper refuses it
+    try {
+      MappingOptionsType options = baseMapping;
+      conf.applyToHipMappingOptions(options);
+      auto mapped = Backend::compileWithTcMapper(function.name, function, firstInputs, options);
+      std::string key = mapped.source;
+      for (const auto& k : mapped.kernels) {
+        for (int a = 0; a < 3; ++a) key += "|" + std::to_string(k.grid[a]) + "," + std::to_string(k.block[a]);
+      }
+      return key;
+    } catch (const std::exception&) {
+      return std::string();
+    }
+  };
+  size_t resampled = 0;
+  // bred candidates that would repeat a measured mapping are mutated again (mapping costs a
+  // millisecond or two, no JIT)
+  auto diversify = [&](Population& population) {
+    if (settings.resampleDuplicates == 0) return;
+    std::set<std::string> thisGeneration;
+    for (size_t i = 0; i < population.size(); ++i) {
+      std::string key = mappingKey(population[i]->configuration);
+      if (i >= search.numberElites) {
+        for (size_t attempt = 0; attempt < settings.resampleDuplicates &&
+             (key.empty() || outcomes.count(key) || thisGeneration.count(key));
+             ++attempt) {
+          search.remutate(*population[i]);
+          key = mappingKey(population[i]->configuration);
+          ++resampled;
+        }
+      }
+      if (!key.empty()) thisGeneration.insert(key);
+    }
+  };
   auto evaluatePopulation = [&](Population& population) {
     std::atomic<size_t> cursor{0};
     std::mutex mu;
@@ -638,7 +679,7 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
     if (settings.verbose || flags().tuner_gen_log_generations) {
       std::sort(generationTimes.begin(), generationTimes.end());
       std::cerr << "[tuner] " << what << ": " << generationTimes.size() << "/" << size
-                << " valid, " << duplicates << " duplicate mappings so far";
+                << " valid, " << duplicates << " duplicate mappings so far, " << resampled << " mutated again";
       if (!generationTimes.empty()) {
         std::cerr << " (best/median/worst) " << generationTimes.front().toMicroSecondsF() << "/"
                   << generationTimes[generationTimes.size() / 2].toMicroSecondsF() << "/"
@@ -650,7 +691,10 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
   for (size_t gen = 0; gen < settings.generations; ++gen) {
     report("generation " + std::to_string(gen), evaluatePopulation(search.population), search.population.size());
     if (detail::tunerSignal == SIGINT) break;
-    if (gen + 1 < settings.generations) search.updateParameters();
+    if (gen + 1 < settings.generations) {
+      search.updateParameters();
+      diversify(search.population);
+    }
   }
   // Refinement (deviation): the genetic search recombines whole candidates; the last few percent
   // are usually one gene away from its best one.

@@ -34,6 +34,10 @@ class GeneticSearch {
   // Requires a recorded runtime on every valid candidate; produces the next generation.
   void updateParameters();
 
+  // Mutates one candidate once more (deviation: the autotuner calls it for bred candidates that
+  // would repeat a mapping it has measured).
+  void remutate(CandidateConfiguration& candidate) { mutate(candidate); }
+
   Population population;
   TuningConfiguration lastBestConf;
   const size_t numGenerations;

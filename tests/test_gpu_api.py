@@ -126,6 +126,22 @@ def test_autotune_survives_unmappable_candidates():
     assert 1 <= len(best) <= 2
 
 
+@pytest.mark.parametrize("resample", [0, 4])
+def test_autotune_with_and_without_mutating_duplicates_again(resample):
+    """Bred candidates that would repeat a measured mapping are mutated again by default;
+    `resample_duplicates=0` is the reference's behaviour.  Both searches return a correct winner."""
+    rng = np.random.Generator(np.random.Philox(9))
+    A, B = (rng.integers(-3, 4, size=(48, 40)).astype(np.float32) for _ in range(2))
+    ins = [torch.from_numpy(A).cuda(), torch.from_numpy(B.T.copy()).cuda()]
+    best = tc.autotune(MM, "matmul", ins, "naive", generations=3, pop_size=12, threads=8, seed=5, number_elites=2,
+                       resample_duplicates=resample)
+    assert len(best) == 1
+    ex = tc.compile(MM, "matmul", ins, best[0])
+    (out,) = tc.prepare_outputs(MM, "matmul", ins)
+    tc.run(ex, ins, [out])
+    assert np.array_equal(out.cpu().numpy(), A @ B.T)            # small integers: exact in any order
+
+
 def test_define_compiles_on_demand_and_memoises():
     defs = """
     def add(float(N) A, float(N) B) -> (C) { C(i) = A(i) + B(i) }
