@@ -155,6 +155,46 @@ def launch_floor(steps):
     return out
 
 
+ADD4_TC = "def add4(float(N) A, float(N) B, float(N) C, float(N) D) -> (O) { O(i) = A(i) + B(i) + C(i) + D(i) }"
+STREAM_PROBES = [
+    # name, TC, entry, input shapes, mapping options (each the best of a sweep over block shapes), bytes per launch
+    ("copy 1:1", COPY_TC, "copy", [(COPY_ELEMS,)],
+     "naive;tile=1024;mapToThreads=128;mapToBlocks=2097152;vectorWidth=2;unroll=8;useReadOnlyCache=1", 2 * 4 * COPY_ELEMS),
+    # four reads to one write, 25 690 112 floats each: the mix and the volume of the large tensordot
+    ("add4 4:1", ADD4_TC, "add4", [(25690112,)] * 4,
+     "naive;tile=3136;mapToThreads=784;mapToBlocks=1000000;vectorWidth=2;unroll=128;useReadOnlyCache=1", 5 * 4 * 25690112),
+    # the same with the tensordot's block: 196 threads in lanes of four
+    ("add4 4:1, 196 threads x 4 lanes", ADD4_TC, "add4", [(25690112,)] * 4,
+     "naive;tile=3136;mapToThreads=196;mapToBlocks=1000000;vectorWidth=4;unroll=128;useReadOnlyCache=1", 5 * 4 * 25690112),
+    # reads only, the shape of the moments workload: one row per block
+    ("rowsum 1:0", "def rowsum(float(M, N) X) -> (s) { s(m) +=! X(m, n) }", "rowsum", [(1024, 32768)],
+     "naive;tile=1;mapToThreads=512;mapToBlocks=1024;matchLibraryCalls=1;unroll=8;vectorWidth=4;useReadOnlyCache=1",
+     4 * (1024 * 32768 + 1024)),
+]
+
+
+def stream_probes(steps):
+    """Kernels that do nothing but move data, through the same backend and launched like the
+    workloads: what the memory system delivers for a read:write mix of 1:1, of 4:1 (the large
+    tensordot's) and for reads alone (the moments').  Block shape matters: over thread counts, lane
+    widths and elements per block the 4:1 stream measures 4.7 to 7.1 TB/s (blocks whose share is a
+    power of two of 8 KiB or more are the slow ones), so each probe runs at the best shape found.
+    The workloads' fractions of the 8 TB/s peak are to be read against these."""
+    import numpy as np
+    import tensorcomprehensions_amd as tc
+    out = {}
+    for label, src, entry, shapes, opts, nbytes in STREAM_PROBES:
+        ins = [to_device(np.ones(shape, dtype=np.float32)) for shape in shapes]
+        ex = tc.compile(src, entry, ins, opts)
+        outs = tc.prepare_outputs(src, entry, ins)
+        spin(ex, ins, outs, SPIN_MS)
+        us = sorted(tc.profile_repeated(ex, ins, outs, steps) / steps for _ in range(5))[2]
+        out[label] = {"us_per_launch": round(us, 2), "bytes": nbytes, "gb_per_s": round(nbytes / us / 1e3, 1),
+                      "kernel": ex.kernel_name(), "launch": ex.launch_bounds()}
+        del ins, outs
+    return out
+
+
 def measured_traffic(name, options):
     """HBM bytes per launch from the committed counter summary of this workload, if there is one
     and it was taken under the options being timed."""
@@ -331,6 +371,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--floor", action="store_true",
                     help="also time near-empty copy kernels of 1, 64 and 500 blocks (the cost of a launch)")
+    ap.add_argument("--stream", action="store_true",
+                    help="also time kernels that only move data (copy, four reads to one write, reads alone)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch a plain copy kernel of known size (reference point for HBM byte counters)")
     a = ap.parse_args()
@@ -388,6 +430,8 @@ def main():
         line["others"] = others
     if a.floor:
         line["launch_floor"] = launch_floor(a.steps)
+    if a.stream:
+        line["stream_probes"] = stream_probes(a.steps)
     if a.suite:
         line["suite"] = measure_suite(a.steps, a.warmup)
     print(json.dumps(line))
