@@ -413,32 +413,86 @@ void emitKernel(KernelCtx& kc, const DeviceLimits& limits, Emitter& em) {
       }
     }
   }
-  // Producer -> consumer through a register (usePrivateMemory): a block-wide reduction over a
-  // one-dimensional block leaves its result in every thread.  When the block produces one element
-  // per kernel-level iteration and the later stages read exactly that element, they use the
-  // register (the reference promotes such written scalars to registers,
-  // memory_promotion_heuristic.cc:581-616).
+  // Producer -> consumer through a register (usePrivateMemory): a block-wide reduction along
+  // threadIdx.x leaves its result in every thread of the row.  When the element a thread has just
+  // finished is the very element every later read of that tensor in the kernel asks of it, the
+  // readers use the register (the reference promotes such written scalars to registers,
+  // memory_promotion_heuristic.cc:581-616).  That holds when each subscript, on both sides, is one
+  // parallel variable that the two stages tile alike at kernel level and spread alike over the
+  // blocks and over threadIdx.y/z with one point per thread.
   std::vector<std::string> forwardDecls;
-  if (kc.opts.usePrivateMemoryValue && k.block[1] == 1 && k.block[2] == 1) {
+  if (kc.opts.usePrivateMemoryValue) {
+    auto findVar = [](const StagePlan& st, const std::string& name, int* pos) -> const LoopVar* {
+      for (size_t v = 0; v < st.vars.size(); ++v) {
+        if (st.vars[v].name == name) {
+          *pos = static_cast<int>(v);
+          return &st.vars[v];
+        }
+      }
+      return nullptr;
+    };
+    // the single variable of a subscript `v + c`; null otherwise
+    auto plainVar = [&](const StagePlan& st, const ExprRef& e, int* pos, int64_t* constant) -> const LoopVar* {
+      Affine a = ir::toAffine(e);
+      if (!a.valid) return nullptr;
+      const LoopVar* found = nullptr;
+      for (const auto& c : a.coef) {
+        if (c.second == 0) continue;
+        if (c.second != 1 || found) return nullptr;
+        found = findVar(st, c.first, pos);
+        if (!found) return nullptr;
+      }
+      *constant = a.constant;
+      return found;
+    };
     for (size_t i = 0; i + 1 < gens.size(); ++i) {
       const StagePlan& prod = k.stages[i];
       const std::string& t = prod.tensor;
-      if (!prod.threadReduction || prod.atomic || prod.mfma) continue;
+      if (!prod.threadReduction || prod.atomic || prod.mfma || prod.accCount != 1) continue;
       bool sole = true;
       for (size_t j = 0; j < k.stages.size(); ++j) sole &= j == i || k.stages[j].tensor != t;
       if (!sole || tensorsRead(prod).count(t)) continue;
-      auto wbox = gens[i].writeBox();
-      bool ok = wbox.valid;
-      for (size_t d = 0; ok && d < wbox.extents.size(); ++d) ok = wbox.extents[d] == 1;
+      // the producer's side: one point per thread, rows along threadIdx.y/z only
+      std::vector<const LoopVar*> pvars;
+      std::vector<int> ppos;
+      std::vector<int64_t> pconst;
+      bool ok = true;
+      bool axisUsed[3] = {false, false, false};
+      for (const auto& sub : prod.lhsSubs) {
+        int pos = -1;
+        int64_t c = 0;
+        const LoopVar* v = plainVar(prod, sub, &pos, &c);
+        ok = ok && v && !v->reduction && !v->vectorLane && v->perThread == 1 && v->threadAxis != 0 &&
+            (pos < k.sharedDepth || v->numTiles == 1);
+        if (!ok) break;
+        if (v->threadAxis > 0) axisUsed[v->threadAxis] = true;
+        pvars.push_back(v);
+        ppos.push_back(pos);
+        pconst.push_back(c);
+      }
+      // a row of threads that works on no element of the tensor reduces nothing but identities
+      for (int a = 1; a < 3 && ok; ++a) ok = k.block[a] == 1 || axisUsed[a];
       bool anyReader = false;
       for (size_t j = i + 1; j < gens.size() && ok; ++j) {
-        if (!tensorsRead(k.stages[j]).count(t)) continue;
+        const StagePlan& cons = k.stages[j];
+        if (!tensorsRead(cons).count(t)) continue;
         anyReader = true;
-        ok = k.stages[j].views.at(t).extents == prod.views.at(t).extents;
-        auto rbox = ok ? gens[j].readBox(t) : StageCodegen::IterationBox();
-        ok = ok && rbox.valid && rbox.low.size() == wbox.low.size();
-        for (size_t d = 0; ok && d < wbox.low.size(); ++d) {
-          ok = rbox.extents[d] == 1 && rbox.low[d].coef == wbox.low[d].coef && rbox.low[d].constant == wbox.low[d].constant;
+        ok = cons.views.at(t).extents == prod.views.at(t).extents;
+        for (const auto& stmt : cons.stmts) {
+          visit(stmt.rhs, [&](const ExprRef& e) {
+            if (!ok || e->kind != Expr::Load || e->name != t) return;
+            ok = e->args.size() == pvars.size();
+            for (size_t d = 0; ok && d < pvars.size(); ++d) {
+              int pos = -1;
+              int64_t c = 0;
+              const LoopVar* v = plainVar(cons, e->args[d], &pos, &c);
+              const LoopVar* w = pvars[d];
+              ok = v && c == pconst[d] && !v->reduction && !v->vectorLane && v->perThread == 1 && v->min == w->min &&
+                  v->extent == w->extent && v->tile == w->tile && v->numTiles == w->numTiles &&
+                  v->blockAxis == w->blockAxis && v->gridExtent == w->gridExtent && v->threadAxis == w->threadAxis &&
+                  (v->numTiles == 1 || (pos == ppos[d] && pos < k.sharedDepth));
+            }
+          });
         }
       }
       if (!anyReader || !ok) continue;

@@ -155,6 +155,10 @@ SOFTMAX = """def softmax(float(M, N) X) -> (mx, s, Y) {
     ((5, 4096), "naive;tile=1,0;mapToThreads=512;mapToBlocks=256;matchLibraryCalls=1;usePrivateMemory=1;unroll=64;vectorWidth=2;outerScheduleFusionStrategy=Max"),
     # a row of threads that is no multiple of the wavefront
     ((19, 300), "naive;tile=1;mapToThreads=100;mapToBlocks=4;matchLibraryCalls=1;usePrivateMemory=1;useSharedMemory=1;outerScheduleFusionStrategy=Max"),
+    # rows of the tensor along threadIdx.y: a wavefront per row, two rows per wavefront, two wavefronts per row
+    ((37, 1000), "naive;tile=4;mapToThreads=64,4;mapToBlocks=64;matchLibraryCalls=1;usePrivateMemory=1;outerScheduleFusionStrategy=Max"),
+    ((37, 300), "naive;tile=8;mapToThreads=32,8;mapToBlocks=3;matchLibraryCalls=1;usePrivateMemory=1;outerScheduleFusionStrategy=Max"),
+    ((9, 2048), "naive;tile=2;mapToThreads=128,2;mapToBlocks=64;matchLibraryCalls=1;usePrivateMemory=1;vectorWidth=4;outerScheduleFusionStrategy=Max"),
 ])
 def test_reduction_results_forwarded_in_registers(shape, options):
     """The maximum and the sum of a row are handed to the later stages in a register: same values

@@ -408,10 +408,23 @@ def test_block_wide_reduction_result_is_forwarded_in_a_register():
     # blocks that loop over rows: the register is set anew in every iteration
     looped, launches = mapped(moments, "moments", [(37, 1000)], base + ";mapToBlocks=8;usePrivateMemory=1")
     assert launches[0][0] == (8, 1, 1) and "rfwd0_mean" in looped
-    # two rows per block, or rows along threadIdx.y: the value differs between threads' rows
-    for other in (base.replace("tile=1", "tile=2") + ";mapToBlocks=64;usePrivateMemory=1",
-                  base.replace("tile=1", "tile=2").replace("mapToThreads=128", "mapToThreads=64,2") + ";mapToBlocks=64;usePrivateMemory=1"):
-        assert "rfwd0_mean" not in mapped(moments, "moments", [(37, 1000)], other)[0], other
+    # rows along threadIdx.y, one per thread: every thread keeps the result of its own row, and a
+    # block whose rows are single wavefronts needs no block barrier at all
+    rows, launches = mapped(moments, "moments", [(37, 1000)],
+                            base.replace("tile=1", "tile=4").replace("mapToThreads=128", "mapToThreads=64,4") + ";mapToBlocks=64;usePrivateMemory=1")
+    assert launches == [((10, 1, 1), (64, 4, 1))] and "- rfwd0_mean)" in rows.split("// stage 1")[1]
+    kernel = rows[rows.index('extern "C"'):]
+    assert "__syncthreads();" not in kernel and "const int p_m = (int)threadIdx.y;" in kernel
+    # two rows per thread: the register would have to be an array indexed like the reader's loop
+    two = base.replace("tile=1", "tile=2") + ";mapToBlocks=64;usePrivateMemory=1"
+    assert "rfwd0_mean" not in mapped(moments, "moments", [(37, 1000)], two)[0]
+    # a second row of threads that only the reader uses would reduce nothing but identities
+    spread = """def spread(float(M, N) X) -> (s, Y) {
+        s(m) +=! X(m, r_n)
+        Y(m, j, n) = X(m, n) - s(m) where j in 0:4 }"""
+    src, launches = mapped(spread, "spread", [(37, 256)],
+                           "naive;tile=1,4,0;mapToThreads=64,4;mapToBlocks=64;matchLibraryCalls=1;usePrivateMemory=1;outerScheduleFusionStrategy=Max")
+    assert launches[0][1][1] == 4 and "rfwd0_s" not in src
 
 
 def test_reduction_blocks_divides_a_sum_among_blocks():
