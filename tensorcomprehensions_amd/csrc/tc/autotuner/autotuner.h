@@ -175,6 +175,22 @@ inline std::vector<HipMappingOptions> heuristicSeeds(
       seeds.push_back(o);
     }
   }
+  // short rows: four of them per block along threadIdx.y, a wavefront each (the results of the
+  // reductions then reach the later stages in registers and the block needs no barrier)
+  {
+    HipMappingOptions o = base;
+    std::vector<uint64_t> rows(std::max<size_t>(1, smallestOutputRank), 1);
+    rows.back() = 4;
+    rows.push_back(0);
+    o.generic.tile(rows);
+    o.generic.unroll(64);
+    o.generic.matchLibraryCallsValue = true;
+    o.generic.outerScheduleOptions.fusionStrategy = FusionStrategy::Max;
+    o.mapToThreads(64, 4).mapToBlocks(largest, 256).useReadOnlyCache(true).usePrivateMemory(true);
+    o.vectorWidthValue = 4;
+    o.collapseContiguousValue = true;
+    seeds.push_back(o);
+  }
   // few outputs, long sums: the rows as above, the outermost reduction index divided among blocks
   // (the slice number is the first variable of the divided statement)
   if (fewOutputs) {

@@ -67,13 +67,15 @@ def test_structured_seeds_are_members_of_the_search_space():
     mapping next to it; every seed is expressible in the space built from the same shapes (a seed
     that is not is left out), here for the tensordot, the row moments and the batched matmul."""
     seeds = tc.host_query("tuner_seeds", "5:32x512x8x28x28;32x8x2x28x28").split("\n")
-    assert len(seeds) == 17                                   # (3 streaming + 2 reduction) x {256, 196, 392} threads + 2 mfma
+    assert len(seeds) == 18                                   # (3 streaming + 2 reduction) x {256, 196, 392} threads + short rows + 2 mfma
     parsed = [dict(kv.split("=") for kv in tc.MappingOptions(s).normalized().split(";")) for s in seeds]
     assert {p["mapToThreads"] for p in parsed} == {"256", "196", "392", "64,4"}     # 28*28/4, 28*28/2
     assert any(p["tile"] == "1,8,0,0,0" and p["vectorWidth"] == "4" and p["mapToThreads"] == "196" for p in parsed)
-    assert sum(p["matchLibraryCalls"] == "1" for p in parsed) == 6 and sum(p["useMfma"] == "1" for p in parsed) == 2
+    assert sum(p["matchLibraryCalls"] == "1" for p in parsed) == 7 and sum(p["useMfma"] == "1" for p in parsed) == 2
     rows = tc.host_query("tuner_seeds", "1:1024x32768").split("\n")
-    assert len(rows) == 7                                     # no merged extent of at most 4096: 256 threads only
+    assert len(rows) == 8                                     # no merged extent of at most 4096: 256 threads only
+    # short rows: four per block along threadIdx.y, a wavefront each
+    assert sum(";tile=4,0;" in r and "mapToThreads=64,4" in r and "usePrivateMemory=1" in r for r in rows) == 1
     # row reductions: one row per block (tile 1 on each dimension of the lowest-rank output), the
     # reduction dimension whole, a grid limit that covers all rows
     assert sum(";tile=1,0;" in r and "matchLibraryCalls=1" in r and "mapToBlocks=32768,256" in r for r in rows) == 2
