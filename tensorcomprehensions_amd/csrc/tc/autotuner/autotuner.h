@@ -306,6 +306,23 @@ inline TuningConfiguration setupTuningParameters(
 
 } // namespace detail
 
+// The reference's form of the cache-file query (tc/autotuner/options_cache-inl.h:337-353): the
+// key is derived from the TC text, the entry point and the input tensors.  Empty when the file
+// does not exist.
+template <typename Backend>
+std::vector<typename Backend::MappingOptionsType> loadTopKFromCacheFile(
+    const std::string& tc, const std::string& entryPoint, const std::string& cacheFilename,
+    const std::vector<const DLConstTensor*>& inputs, size_t count) {
+  auto defs = tc::detail::parse(tc);
+  TC_CHECK_EQ(defs.count(entryPoint), 1u) << "attempting to access undefined function " << entryPoint;
+  CompilerOptions quiet;
+  quiet.emitWarnings = false;
+  std::ostringstream canon;
+  canon << lang::canonicalize(lang::Sema(quiet).checkFunction(defs.at(entryPoint)));
+  return loadTopKFromCacheFile<Backend>(
+      canon.str(), makeTensorInfoVector(inputs), tc::inferOutputTensorInfo(tc, entryPoint, inputs), cacheFilename, count);
+}
+
 template <typename Backend, typename SearchStrategy>
 class Autotuner {
  public:

@@ -1,6 +1,7 @@
 """The C++ ATen-level surface (tc::aten::compile<HipBackend>, prepareOutputs, profile,
-ATenAutotuner<HipBackend, GeneticSearch>) exercised by the port of the reference's introductory
-example, tc/examples/tensordot.cc:37-90."""
+ATenAutotuner<HipBackend, GeneticSearch>, the options-cache file helpers) exercised by the
+reference's examples on the HIP backend: tc/examples/tensordot.cc:37-90 and
+tc/examples/blockdiagperm.cc:45-152."""
 import os
 import re
 import subprocess
@@ -22,3 +23,24 @@ def test_tensordot_example_runs_and_matches_einsum():
     diff = float(re.search(r"max \|diff\| vs at::einsum: ([0-9.e+-]+)", out.stdout).group(1))
     assert diff <= 1e-5 * 4 * 16          # 1e-5 * sqrt(16) * max|ref| (inputs in [0,1): ref <= 16)
     assert "tc::HipMappingOptions::makeNaiveMappingOptions()" in out.stdout
+
+
+def test_blockdiagperm_example_reinforces_its_cache_file(tmp_path):
+    """Two comprehensions tuned one after the other; the first run starts from the naive options
+    and leaves its best options in the cache file, the second run starts from them
+    (loadTopKFromCacheFile / appendTopKToCacheFile, tc/autotuner/options_cache-inl.h:337-370)."""
+    exe = os.path.join(ROOT, "examples", "blockdiagperm")
+    if not os.path.exists(exe):
+        pytest.fail("examples/blockdiagperm not built (make -C tensorcomprehensions_amd/csrc example)")
+    cache = str(tmp_path / "blockdiagperm.options")
+    starts = []
+    for _ in range(2):
+        out = subprocess.run([exe, "2", "8", cache], capture_output=True, text=True, timeout=300)
+        print(out.stdout[-2000:], out.stderr[-2000:], flush=True)
+        assert out.returncode == 0 and out.stdout.count("ran in:") == 2
+        diff = float(re.search(r"vs at::einsum: ([0-9.e+-]+)", out.stdout).group(1))
+        assert diff <= 1e-5 * 8 * 50      # 1e-5 * sqrt(50) * max|ref| (inputs in [0,1): ref <= 50)
+        assert "permutation equals at::index_select: yes" in out.stdout
+        starts.append(re.search(r"starts from (the naive|cached) options", out.stdout).group(1))
+        assert os.path.getsize(cache) > 0
+    assert starts == ["the naive", "cached"]
