@@ -1,7 +1,7 @@
 """The C++ ATen-level surface (tc::aten::compile<HipBackend>, prepareOutputs, profile,
 ATenAutotuner<HipBackend, GeneticSearch>, the options-cache file helpers) exercised by the
-reference's examples on the HIP backend: tc/examples/tensordot.cc:37-90 and
-tc/examples/blockdiagperm.cc:45-152."""
+reference's examples on the HIP backend: tc/examples/tensordot.cc:37-90,
+tc/examples/blockdiagperm.cc:45-152 and tc/examples/group_normalization.cc:45-140."""
 import os
 import re
 import subprocess
@@ -44,3 +44,23 @@ def test_blockdiagperm_example_reinforces_its_cache_file(tmp_path):
         starts.append(re.search(r"starts from (the naive|cached) options", out.stdout).group(1))
         assert os.path.getsize(cache) > 0
     assert starts == ["the naive", "cached"]
+
+
+@pytest.mark.parametrize("start", ["naive", "best"])
+def test_group_normalization_example_matches_group_norm(start):
+    """One comprehension with two reductions and the normalising statement, tuned from the naive
+    options or from options written with the fluent C++ builder
+    (tc/examples/group_normalization.cc:45-63), against at::group_norm."""
+    exe = os.path.join(ROOT, "examples", "group_normalization")
+    if not os.path.exists(exe):
+        pytest.fail("examples/group_normalization not built (make -C tensorcomprehensions_amd/csrc example)")
+    out = subprocess.run([exe, "2", "8", start], capture_output=True, text=True, timeout=300)
+    print(out.stdout[-2500:], out.stderr[-2000:], flush=True)
+    assert out.returncode == 0 and out.stdout.count("ran in:") == 1
+    diff = float(re.search(r"vs at::group_norm: ([0-9.e+-]+)", out.stdout).group(1))
+    # sums of 36 864 terms, a variance from a difference of two of them, outputs of a few units
+    assert diff <= 1e-4
+    assert "tc::HipMappingOptions::makeNaiveMappingOptions()" in out.stdout
+    if start == "best":
+        microseconds = float(re.search(r"ran in: ([0-9.]+)us", out.stdout).group(1))
+        assert microseconds < 80           # the builder-written options or better (they measure 47 us)
