@@ -1,0 +1,137 @@
+// Host-side driver for a build of the library with AddressSanitizer and UndefinedBehaviorSanitizer:
+// front end, range inference, mapper, code generator and the option codecs run over a corpus of
+// comprehensions x mapping options through the C ABI (tc_map and friends; no GPU call is made).
+// Refusals are fine; a sanitizer report or a crash fails the run.
+//
+// Corpus file, one record per comprehension:
+//   entry point
+//   tensor specs:  <code>:<bits>:<d0>x<d1>...  separated by blanks (code 0 int, 1 uint, 2 float)
+//   the TC text, ended by a line "%%"
+//   option texts, one per line, ended by a line "@@"
+#include <cstdio>
+#include <cstdlib>
+#include <fstream>
+#include <iostream>
+#include <sstream>
+#include <string>
+#include <vector>
+
+#include "tc_hip.h"
+
+namespace {
+struct Tensor {
+  std::vector<int64_t> shape;
+  tc_dl_tensor t;
+};
+
+std::vector<Tensor> parseSpecs(const std::string& line) {
+  std::vector<Tensor> out;
+  std::istringstream ss(line);
+  std::string spec;
+  while (ss >> spec) {
+    Tensor x;
+    unsigned code = 0, bits = 0;
+    size_t a = spec.find(':'), b = spec.find(':', a + 1);
+    code = std::stoul(spec.substr(0, a));
+    bits = std::stoul(spec.substr(a + 1, b - a - 1));
+    std::string dims = spec.substr(b + 1);
+    std::istringstream ds(dims);
+    std::string d;
+    while (std::getline(ds, d, 'x')) {
+      if (!d.empty()) x.shape.push_back(std::stoll(d));
+    }
+    x.t.data = nullptr;
+    x.t.ctx = {10, 0};
+    x.t.dtype = {static_cast<uint8_t>(code), static_cast<uint8_t>(bits), 1};
+    x.t.strides = nullptr;
+    x.t.byte_offset = 0;
+    out.push_back(x);
+  }
+  for (auto& x : out) {
+    x.t.ndim = static_cast<int32_t>(x.shape.size());
+    x.t.shape = x.shape.data();
+  }
+  return out;
+}
+} // namespace
+
+int main(int argc, char** argv) {
+  if (argc < 2) {
+    std::cerr << "usage: mapper_sanitized <corpus file>\n";
+    return 2;
+  }
+  std::ifstream in(argv[1]);
+  std::string entry;
+  size_t mapped = 0, refused = 0, records = 0, damagedMessages = 0;
+  unsigned long long lcg = 88172645463325252ULL;
+  while (std::getline(in, entry)) {
+    if (entry.empty()) continue;
+    std::string specs, line, text;
+    std::getline(in, specs);
+    while (std::getline(in, line) && line != "%%") text += line + "\n";
+    std::vector<Tensor> tensors = parseSpecs(specs);
+    std::vector<const tc_dl_tensor*> ptrs;
+    for (auto& x : tensors) ptrs.push_back(&x.t);
+    ++records;
+    // front end alone
+    for (const char* what : {"function", "sema", "canonical"}) {
+      char* dump = nullptr;
+      if (tc_lang_dump(text.c_str(), what, &dump) == 0) tc_free(dump);
+    }
+    tc_tensor_info infos[16];
+    int count = 0;
+    tc_infer_output_info(text.c_str(), entry.c_str(), ptrs.data(), static_cast<int>(ptrs.size()), infos, 16, &count);
+    while (std::getline(in, line) && line != "@@") {
+      if (line.empty()) continue;
+      // option codecs: text -> normal form -> wire -> text -> C++
+      char* normal = nullptr;
+      if (tc_options_normalize(line.c_str(), &normal) == 0) {
+        void* bytes = nullptr;
+        size_t size = 0;
+        if (tc_options_to_serialized(normal, &bytes, &size) == 0) {
+          char* back = nullptr;
+          if (tc_options_from_serialized(bytes, size, &back) == 0) {
+            if (std::string(back) != normal) {
+              std::cerr << "options changed on the wire: " << normal << " -> " << back << "\n";
+              return 1;
+            }
+            tc_free(back);
+          }
+          // damaged messages must be refused or read as something else, never read out of bounds
+          std::vector<unsigned char> damaged(static_cast<unsigned char*>(bytes), static_cast<unsigned char*>(bytes) + size);
+          for (int round = 0; round < 6 && !damaged.empty(); ++round) {
+            lcg = lcg * 6364136223846793005ULL + 1442695040888963407ULL;
+            std::vector<unsigned char> m = damaged;
+            size_t at = (lcg >> 33) % m.size();
+            switch ((lcg >> 20) % 4) {
+              case 0: m.resize(at); break;                                          // truncated
+              case 1: m[at] = static_cast<unsigned char>(lcg >> 12); break;          // one byte replaced
+              case 2: m[at] |= 0x80; break;                                          // a varint that runs on
+              default: m.insert(m.begin() + at, 10, static_cast<unsigned char>(0xff)); break;
+            }
+            char* garbage = nullptr;
+            if (tc_options_from_serialized(m.data(), m.size(), &garbage) == 0) tc_free(garbage);
+            ++damagedMessages;
+          }
+          tc_free(bytes);
+        }
+        char* cpp = nullptr;
+        if (tc_options_to_cpp(normal, &cpp) == 0) tc_free(cpp);
+        tc_free(normal);
+      }
+      char* source = nullptr;
+      int kernels = 0;
+      unsigned grids[24], blocks[24];
+      if (tc_map(text.c_str(), entry.c_str(), ptrs.data(), static_cast<int>(ptrs.size()), line.c_str(), &source, &kernels,
+                 grids, blocks) == 0) {
+        ++mapped;
+        tc_free(source);
+      } else {
+        ++refused;
+      }
+    }
+  }
+  std::cout << records << " comprehension(s), " << mapped << " mapping(s), " << refused << " refused, " << damagedMessages
+            << " damaged option message(s) read\n";
+  return 0;
+}
