@@ -12,6 +12,7 @@
 #include <cstdlib>
 #include <fstream>
 #include <iostream>
+#include <iterator>
 #include <sstream>
 #include <string>
 #include <vector>
@@ -59,6 +60,50 @@ int main(int argc, char** argv) {
   if (argc < 2) {
     std::cerr << "usage: mapper_sanitized <corpus file>\n";
     return 2;
+  }
+  // the tuner's host side: value sets, the genetic search on a synthetic cost, the options cache
+  // (a sample cache written to a scratch file, read back, then read again from damaged copies)
+  const std::string scratch = std::string(argv[1]) + ".cache";
+  for (auto q : std::vector<std::pair<const char*, std::string>>{
+           {"powers2_and_ceil_divisors", "72"},
+           {"search_space", "500x26x72;500x72x26"},
+           {"tuner_seeds", "5:32x512x8x28x28;32x8x2x28x28"},
+           {"genetic_search", "seed=3;generations=6;pop_size=20"},
+           {"options_cache_selftest", scratch},
+           {"options_cache_write_sample", scratch},
+           {"options_cache_dump", scratch}}) {
+    char* answer = nullptr;
+    if (tc_host_query(q.first, q.second.c_str(), &answer) != 0) {
+      std::cerr << "host query " << q.first << " failed: " << tc_last_error() << "\n";
+      return 1;
+    }
+    tc_free(answer);
+  }
+  size_t damagedFiles = 0;
+  {
+    std::ifstream f(scratch, std::ios::binary);
+    std::vector<char> file((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+    unsigned long long r = 2463534242ULL;
+    int64_t shape[2] = {8, 16};
+    tc_dl_tensor t{nullptr, {10, 0}, 2, {2, 32, 1}, shape, nullptr, 0};
+    const tc_dl_tensor* ins[1] = {&t};
+    const char* tc = "def copy(float(N, M) I) -> (O) { O(n, m) = I(n, m) }";
+    for (int round = 0; round < 300 && !file.empty(); ++round) {
+      r = r * 6364136223846793005ULL + 1442695040888963407ULL;
+      std::vector<char> m = file;
+      size_t at = (r >> 33) % m.size();
+      switch ((r >> 20) % 4) {
+        case 0: m.resize(at); break;
+        case 1: m[at] = static_cast<char>(r >> 12); break;
+        case 2: m[at] = static_cast<char>(m[at] | 0x80); break;
+        default: m.insert(m.begin() + at, 10, static_cast<char>(0xff)); break;
+      }
+      const std::string path = scratch + ".damaged";
+      std::ofstream(path, std::ios::binary).write(m.data(), static_cast<std::streamsize>(m.size()));
+      char* best = nullptr;
+      if (tc_options_cache_load(tc, "copy", ins, 1, path.c_str(), 1, &best) == 0) tc_free(best);
+      ++damagedFiles;
+    }
   }
   std::ifstream in(argv[1]);
   std::string entry;
@@ -132,6 +177,6 @@ int main(int argc, char** argv) {
     }
   }
   std::cout << records << " comprehension(s), " << mapped << " mapping(s), " << refused << " refused, " << damagedMessages
-            << " damaged option message(s) read\n";
+            << " damaged option message(s) and " << damagedFiles << " damaged cache file(s) read\n";
   return 0;
 }
