@@ -237,7 +237,11 @@ struct Lowering {
       case lang::TK_CAST:
         return mk(Expr::Cast, scalarOf(lang::Cast(e).type()), "", {lower(lang::Cast(e).value(), lets)});
       case '?':
-        return mk(Expr::Select, scalarOf(sema.typeOfExpr(e)), "?", {sub(0), sub(1), sub(2)});
+      {
+        // (operands first, the list after: see lang::Parser::parseExp)
+        ExprRef cond = sub(0), yes = sub(1), no = sub(2);
+        return mk(Expr::Select, scalarOf(sema.typeOfExpr(e)), "?", {cond, yes, no});
+      }
       case '-':
         if (e->trees().size() == 1) {
           return mk(Expr::Unary, scalarOf(sema.typeOfExpr(e)), "-", {sub(0)});
@@ -246,7 +250,10 @@ struct Lowering {
       case '+': case '*': case '/': case '%': case lang::TK_MIN: case lang::TK_MAX:
       case lang::TK_EQ: case lang::TK_NE: case lang::TK_LE: case lang::TK_GE: case '<': case '>':
       case lang::TK_AND: case lang::TK_OR:
-        return mk(Expr::Binary, scalarOf(sema.typeOfExpr(e)), opName(e->kind()), {sub(0), sub(1)});
+      {
+        ExprRef left = sub(0), right = sub(1);
+        return mk(Expr::Binary, scalarOf(sema.typeOfExpr(e)), opName(e->kind()), {left, right});
+      }
       case '!':
         return mk(Expr::Unary, scalarOf(sema.typeOfExpr(e)), "!", {sub(0)});
       default:

@@ -52,7 +52,10 @@ class Parser {
         TreeRef no = parseExp(prec - 1);
         left = Tree::make('?', r, {left, yes, no});
       } else {
-        left = Tree::make(op, r, {left, parseExp(prec)});
+        // (the operand is parsed before the list is formed: an exception thrown while a braced
+        // list is being built leaves its earlier elements undestroyed with GCC before 12)
+        TreeRef right = parseExp(prec);
+        left = Tree::make(op, r, {left, right});
       }
     }
     return left;

@@ -107,7 +107,7 @@ int main(int argc, char** argv) {
   }
   std::ifstream in(argv[1]);
   std::string entry;
-  size_t mapped = 0, refused = 0, records = 0, damagedMessages = 0;
+  size_t mapped = 0, refused = 0, records = 0, damagedMessages = 0, damagedDefinitions = 0;
   unsigned long long lcg = 88172645463325252ULL;
   while (std::getline(in, entry)) {
     if (entry.empty()) continue;
@@ -126,6 +126,30 @@ int main(int argc, char** argv) {
     tc_tensor_info infos[16];
     int count = 0;
     tc_infer_output_info(text.c_str(), entry.c_str(), ptrs.data(), static_cast<int>(ptrs.size()), infos, 16, &count);
+    // damaged definitions must end in an error report, not in a crash
+    for (int round = 0; round < 40; ++round) {
+      lcg = lcg * 6364136223846793005ULL + 1442695040888963407ULL;
+      std::string m = text;
+      size_t at = (lcg >> 33) % m.size();
+      static const char pool[] = "(),+-*/=!<>?:{}[]% 019.eE\nrxab#";
+      switch ((lcg >> 20) % 5) {
+        case 0: m.erase(at, 1 + (lcg >> 10) % 4); break;
+        case 1: m.insert(at, 1, pool[(lcg >> 12) % (sizeof(pool) - 1)]); break;
+        case 2: m[at] = pool[(lcg >> 12) % (sizeof(pool) - 1)]; break;
+        case 3: m.resize(at); break;
+        default: m.insert(at, m.substr(at / 2, 1 + (lcg >> 8) % 12)); break;
+      }
+      char* dump = nullptr;
+      if (tc_lang_dump(m.c_str(), "sema", &dump) == 0) tc_free(dump);
+      tc_infer_output_info(m.c_str(), entry.c_str(), ptrs.data(), static_cast<int>(ptrs.size()), infos, 16, &count);
+      char* source = nullptr;
+      int kernels = 0;
+      unsigned grids[24], blocks[24];
+      if (tc_map(m.c_str(), entry.c_str(), ptrs.data(), static_cast<int>(ptrs.size()), "naive", &source, &kernels, grids, blocks) == 0) {
+        tc_free(source);
+      }
+      ++damagedDefinitions;
+    }
     while (std::getline(in, line) && line != "@@") {
       if (line.empty()) continue;
       // option codecs: text -> normal form -> wire -> text -> C++
@@ -177,6 +201,7 @@ int main(int argc, char** argv) {
     }
   }
   std::cout << records << " comprehension(s), " << mapped << " mapping(s), " << refused << " refused, " << damagedMessages
-            << " damaged option message(s) and " << damagedFiles << " damaged cache file(s) read\n";
+            << " damaged option message(s) and " << damagedFiles << " damaged cache file(s) read, " << damagedDefinitions
+            << " damaged definition(s) parsed\n";
   return 0;
 }
