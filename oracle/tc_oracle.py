@@ -596,6 +596,10 @@ class Analysis:
                 lo = self._type(w[2], s, index_env, lets, allow_access=False)
                 hi = self._type(w[3], s, index_env, lets, allow_access=False)
                 solution[w[1]] = (self._const_int(lo), self._const_int(hi) - 1)   # tc2halide.cc:652-669
+                if solution[w[1]][1] < solution[w[1]][0]:
+                    # (the reference checks inferred ranges only, tc2halide.cc:433-436; a range given
+                    # empty is refused here like an inferred one: nothing would run over it)
+                    raise TcError(f"Empty range for variable {w[1]}: {solution[w[1]][0]}:{solution[w[1]][1] + 1}.")
             else:
                 exists.append(self._type(w[1], s, index_env, lets))
         s.rhs = self._type(s.rhs, s, index_env, lets)

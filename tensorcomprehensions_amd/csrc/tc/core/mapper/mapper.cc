@@ -166,6 +166,7 @@ void mapKernel(KernelCtx& kc, const DeviceLimits& limits) {
     // tile sizes by band position (lanes do not take a position)
     int pos = 0;
     for (auto& v : st.vars) {
+      TC_CHECK_GT(v.extent, 0) << "loop variable " << v.name << " has no points";
       if (v.vectorLane) {
         v.tile = v.extent;
         v.numTiles = 1;

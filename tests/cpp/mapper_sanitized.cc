@@ -127,7 +127,7 @@ int main(int argc, char** argv) {
     int count = 0;
     tc_infer_output_info(text.c_str(), entry.c_str(), ptrs.data(), static_cast<int>(ptrs.size()), infos, 16, &count);
     // damaged definitions must end in an error report, not in a crash
-    for (int round = 0; round < 40; ++round) {
+    for (int round = 0; round < 100; ++round) {
       lcg = lcg * 6364136223846793005ULL + 1442695040888963407ULL;
       std::string m = text;
       size_t at = (lcg >> 33) % m.size();

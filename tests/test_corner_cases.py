@@ -150,6 +150,26 @@ def test_a_tensor_takes_the_bounds_of_its_last_definition_in_every_statement():
     assert o.tolist() == [3.0]
 
 
+@pytest.mark.parametrize("text,shapes", [
+    ("def f(float(N) A) -> (O) { O(i) = A(i) where i in 2:2 }", [(5,)]),
+    ("def f(float(N) A) -> (O) { O(i) = A(i) where i in 4:1 }", [(5,)]),
+    # empty for one statement of a tensor that a later statement defines over five elements
+    ("def f(float(N, K) A, float(N, P) B) -> (O) { O(i) = float(1.5) where i in 0:0\n O(i) += A(i, i) + B(i, j) }", [(5, 6), (5, 7)]),
+    ("def f(float(N) A) -> (O) { O(i) +=! A(i + j) where j in 3:3 }", [(5,)]),
+])
+def test_a_range_given_empty_is_refused(text, shapes):
+    """`where i in a:b` with b <= a: nothing would run over it (a loop variable without points used
+    to reach the mapper and divide by its tile size of zero).  The reference checks inferred
+    ranges only (tc2halide.cc:433-436); front end and oracle refuse the given ones alike."""
+    from oracle import tc_oracle
+    with pytest.raises(tc.TcError, match="Empty range for variable"):
+        tc.infer_output_tensor_info(text, "f", [F(*s) for s in shapes])
+    with pytest.raises(tc.TcError, match="Empty range for variable"):
+        tc.map_only(text, "f", [F(*s) for s in shapes], "naive")
+    with pytest.raises(tc_oracle.TcError, match="Empty range for variable"):
+        tc_oracle.infer_output_shapes(text, "f", shapes)
+
+
 def test_later_statement_cannot_narrow_into_the_tensors_first_type():
     """`O` is int32 by its first definition; accumulating floats into it would be an update
     definition of another type, which the reference's Halide lowering refuses.  The front end and

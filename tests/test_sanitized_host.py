@@ -5,7 +5,7 @@ suite at its test and default sizes, and seeded random comprehensions, each unde
 mapping options (the space the genetic search draws from); every option set also goes through the
 wire codec, and damaged copies of its message (truncated, bytes replaced, varints that run on)
 are read back; the tuner's host side (value sets, the genetic search on a synthetic cost, the
-options cache and 300 damaged copies of a cache file) runs as well, and 40 damaged copies of every
+options cache and 300 damaged copies of a cache file) runs as well, and 100 damaged copies of every
 definition go through parser, semantic analysis and mapper (an error report is the only
 acceptable outcome; a leak on that path counts as a failure).  No GPU call is made.  A sanitizer report aborts the driver."""
 import os
@@ -80,4 +80,4 @@ def test_host_code_is_clean_under_address_and_undefined_behaviour_sanitizers(tmp
     assert "ERROR: AddressSanitizer" not in run.stderr and "runtime error:" not in run.stderr
     comprehensions, mappings = (int(x) for x in re.findall(r"(\d+) comprehension\(s\), (\d+) mapping", run.stdout)[0])
     assert comprehensions >= 130 and mappings >= 3000
-    assert "and 300 damaged cache file(s) read" in run.stdout and "5480 damaged definition(s) parsed" in run.stdout
+    assert "and 300 damaged cache file(s) read" in run.stdout and "13700 damaged definition(s) parsed" in run.stdout
