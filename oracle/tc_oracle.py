@@ -596,10 +596,6 @@ class Analysis:
                 lo = self._type(w[2], s, index_env, lets, allow_access=False)
                 hi = self._type(w[3], s, index_env, lets, allow_access=False)
                 solution[w[1]] = (self._const_int(lo), self._const_int(hi) - 1)   # tc2halide.cc:652-669
-                if solution[w[1]][1] < solution[w[1]][0]:
-                    # (the reference checks inferred ranges only, tc2halide.cc:433-436; a range given
-                    # empty is refused here like an inferred one: nothing would run over it)
-                    raise TcError(f"Empty range for variable {w[1]}: {solution[w[1]][0]}:{solution[w[1]][1] + 1}.")
             else:
                 exists.append(self._type(w[1], s, index_env, lets))
         s.rhs = self._type(s.rhs, s, index_env, lets)
@@ -976,11 +972,22 @@ def build(an: Analysis, native: bool = False, in_tree: bool = False) -> ctypes.C
     return lib
 
 
+def refuse_empty_ranges(an: "Analysis"):
+    """Range inference accepts `where i in 8:4` and reports a negative extent, as the reference's
+    does (test/test_inference.cc:498-511, "silently infers a negative size"); nothing can be run
+    over such a range, so executing the definition is refused."""
+    for s in an.d.stmts:
+        for v, (lo, hi) in s.ranges.items():
+            if hi < lo:
+                raise TcError(f"Empty range for variable {v}: {lo}:{hi + 1}.")
+
+
 def run(tc: str, entry: str, inputs: Sequence[np.ndarray], outputs: Optional[Sequence[np.ndarray]] = None,
         native: bool = False):
     """Execute `entry` on numpy inputs with the compiled canonical loop nest.  Returns the list
     of output arrays.  `outputs` may carry pre-existing values for non-initialising reductions."""
     an = analyze(tc, entry, [a.shape for a in inputs])
+    refuse_empty_ranges(an)
     for name, a in zip(an.inputs, inputs):
         want = _NPTYPE[an.tensors[name].scalar]
         if an.tensors[name].scalar == "bool" and a.dtype == np.bool_:
@@ -1003,6 +1010,7 @@ def run_python(tc: str, entry: str, inputs: Sequence[np.ndarray], acc_dtype=None
     """Pure-Python execution of the same nest for tiny shapes (float32 arithmetic per operation
     unless acc_dtype is given, e.g. np.float64 for a brute-force high-precision answer)."""
     an = analyze(tc, entry, [a.shape for a in inputs])
+    refuse_empty_ranges(an)
     env = {n: np.asarray(a) for n, a in zip(an.inputs, inputs)}
     for o, sc, shape in an.output_shapes():
         env[o] = np.zeros(shape, dtype=acc_dtype or _NPTYPE[sc])

@@ -949,6 +949,16 @@ MappedProgram mapToHip(
     const HipMappingOptions& optionsIn,
     const std::string& specializedName,
     const DeviceLimits& limits) {
+  // Range inference accepts `where i in 8:4` and reports a negative extent, as the reference's does
+  // (test/test_inference.cc:498-511: "silently infers a negative size"); nothing can be launched
+  // over such a range.
+  for (const auto& s : given.statements) {
+    for (const auto& r : s.ranges) {
+      if (r.second.max < r.second.min) {
+        throw lang::errorAt(s.tree) << "Empty range for variable " << r.first << ": " << r.second.min << ":" << r.second.max + 1;
+      }
+    }
+  }
   bool shifted = false;
   for (const auto& t : given.outputs) {
     for (auto m : t.mins) shifted |= m != 0;

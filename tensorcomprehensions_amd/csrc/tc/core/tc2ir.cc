@@ -443,11 +443,6 @@ struct Lowering {
         lang::RangeConstraint rc(w);
         int64_t lo = constantOf(lower(rc.start(), lets), rc.start());
         int64_t hi = constantOf(lower(rc.end(), lets), rc.end()) - 1; // [a, b)
-        if (hi < lo) {
-          // (the reference checks inferred ranges only, tc2halide.cc:433-436; a range given empty
-          // is refused like an inferred one: no kernel can be launched over it)
-          throw lang::errorAt(w) << "Empty range for variable " << rc.ident().name() << ": " << lo << ":" << hi + 1;
-        }
         solution[rc.ident().name()] = Range{lo, hi};
       } else if (w->kind() == lang::TK_EXISTS) {
         existsExprs.push_back(lower(w->tree(0), lets));

@@ -159,15 +159,16 @@ def test_a_tensor_takes_the_bounds_of_its_last_definition_in_every_statement():
 ])
 def test_a_range_given_empty_is_refused(text, shapes):
     """`where i in a:b` with b <= a: nothing would run over it (a loop variable without points used
-    to reach the mapper and divide by its tile size of zero).  The reference checks inferred
-    ranges only (tc2halide.cc:433-436); front end and oracle refuse the given ones alike."""
+    to reach the mapper and divide by its tile size of zero).  Range inference itself accepts it and
+    reports a negative extent, as the reference's does (test/test_inference.cc:498-511, a known
+    answer of tests/test_inference.py); mapping, compiling and the oracle's execution refuse it."""
     from oracle import tc_oracle
     with pytest.raises(tc.TcError, match="Empty range for variable"):
-        tc.infer_output_tensor_info(text, "f", [F(*s) for s in shapes])
-    with pytest.raises(tc.TcError, match="Empty range for variable"):
         tc.map_only(text, "f", [F(*s) for s in shapes], "naive")
+    with pytest.raises(tc.TcError, match="Empty range for variable"):
+        tc.compile(text, "f", [F(*s) for s in shapes], "naive")
     with pytest.raises(tc_oracle.TcError, match="Empty range for variable"):
-        tc_oracle.infer_output_shapes(text, "f", shapes)
+        tc_oracle.run(text, "f", [np.zeros(s, np.float32) for s in shapes])
 
 
 def test_later_statement_cannot_narrow_into_the_tensors_first_type():
