@@ -5,6 +5,7 @@
 
 #include "capi/tc_capi_internal.h"
 #include "tc/autotuner/autotuner.h"
+#include "tc/autotuner/model_backend.h"
 #include "tc/core/hip/hip_tc_executor.h"
 
 namespace {
@@ -19,6 +20,54 @@ std::map<std::string, std::string> parseSettings(const char* s) {
   }
   return m;
 }
+
+// "key=value;..." -> settings, fixed parameters and the number of results asked for
+void readTunerSettings(const char* text, tc::autotune::TunerSettings& st, tc::autotune::TuningParameterFixer& fixer, size_t& topK) {
+  using namespace tc;
+  for (const auto& kv : parseSettings(text)) {
+    const std::string &k = kv.first, &v = kv.second;
+    auto num = [&]() { return static_cast<size_t>(std::stoull(v)); };
+    auto list = [&]() {
+      std::vector<size_t> out;
+      std::stringstream ss(v);
+      std::string item;
+      while (std::getline(ss, item, ',')) out.push_back(std::stoull(item));
+      return out;
+    };
+    if (k == "generations") st.generations = num();
+    else if (k == "pop_size") st.populationSize = num();
+    else if (k == "crossover_rate") st.crossOverRate = static_cast<uint8_t>(num());
+    else if (k == "mutation_rate") st.mutationRate = static_cast<uint8_t>(num());
+    else if (k == "number_elites") st.numberElites = num();
+    else if (k == "threads") st.threads = num();
+    else if (k == "seed") st.seed = static_cast<int64_t>(std::stoll(v));
+    else if (k == "top_k") topK = num();
+    else if (k == "verbose") st.verbose = num() != 0;
+    else if (k == "max_unroll") st.maxUnroll = num();
+    else if (k == "min_launch_total_threads") st.minLaunchTotalThreads = num();
+    else if (k == "max_serial_depth_ratio") st.maxSerialDepthRatio = std::stod(v);
+    else if (k == "seed_heuristics") st.seedHeuristics = num() != 0;
+    else if (k == "refinement_rounds") st.refinementRounds = num();
+    else if (k == "fix_inert") st.fixInertParameters = num() != 0;
+    else if (k == "resample_duplicates") st.resampleDuplicates = num();
+    else if (k == "cache_file") st.cacheFile = v;
+    else if (k == "fix_tile") fixer.fixTilingParameters(list());
+    else if (k == "fix_block") fixer.fixBlockParameters(list());
+    else if (k == "fix_grid") fixer.fixGridParameters(list());
+    else if (k == "fix_unroll") fixer.fixUnrollFactor(num());
+    else if (k == "fix_use_shared_memory") fixer.fixUseSharedMemory(num() != 0);
+    else if (k == "fix_match_library_calls") fixer.fixMatchLibraryCalls(num() != 0);
+    else if (k == "fix_vector_width") fixer.fixVectorWidth(num());
+    else if (k == "fix_collapse_contiguous") fixer.fixCollapseContiguous(num() != 0);
+    else if (k == "fix_outer_fusion") {
+      FusionStrategy fs;
+      TC_CHECK(fusionStrategyFromString(v, &fs)) << "unknown fusion strategy " << v;
+      fixer.fixOuterScheduleFusionStrategy(fs);
+    } else {
+      TC_CHECK(false) << "unknown tuner setting '" << k << "'";
+    }
+  }
+}
 } // namespace
 
 extern "C" int tc_autotune(
@@ -30,49 +79,7 @@ extern "C" int tc_autotune(
     autotune::TunerSettings st;
     autotune::TuningParameterFixer fixer;
     size_t topK = 1;
-    for (const auto& kv : parseSettings(settingsText)) {
-      const std::string &k = kv.first, &v = kv.second;
-      auto num = [&]() { return static_cast<size_t>(std::stoull(v)); };
-      auto list = [&]() {
-        std::vector<size_t> out;
-        std::stringstream ss(v);
-        std::string item;
-        while (std::getline(ss, item, ',')) out.push_back(std::stoull(item));
-        return out;
-      };
-      if (k == "generations") st.generations = num();
-      else if (k == "pop_size") st.populationSize = num();
-      else if (k == "crossover_rate") st.crossOverRate = static_cast<uint8_t>(num());
-      else if (k == "mutation_rate") st.mutationRate = static_cast<uint8_t>(num());
-      else if (k == "number_elites") st.numberElites = num();
-      else if (k == "threads") st.threads = num();
-      else if (k == "seed") st.seed = static_cast<int64_t>(std::stoll(v));
-      else if (k == "top_k") topK = num();
-      else if (k == "verbose") st.verbose = num() != 0;
-      else if (k == "max_unroll") st.maxUnroll = num();
-      else if (k == "min_launch_total_threads") st.minLaunchTotalThreads = num();
-      else if (k == "max_serial_depth_ratio") st.maxSerialDepthRatio = std::stod(v);
-      else if (k == "seed_heuristics") st.seedHeuristics = num() != 0;
-      else if (k == "refinement_rounds") st.refinementRounds = num();
-      else if (k == "fix_inert") st.fixInertParameters = num() != 0;
-      else if (k == "resample_duplicates") st.resampleDuplicates = num();
-      else if (k == "cache_file") st.cacheFile = v;
-      else if (k == "fix_tile") fixer.fixTilingParameters(list());
-      else if (k == "fix_block") fixer.fixBlockParameters(list());
-      else if (k == "fix_grid") fixer.fixGridParameters(list());
-      else if (k == "fix_unroll") fixer.fixUnrollFactor(num());
-      else if (k == "fix_use_shared_memory") fixer.fixUseSharedMemory(num() != 0);
-      else if (k == "fix_match_library_calls") fixer.fixMatchLibraryCalls(num() != 0);
-      else if (k == "fix_vector_width") fixer.fixVectorWidth(num());
-      else if (k == "fix_collapse_contiguous") fixer.fixCollapseContiguous(num() != 0);
-      else if (k == "fix_outer_fusion") {
-        FusionStrategy fs;
-        TC_CHECK(fusionStrategyFromString(v, &fs)) << "unknown fusion strategy " << v;
-        fixer.fixOuterScheduleFusionStrategy(fs);
-      } else {
-        TC_CHECK(false) << "unknown tuner setting '" << k << "'";
-      }
-    }
+    readTunerSettings(settingsText, st, fixer, topK);
     // base options: one per line
     std::vector<HipMappingOptions> bases;
     std::stringstream bs(baseOptions ? baseOptions : "naive");
@@ -380,6 +387,55 @@ extern "C" int tc_host_query(const char* what, const char* arg, char** out) {
       }
     } else if (w == "genetic_search") {
       result = runSyntheticSearch(parseSettings(a.c_str()));
+    } else if (w == "tune_on_model") {
+      // "<settings>|<entry point>|<shape>;<shape>...|<tc text>": the whole tune() on the host
+      // against the cost model of tc/autotuner/model_backend.h (float tensors), from the naive
+      // options -> "best=<option text>\ncost_ns=<its modelled time>\nnaive_ns=<that of the naive options>"
+      size_t p1 = a.find('|'), p2 = a.find('|', p1 + 1), p3 = a.find('|', p2 + 1);
+      TC_CHECK(p1 != std::string::npos && p2 != std::string::npos && p3 != std::string::npos)
+          << "expected <settings>|<entry point>|<shapes>|<tc text>";
+      tc::autotune::TunerSettings st;
+      tc::autotune::TuningParameterFixer fixer;
+      size_t topK = 1;
+      readTunerSettings(a.substr(0, p1).c_str(), st, fixer, topK);
+      const std::string entry = a.substr(p1 + 1, p2 - p1 - 1), text = a.substr(p3 + 1);
+      std::vector<std::vector<int64_t>> shapes;
+      std::stringstream ss(a.substr(p2 + 1, p3 - p2 - 1));
+      std::string sh;
+      while (std::getline(ss, sh, ';')) {
+        std::vector<int64_t> dims;
+        std::stringstream ds(sh);
+        std::string d;
+        while (std::getline(ds, d, 'x')) dims.push_back(std::stoll(d));
+        shapes.push_back(dims);
+      }
+      std::vector<DLConstTensor> ts(shapes.size());
+      std::vector<const DLConstTensor*> ins;
+      for (size_t i = 0; i < shapes.size(); ++i) {
+        ts[i] = DLConstTensor{nullptr, {kDLROCM, 0}, static_cast<int>(shapes[i].size()), {2, 32, 1}, shapes[i].data(), nullptr, 0};
+        ins.push_back(&ts[i]);
+      }
+      auto infos = tc::inferOutputTensorInfo(text, entry, ins);
+      std::vector<DLTensor> os(infos.size());
+      std::vector<const DLTensor*> outs;
+      for (size_t i = 0; i < infos.size(); ++i) {
+        os[i] = DLTensor{nullptr, {kDLROCM, 0}, static_cast<int>(infos[i].shape.size()), infos[i].dtype, infos[i].shape.data(), nullptr, 0};
+        outs.push_back(&os[i]);
+      }
+      using Model = tc::autotune::ModelBackend;
+      tc::autotune::Autotuner<Model, tc::autotune::GeneticSearch> tuner;
+      std::unordered_map<size_t, std::vector<const DLConstTensor*>> inMap{{0, ins}};
+      std::unordered_map<size_t, std::vector<const DLTensor*>> outMap{{0, outs}};
+      HipMappingOptions naive = HipMappingOptions::makeNaiveMappingOptions();
+      auto best = tuner.tune(text, entry, inMap, outMap, {naive}, topK, fixer, st);
+      TC_CHECK(!best.empty()) << "the search found no candidate";
+      auto costOf = [&](const HipMappingOptions& o) {
+        auto ex = tc::compile<Model>(text, entry, ins, o);
+        return ex->profile(ins, outs).kernelRuntime.toNanoSeconds();
+      };
+      std::ostringstream os2;
+      os2 << "best=" << best[0].toText() << "\ncost_ns=" << costOf(best[0]) << "\nnaive_ns=" << costOf(naive);
+      result = os2.str();
     } else if (w == "options_cache_selftest") {
       result = cacheSelfTest(a);
     } else if (w == "options_cache_write_sample") {

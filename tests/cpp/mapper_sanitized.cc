@@ -107,7 +107,7 @@ int main(int argc, char** argv) {
   }
   std::ifstream in(argv[1]);
   std::string entry;
-  size_t mapped = 0, refused = 0, records = 0, damagedMessages = 0, damagedDefinitions = 0;
+  size_t mapped = 0, refused = 0, records = 0, damagedMessages = 0, damagedDefinitions = 0, tuned = 0;
   unsigned long long lcg = 88172645463325252ULL;
   while (std::getline(in, entry)) {
     if (entry.empty()) continue;
@@ -149,6 +149,27 @@ int main(int argc, char** argv) {
         tc_free(source);
       }
       ++damagedDefinitions;
+    }
+    // the whole tuning loop on the cost model (compile threads, evaluation thread, duplicates,
+    // refinement) for every fifth definition with float tensors only
+    bool allFloat = true;
+    std::string shapesArg;
+    for (const auto& x : tensors) {
+      allFloat = allFloat && x.t.dtype.code == 2 && x.t.dtype.bits == 32;
+      if (!shapesArg.empty()) shapesArg += ";";
+      for (size_t d = 0; d < x.shape.size(); ++d) shapesArg += (d ? "x" : "") + std::to_string(x.shape[d]);
+    }
+    if (allFloat && !tensors.empty() && records % 5 == 1) {
+      bool scalarInput = false;
+      for (const auto& x : tensors) scalarInput = scalarInput || x.shape.empty();
+      if (!scalarInput) {
+        const std::string arg = "generations=3;pop_size=12;threads=8;seed=" + std::to_string(records) + "|" + entry + "|" + shapesArg + "|" + text;
+        char* answer = nullptr;
+        if (tc_host_query("tune_on_model", arg.c_str(), &answer) == 0) {
+          tc_free(answer);
+          ++tuned;
+        }
+      }
     }
     while (std::getline(in, line) && line != "@@") {
       if (line.empty()) continue;
@@ -202,6 +223,6 @@ int main(int argc, char** argv) {
   }
   std::cout << records << " comprehension(s), " << mapped << " mapping(s), " << refused << " refused, " << damagedMessages
             << " damaged option message(s) and " << damagedFiles << " damaged cache file(s) read, " << damagedDefinitions
-            << " damaged definition(s) parsed\n";
+            << " damaged definition(s) parsed, " << tuned << " tuned on the cost model\n";
   return 0;
 }

@@ -90,3 +90,42 @@ def test_window_seeds_for_convolutions():
     assert len(windows) == 2
     assert all(";tile=1,1,0,0,0;" in s and "useSharedMemory=1" in s and "collapseContiguous=0" in s for s in windows)
     assert not any("mapToThreads=54" in s for s in tc.host_query("tuner_seeds", "1,54:1024x54").split("\n"))
+
+
+def model_tune(settings, name="c5_moments"):
+    """The whole tune() on the host against a cost model (tc/autotuner/model_backend.h)."""
+    from tests import workloads as W
+    text, entry, shapes, _, _ = W.CONFIGS[name]
+    arg = settings + "|" + entry + "|" + ";".join("x".join(map(str, s)) for s in shapes) + "|" + text
+    fields = dict(line.split("=", 1) for line in tc.host_query("tune_on_model", arg).split("\n"))
+    return fields["best"], int(fields["cost_ns"]), int(fields["naive_ns"])
+
+
+def test_the_tuning_loop_runs_on_the_host_against_a_cost_model():
+    """Compile threads, the evaluation thread, duplicate and refused mappings, the refinement
+    rounds: the tuner's own machinery on a deterministic cost of the mapping (a charge per launch
+    and per statement instance of the busiest thread), with the real front end and mapper."""
+    base = "generations=4;pop_size=20;threads=4;seed=3"
+    best, cost, naive = model_tune(base)
+    assert cost < naive / 10 and tc.MappingOptions(best).normalized() == best
+    assert model_tune(base) == (best, cost, naive)                      # a seeded search repeats itself
+    # without the structured members of generation 0 and without the refinement the search still leaves the naive options
+    _, unseeded, _ = model_tune(base + ";seed_heuristics=0;refinement_rounds=0")
+    assert cost <= unseeded < naive
+    # mutating repeated mappings again never makes a generation worse informed
+    _, plain, _ = model_tune(base + ";seed_heuristics=0;resample_duplicates=0")
+    _, resampled, _ = model_tune(base + ";seed_heuristics=0;resample_duplicates=4")
+    assert plain < naive and resampled < naive
+    for name in ("c2_tensordot", "c3_batch_matmul", "c4_group_convolution"):
+        _, c, n = model_tune("generations=3;pop_size=16;threads=8;seed=5", name)
+        assert c <= n, name
+
+
+def test_tuning_on_the_model_reinforces_its_cache_file(tmp_path):
+    """cache_file: the first run leaves its best options in `<file>.model` (the backend's suffix,
+    as `.cuda` in the reference), a second run starts from them and cannot end worse."""
+    cache = str(tmp_path / "tuned.options")
+    first = model_tune(f"generations=2;pop_size=10;threads=2;seed=1;seed_heuristics=0;cache_file={cache}")
+    assert (tmp_path / "tuned.options.model").stat().st_size > 0
+    second = model_tune(f"generations=2;pop_size=10;threads=2;seed=2;seed_heuristics=0;cache_file={cache}")
+    assert second[1] <= first[1]

@@ -7,7 +7,9 @@ wire codec, and damaged copies of its message (truncated, bytes replaced, varint
 are read back; the tuner's host side (value sets, the genetic search on a synthetic cost, the
 options cache and 300 damaged copies of a cache file) runs as well, and 100 damaged copies of every
 definition go through parser, semantic analysis and mapper (an error report is the only
-acceptable outcome; a leak on that path counts as a failure).  No GPU call is made.  A sanitizer report aborts the driver."""
+acceptable outcome; a leak on that path counts as a failure); every fifth definition is tuned
+against the cost model of tc/autotuner/model_backend.h (eight compile threads and the evaluation
+thread under the sanitizers).  No GPU call is made.  A sanitizer report aborts the driver."""
 import os
 import random
 import re
@@ -81,3 +83,16 @@ def test_host_code_is_clean_under_address_and_undefined_behaviour_sanitizers(tmp
     comprehensions, mappings = (int(x) for x in re.findall(r"(\d+) comprehension\(s\), (\d+) mapping", run.stdout)[0])
     assert comprehensions >= 130 and mappings >= 3000
     assert "and 300 damaged cache file(s) read" in run.stdout and "13700 damaged definition(s) parsed" in run.stdout
+    assert int(re.findall(r"(\d+) tuned on the cost model", run.stdout)[0]) >= 15
+
+
+def test_the_tuning_loop_is_clean_under_thread_sanitizer():
+    """Nine tunings (three definitions, three seeds, eight compile threads each) against the cost
+    model, in a build of the library with ThreadSanitizer."""
+    build = subprocess.run(["make", "-C", CSRC, "-j8", "tsan"], capture_output=True, text=True)
+    assert build.returncode == 0, build.stdout[-3000:] + build.stderr[-3000:]
+    env = dict(os.environ, TSAN_OPTIONS="halt_on_error=1")
+    run = subprocess.run([os.path.join(CSRC, "build", "tsan", "tuner_threads")], capture_output=True, text=True, env=env, timeout=600)
+    print(run.stdout[-300:], run.stderr[-4000:], flush=True)
+    assert run.returncode == 0 and "9 tunings done" in run.stdout
+    assert "ThreadSanitizer" not in run.stderr
