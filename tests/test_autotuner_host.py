@@ -105,7 +105,9 @@ def test_the_tuning_loop_runs_on_the_host_against_a_cost_model():
     """Compile threads, the evaluation thread, duplicate and refused mappings, the refinement
     rounds: the tuner's own machinery on a deterministic cost of the mapping (a charge per launch
     and per statement instance of the busiest thread), with the real front end and mapper."""
-    base = "generations=4;pop_size=20;threads=4;seed=3"
+    # (one compile thread: with several, the order in which candidates reach the evaluation thread,
+    # and with it what is pruned against the best so far, depends on the scheduling of the threads)
+    base = "generations=4;pop_size=20;threads=1;seed=3"
     best, cost, naive = model_tune(base)
     assert cost < naive / 10 and tc.MappingOptions(best).normalized() == best
     assert model_tune(base) == (best, cost, naive)                      # a seeded search repeats itself
