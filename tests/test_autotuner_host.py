@@ -19,6 +19,9 @@ def test_powers2_and_ceil_divisors(n, expected):
     assert [int(x) for x in tc.host_query("powers2_and_ceil_divisors", n).split(",")] == expected
 
 
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
 def test_median_of_even_count_is_integer_mean_of_middle_pair():
     assert tc.host_query("median", "3,1,2,10") == "2"
     assert tc.host_query("median", "5,1,9") == "5"
@@ -131,3 +134,35 @@ def test_tuning_on_the_model_reinforces_its_cache_file(tmp_path):
     assert (tmp_path / "tuned.options.model").stat().st_size > 0
     second = model_tune(f"generations=2;pop_size=10;threads=2;seed=2;seed_heuristics=0;cache_file={cache}")
     assert second[1] <= first[1]
+
+
+@pytest.mark.parametrize("signal_name,ends", [("SIGINT", "finishes the generation"), ("SIGTERM", "aborts")])
+def test_signals_during_tuning(signal_name, ends):
+    """SIGINT lets the running generation finish and returns the best found so far, SIGTERM aborts
+    the search (tc/autotuner/autotuner-inl.h:418-518: the reference's handlers); here on a search
+    far too long to finish, running against the cost model in a child process."""
+    import signal
+    import subprocess
+    import sys
+    import time
+    child = subprocess.Popen(
+        [sys.executable, "-c",
+         "import sys; sys.path.insert(0, %r)\n"
+         "from tests.test_autotuner_host import model_tune\n"
+         "print('started', flush=True)\n"
+         "try:\n"
+         "    best, cost, naive = model_tune('generations=100000;pop_size=60;threads=4;seed=1;refinement_rounds=0')\n"
+         "    print('returned', cost < naive, flush=True)\n"
+         "except Exception as e:\n"
+         "    print('raised', str(e)[:80], flush=True)\n" % ROOT],
+        stdout=subprocess.PIPE, stderr=subprocess.DEVNULL, text=True)
+    assert child.stdout.readline().strip() == "started"
+    time.sleep(1.5)
+    child.send_signal(getattr(signal, signal_name))
+    t0 = time.time()
+    out, _ = child.communicate(timeout=60)
+    assert time.time() - t0 < 30
+    if signal_name == "SIGINT":
+        assert out.strip() == "returned True", (out, ends)
+    else:
+        assert out.strip().startswith("raised") and "Abort requested" in out, (out, ends)
