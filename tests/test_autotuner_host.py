@@ -166,3 +166,17 @@ def test_signals_during_tuning(signal_name, ends):
         assert out.strip() == "returned True", (out, ends)
     else:
         assert out.strip().startswith("raised") and "Abort requested" in out, (out, ends)
+
+
+def test_fixed_parameters_hold_in_every_candidate_of_a_search():
+    """TuningParameterFixer (tc/autotuner/parameters.h:175-220 in the reference): what the caller
+    fixes is not searched, so the winner carries it whatever else the search finds."""
+    settings = ("generations=3;pop_size=16;threads=1;seed=2;seed_heuristics=0;refinement_rounds=1;"
+                "fix_unroll=4;fix_block=128,2;fix_use_shared_memory=1;fix_match_library_calls=0;fix_vector_width=2")
+    best, cost, naive = model_tune(settings, "c2_tensordot")
+    fields = dict(kv.split("=") for kv in best.split(";"))
+    assert fields["unroll"] == "4" and fields["mapToThreads"] == "128,2" and fields["useSharedMemory"] == "1"
+    assert fields["matchLibraryCalls"] == "0" and fields["vectorWidth"] == "2" and cost <= naive
+    arg_top = settings.replace("generations=3", "generations=2") + ";top_k=3"
+    text = tc.host_query("tune_on_model", arg_top + "|moments|64x512|def moments(float(M, N) X) -> (mean) { mean(m) +=! X(m, r_n) / N }")
+    assert text.startswith("best=")
