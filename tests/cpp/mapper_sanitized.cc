@@ -107,7 +107,7 @@ int main(int argc, char** argv) {
   }
   std::ifstream in(argv[1]);
   std::string entry;
-  size_t mapped = 0, refused = 0, records = 0, damagedMessages = 0, damagedDefinitions = 0, tuned = 0;
+  size_t mapped = 0, refused = 0, records = 0, damagedMessages = 0, damagedDefinitions = 0, tuned = 0, damagedOptionTexts = 0;
   unsigned long long lcg = 88172645463325252ULL;
   while (std::getline(in, entry)) {
     if (entry.empty()) continue;
@@ -173,6 +173,30 @@ int main(int argc, char** argv) {
     }
     while (std::getline(in, line) && line != "@@") {
       if (line.empty()) continue;
+      // damaged option texts must be refused or read as other options
+      for (int round = 0; round < 4; ++round) {
+        lcg = lcg * 6364136223846793005ULL + 1442695040888963407ULL;
+        std::string m = line;
+        size_t at = (lcg >> 33) % m.size();
+        static const char pool[] = ";=,0123456789-+.eEtileMaxnv ";
+        switch ((lcg >> 20) % 4) {
+          case 0: m.erase(at, 1 + (lcg >> 10) % 6); break;
+          case 1: m.insert(at, 1, pool[(lcg >> 12) % (sizeof(pool) - 1)]); break;
+          case 2: m[at] = pool[(lcg >> 12) % (sizeof(pool) - 1)]; break;
+          default: m.insert(at, "99999999999999999999"); break;
+        }
+        char* text2 = nullptr;
+        if (tc_options_normalize(m.c_str(), &text2) == 0) {
+          char* source = nullptr;
+          int kernels = 0;
+          unsigned grids[24], blocks[24];
+          if (tc_map(text.c_str(), entry.c_str(), ptrs.data(), static_cast<int>(ptrs.size()), text2, &source, &kernels, grids, blocks) == 0) {
+            tc_free(source);
+          }
+          tc_free(text2);
+        }
+        ++damagedOptionTexts;
+      }
       // option codecs: text -> normal form -> wire -> text -> C++
       char* normal = nullptr;
       if (tc_options_normalize(line.c_str(), &normal) == 0) {
@@ -223,6 +247,7 @@ int main(int argc, char** argv) {
   }
   std::cout << records << " comprehension(s), " << mapped << " mapping(s), " << refused << " refused, " << damagedMessages
             << " damaged option message(s) and " << damagedFiles << " damaged cache file(s) read, " << damagedDefinitions
-            << " damaged definition(s) parsed, " << tuned << " tuned on the cost model\n";
+            << " damaged definition(s) parsed, " << damagedOptionTexts << " damaged option text(s) read, " << tuned
+            << " tuned on the cost model\n";
   return 0;
 }
