@@ -55,6 +55,20 @@ def corpus():
                 opts = ["naive"]
             opts += [random_tcs.random_options(rng, 4) for _ in range(25)]
             out.append(record(entry, specs, text, opts))
+    # sizes at and beyond the 32-bit limits: 2^31 elements and more (64-bit offsets), a single
+    # extent of 2^31 (refused), products of extents that only fit 64 bits
+    huge = [
+        ("copy", "def copy(int8(N, M) I) -> (O) { O(n, m) = I(n, m) }", [("int8", (65544, 32768))]),
+        ("copy", "def copy(int8(N) I) -> (O) { O(n) = I(n) }", [("int8", (2 ** 31 + 8,))]),
+        ("moments", W.MOMENTS, [("float32", (70000, 40000))]),
+        ("mm", "def mm(float(M, K) A, float(K, N) B) -> (C) { C(m, n) +=! A(m, r_k) * B(r_k, n) }",
+         [("float32", (2 ** 20, 2 ** 11)), ("float32", (2 ** 11, 2 ** 20))]),
+        ("outer", "def outer(float(N) a, float(M) b) -> (O) { O(n, m) = a(n) * b(m) }",
+         [("float32", (2 ** 31 - 1,)), ("float32", (3,))]),
+    ]
+    for entry, text, tensors in huge:
+        out.append(record(entry, [spec(d, sh) for d, sh in tensors], text,
+                          ["naive"] + [random_tcs.random_options(rng, 3) for _ in range(10)]))
     attempt = 0
     drawn = 0
     while drawn < 100:
@@ -81,8 +95,10 @@ def test_host_code_is_clean_under_address_and_undefined_behaviour_sanitizers(tmp
     assert run.returncode == 0, run.stderr[-6000:]
     assert "ERROR: AddressSanitizer" not in run.stderr and "runtime error:" not in run.stderr
     comprehensions, mappings = (int(x) for x in re.findall(r"(\d+) comprehension\(s\), (\d+) mapping", run.stdout)[0])
-    assert comprehensions >= 130 and mappings >= 3000
-    assert "and 300 damaged cache file(s) read" in run.stdout and "13700 damaged definition(s) parsed" in run.stdout
+    assert comprehensions >= 135 and mappings >= 3000
+    assert "and 300 damaged cache file(s) read" in run.stdout
+    assert int(re.findall(r"(\d+) damaged definition\(s\) parsed", run.stdout)[0]) >= 13700
+    assert int(re.findall(r"(\d+) refused", run.stdout)[0]) >= 1          # the single extent of 2^31
     assert int(re.findall(r"(\d+) tuned on the cost model", run.stdout)[0]) >= 15
 
 
