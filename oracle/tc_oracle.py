@@ -614,6 +614,10 @@ class Analysis:
             have = self.tensors[s.lhs].scalar
             if _canon(have) != match_types(scalar, have):
                 raise TcError(f" attempting to assign type {scalar} to narrower type {have} without an explicit cast")
+            # ... and an update definition with another number of arguments (the reference's sema
+            # lets it through, tc/lang/sema.h:566-571)
+            if len(self.tensors[s.lhs].extents) != len(s.indices):
+                raise TcError(f"{s.lhs} was defined with {len(self.tensors[s.lhs].extents)} dimensions and is written here with {len(s.indices)}")
         if s.assign in ("+=", "*=", "min=", "max=") and s.lhs not in self.tensors:
             self.warnings.append(f"Reduction without initialization. If {s.lhs} is not pre-initialized ...")
         if s.lhs not in self.outputs:

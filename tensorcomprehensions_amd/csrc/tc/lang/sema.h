@@ -386,6 +386,15 @@ class Sema {
                                 << " dimensions.";
       }
     }
+    // An earlier statement defined the tensor: this one must write it with as many subscripts.
+    // (The reference's sema lets the mismatch through, tc/lang/sema.h:566-571, and Halide refuses
+    // the update definition afterwards; here nothing behind sema would notice.)
+    if (TreeRef earlier = lookup(env_, stmt.ident(), false)) {
+      if (earlier->kind() == TK_TENSOR_TYPE && TensorType(earlier).dims().size() != stmt.indices().size()) {
+        throw errorAt(stmtTree) << name << " was defined with " << TensorType(earlier).dims().size()
+                                << " dimensions and is written here with " << stmt.indices().size();
+      }
+    }
     if (isPlainReduction(stmt.assignment()->kind()) && !lookup(stmt.ident(), false)) {
       ErrorReport w(stmtTree->range());
       std::string tk = kindToToken(stmt.assignment()->kind());

@@ -171,6 +171,27 @@ def test_a_range_given_empty_is_refused(text, shapes):
         tc_oracle.run(text, "f", [np.zeros(s, np.float32) for s in shapes])
 
 
+def test_a_tensor_is_written_with_the_same_number_of_subscripts_by_every_statement():
+    """`O(i) = ...` followed by `O(j, i) = ...`: the reference's sema keeps the first definition's
+    type and lets the second through (tc/lang/sema.h:566-571; Halide then refuses the update
+    definition).  Here the statement is refused by sema and by the oracle: it used to reach the
+    code generator, which read past the strides of the one-dimensional tensor."""
+    from oracle import tc_oracle
+    text = """def f(float(P, M, M) A, float(Q) B) -> (O0, O1) {
+        O0(i) max=! tanh(A(i, j, k) + B(l))
+        O1(i) = O0(i) * 0.5 + 1
+        O1(j, i) = A(i, j, i) * Q }"""
+    for call in (lambda: tc.infer_output_tensor_info(text, "f", [F(3, 4, 4), F(5)]),
+                 lambda: tc.map_only(text, "f", [F(3, 4, 4), F(5)], "naive")):
+        with pytest.raises(tc.TcError, match="O1 was defined with 1 dimensions and is written here with 2"):
+            call()
+    with pytest.raises(tc_oracle.TcError, match="O1 was defined with 1 dimensions and is written here with 2"):
+        tc_oracle.infer_output_shapes(text, "f", [(3, 4, 4), (5,)])
+    # fewer subscripts than before, and an annotated output
+    with pytest.raises(tc.TcError, match="was defined with 2 dimensions and is written here with 1"):
+        tc.map_only("def g(float(N, M) A) -> (O) { O(n, m) = A(n, m)\n O(n) = A(n, 0) }", "g", [F(4, 5)], "naive")
+
+
 def test_later_statement_cannot_narrow_into_the_tensors_first_type():
     """`O` is int32 by its first definition; accumulating floats into it would be an update
     definition of another type, which the reference's Halide lowering refuses.  The front end and
