@@ -1202,7 +1202,17 @@ class StageCodegen {
       if (cond.empty()) {
         em_.line(target + "[a_] = " + combine(s.op, target + "[a_]", rhs) + ";");
       } else {
-        em_.line("const " + accType_.cName() + " r_ = " + rhs + ";");
+        // A double-precision math routine whose result is combined under a condition: hipcc (ROCm
+        // 7.0 and 7.2, -O1 and up) does not finish compiling `r = tanh(x); if (c) acc = max(acc, r)`
+        // inside these loops; with the value pinned in a register first it compiles in a second.
+        bool mathCall = false;
+        visit(s.rhs, [&](const ExprRef& e) { mathCall |= e->kind == Expr::Call; });
+        if (mathCall && accType_.isFloat() && accType_.bits == 64) {
+          em_.line(accType_.cName() + " r_ = " + rhs + ";");
+          em_.line("asm volatile(\"\" : \"+v\"(r_));");
+        } else {
+          em_.line("const " + accType_.cName() + " r_ = " + rhs + ";");
+        }
         em_.line("if (" + cond + ") " + target + "[a_] = " + combine(s.op, target + "[a_]", "r_") + ";");
       }
       closeN(n);

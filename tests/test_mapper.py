@@ -459,3 +459,20 @@ def test_strided_accesses_are_staged_without_the_elements_jumped_over():
         assert "float lds0_I[1056];" in src                                   # 32 rows of 32 (+1: odd pitch)
         assert f"const int g1_ = lo0_I_1 + l1_ * {step};" in src              # strided read of the tensor
         assert f" - lo0_I_1) / {step}];" in src                                # unit stride in the staged array
+
+
+def test_double_math_results_are_pinned_before_a_conditional_combine():
+    """hipcc (ROCm 7.0 and 7.2) does not finish compiling `r = tanh(x); if (c) acc = max(acc, r)` in
+    double precision inside the reduction loops of a partial tile; the generated code pins the
+    value in a register first (an empty asm), and the definition JIT-compiles in a second."""
+    import time
+    text = """def f(double(P, K) A) -> (O0, O1) {
+        O0(j, i) = A(i, j)
+        O1(i) max=! tanh(O0(i, j)) }"""
+    src, _ = tc.map_only(text, "f", [ShapeOnly((70, 33), "float64")], "naive")
+    assert 'double r_ = tanh(' in src and 'asm volatile("" : "+v"(r_));' in src
+    single, _ = mapped(text.replace("double", "float"), "f", [(70, 33)], "naive")
+    assert 'asm volatile("" : "+v"(r_));' not in single.split('extern "C"', 1)[1]
+    t0 = time.time()
+    tc.compile(text, "f", [tc.ShapeOnly((70, 33), "float64")], "naive")
+    assert time.time() - t0 < 60
