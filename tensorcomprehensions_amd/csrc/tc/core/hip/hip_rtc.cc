@@ -55,10 +55,18 @@ std::unique_ptr<HipRTCFunction> HipRTCFunction::Compile(const std::string& name,
   res->name_ = name;
   std::string arch = HipGPUInfo::GPUInfo().GetArch();
   // Packed-FP32 instruction selection is switched off for all device code of this library.
-  // (-munsafe-fp-atomics: floating-point atomic adds become the hardware instruction; tensors live
-  // in ordinary device memory, for which it is exact)
+  // Kernel arguments (the size parameters and the tensor pointers) arrive in scalar registers
+  // with the wavefront instead of being fetched by its first instructions: the group convolution
+  // of 10 us starts 0.1 us earlier in every wavefront (-amdgpu-kernarg-preload-count, at most 16
+  // dwords; arguments beyond that are loaded as before).
   std::vector<const char*> opts = {"-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-                                   "-munsafe-fp-atomics"};
+                                   "-mllvm", "-amdgpu-kernarg-preload-count=16"};
+  // (-munsafe-fp-atomics, only for programs with a reduction divided among blocks: floating-point
+  // atomic adds become the hardware instruction, which is exact for tensors in ordinary,
+  // coarse-grained device memory and may lose updates in fine-grained or managed allocations)
+  if (source.find("__tc::atomicAccumulate(&") != std::string::npos || source.find("__tc::atomicCombine<") != std::string::npos) {
+    opts.push_back("-munsafe-fp-atomics");
+  }
   if (tc::flags().fast_math) opts.push_back("-ffast-math");
   char* code = nullptr;
   char* log = nullptr;

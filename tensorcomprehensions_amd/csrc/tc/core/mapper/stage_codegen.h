@@ -1545,6 +1545,15 @@ class StageCodegen {
     em_.line("// matrix cores: " + std::to_string(tiles) + " tiles of 16x16 per block, " + std::to_string(ksteps) +
              " steps of v_mfma_f32_16x16x4_f32 each, " + std::to_string(st_.waves) + " wavefront(s)");
     // (the register-resident operand is requested first: its latency overlaps the LDS staging)
+    // Wavefronts that still fetch and stage their operands go ahead of the ones that already
+    // multiply: all blocks of a compute unit start together, the first whose operands arrive fill
+    // the matrix pipeline, and at equal priority the instructions of the others (waits, LDS
+    // stores, the barrier) were issued so rarely that the last block of a compute unit began to
+    // multiply 4 us after the first (per-wavefront timestamps on the 16-channel group convolution).
+    bool stagesOutside = false;
+    for (const auto& p : st_.promotions) stagesOutside |= !p.insideReductionTiles && !p.sharedWithEarlierStage;
+    const bool raisePriority = stagesOutside && !suppressCopy;
+    if (raisePriority) em_.line("__builtin_amdgcn_s_setprio(3);");
     em_.line("const int lm_ = threadIdx.x & 15, lj_ = threadIdx.x >> 4;");
     // Lane group lj_ (0..3) owns a contiguous quarter of the flattened reduction and step ks_
     // walks inside it: when a quarter is a whole number of inner-variable periods, the inner
@@ -1659,6 +1668,8 @@ class StageCodegen {
     // Epilogue operands that do not depend on the column (a bias per output row, say) are the
     // same for every tile of the wavefront: fetched once, ahead of the tile loop.
     hoistedLoads_.clear();
+    size_t hoistedCount = 0;
+    std::vector<std::string> hoistedTexts, hoistedTypes;
     if (resident) {
       std::vector<std::pair<std::string, ExprRef>> invariant;
       for (size_t i = 1; i < st_.stmts.size(); ++i) {
@@ -1692,6 +1703,11 @@ class StageCodegen {
         for (size_t h = 0; h < invariant.size(); ++h) {
           hoistedLoads_[invariant[h].first] = "eh" + std::to_string(h) + "_[r_]";
         }
+        hoistedCount = invariant.size();
+        hoistedTexts.clear();
+        for (const auto& h : invariant) hoistedTexts.push_back(h.first);
+        hoistedTypes.clear();
+        for (const auto& h : invariant) hoistedTypes.push_back(st_.views.at(h.second->name).type.cName());
       }
     }
     // Reduction tiling: the outermost reduction variable may run over several tiles; operands
@@ -1699,7 +1715,47 @@ class StageCodegen {
     // tiles of a wavefront live in registers across it.
     const LoopVar& k0 = var(st_.mfmaK[0]);
     const bool kTiled = k0.numTiles > 1;
-    const int64_t tilesPerWave = ceilDiv(tiles, st_.waves);
+    // Surplus columns.  When the columns of a block tile are not a multiple of 16, the last column
+    // tile of every row tile is mostly padding (196 pixels = 12 tiles + 4 columns).  Up to twelve
+    // surplus columns go through v_mfma_f32_4x4x1_16B_f32 instead, four columns a pass: its 16
+    // blocks are the 4 row quads of the row tile x the 4 quarters of the reduction, so a lane
+    // multiplies the same M-side value as in the 16x16x4 instruction (row lm_, quarter lj_) with
+    // the N-side value of column (lane & 3), and the four partial sums of an output element sit
+    // in the lanes that differ in bits 4 and 5.  A pass costs a quarter of a full tile.
+    const int64_t remCols = NT % 16;
+    const int64_t remPasses = ceilDiv(remCols, 4);
+    bool quarterTiles = !kTiled && split == 1 && remCols != 0 && remPasses <= 3 && s.init &&
+                        stepsPerWave <= kMaxResidentSteps;
+    if (quarterTiles) {
+      // Only where the busiest wavefront gets less to do: units are dealt round-robin, full tiles
+      // first, and a pass is priced at half a tile (a quarter of the multiplications, all of the
+      // operand reads, an exchange between lanes).
+      const int64_t full = BT * numMT * (NT / 16), passes = BT * numMT * remPasses, W = st_.waves;
+      double busiest = 0;
+      for (int64_t w = 0; w < W; ++w) {
+        double cost = 0;
+        for (int64_t u = w; u < full + passes; u += W) cost += u < full ? 1.0 : 0.5;
+        busiest = std::max(busiest, cost);
+      }
+      quarterTiles = busiest < static_cast<double>(ceilDiv(tiles, W));
+    }
+    const int64_t numNTfull = quarterTiles ? NT / 16 : numNT;
+    const int64_t fullTiles = BT * numMT * numNTfull;
+    const int64_t remUnits = quarterTiles ? BT * numMT * remPasses : 0;
+    const int64_t tilesPerWave = ceilDiv(quarterTiles ? fullTiles + remUnits : tiles, st_.waves);
+    // (in a quarter-tile pass lane l finishes rows 4*((l >> 2) & 3) .. +3 of column (l & 3))
+    const std::string quadOfLane = "((threadIdx.x >> 2) & 3)";
+    if (quarterTiles && hoistedCount > 0) {
+      for (size_t h = 0; h < hoistedCount; ++h) em_.line(hoistedTypes[h] + " er" + std::to_string(h) + "_[4];");
+      em_.line("#pragma unroll");
+      em_.open("for (int r_ = 0; r_ < 4; ++r_)");
+      em_.line("const int bt_ = 0, mpos_ = 4 * " + quadOfLane + " + r_;");
+      em_.line("(void)bt_;");
+      if (!st_.mfmaBatch.empty()) decodeGroup(st_.mfmaBatch, "bt_", true);
+      decodeGroup(st_.mfmaM, "mpos_", true);
+      for (size_t h = 0; h < hoistedCount; ++h) em_.line("er" + std::to_string(h) + "_[r_] = " + hoistedTexts[h] + ";");
+      em_.close();
+    }
     auto stagePromotions = [&](bool inside) {
       bool any = false;
       for (const auto& p : st_.promotions) any |= p.insideReductionTiles == inside;
@@ -1715,14 +1771,28 @@ class StageCodegen {
       stageFootprints(inside);
     };
     // decodes the output tile tl_ of this wavefront: batch and column indices, nok_
+    // (columnsCached: the column indices of the unrolled tile j_ were decoded ahead of the staging)
+    bool columnsCached = false;
+    auto cachedColumns = [&]() {
+      for (size_t i = 0; i < st_.mfmaN.size(); ++i) {
+        em_.line("const int " + iv(var(st_.mfmaN[i])) + " = dn" + std::to_string(i) + "_[j_];");
+      }
+      em_.line("const bool nok_ = dok_[j_];");
+      em_.line("(void)nok_;");
+    };
     auto decodeTile = [&]() {
-      em_.line("const int nt_ = tl_ % " + std::to_string(numNT) + ", mt_ = (tl_ / " + std::to_string(numNT) + ") % " +
-               std::to_string(numMT) + ", bt_ = tl_ / " + std::to_string(numNT * numMT) + ";");
+      em_.line("const int nt_ = tl_ % " + std::to_string(numNTfull) + ", mt_ = (tl_ / " + std::to_string(numNTfull) + ") % " +
+               std::to_string(numMT) + ", bt_ = tl_ / " + std::to_string(numNTfull * numMT) + ";");
+      em_.line("(void)nt_;");
       // A row of the product depends on one row of the M-side operand only and a column on one
       // column of the N-side operand, so lanes past the end of a partial tile may load any legal
       // element (clamped indices): their results are never stored.
       std::string bok = st_.mfmaBatch.empty() ? "true" : decodeGroup(st_.mfmaBatch, "bt_", true);
       em_.line("const bool bok_ = " + bok + ";");
+      if (columnsCached) {
+        cachedColumns();
+        return;
+      }
       em_.line("const int npos_ = nt_ * 16 + lm_;");
       em_.line("const bool nok_ = bok_ && " + decodeGroup(st_.mfmaN, "npos_", true) + ";");
       em_.line("(void)nok_;");
@@ -1784,7 +1854,7 @@ class StageCodegen {
     // to legal points, so the epilogue's loads need no guard: the four rows are finished first
     // (their loads issue together and, when they do not depend on the column, move out of the
     // tile loop), then stored under one test of the column.
-    auto finish = [&](const std::string& acc) {
+    auto finish = [&](const std::string& acc, const std::string& columnOk = "nok_") {
       const bool mExact = groupExact(st_.mfmaM, MT, 16);
       em_.line(accType_.cName() + " out_[4];");
       em_.line("#pragma unroll");
@@ -1807,13 +1877,73 @@ class StageCodegen {
       }
       em_.line("out_[r_] = acc_[0];");
       em_.close();
-      em_.open("if (nok_)");
+      em_.open("if (" + columnOk + ")");
       em_.line("#pragma unroll");
       em_.open("for (int r_ = 0; r_ < 4; ++r_)");
       em_.line("const int mpos_ = mt_ * 16 + 4 * lj_ + r_;");
       std::string mok = decodeGroup(st_.mfmaM, "mpos_", true);
       em_.line(storeStmt(mExact ? "true" : mok, "out_[r_]"));
       em_.close();
+      em_.close();
+    };
+    // One quarter-tile pass, unit tl_ - fullTiles of the block: four surplus columns of one row tile.
+    auto decodeQuarter = [&]() {
+      const std::string Q = std::to_string(remPasses);
+      em_.line("const int ru_ = tl_ - " + std::to_string(fullTiles) + ";");
+      em_.line("const int rp_ = ru_ % " + Q + ", mt_ = (ru_ / " + Q + ") % " + std::to_string(numMT) + ", bt_ = ru_ / " +
+               std::to_string(remPasses * numMT) + ";");
+      em_.line("(void)rp_;");
+      std::string bok = st_.mfmaBatch.empty() ? "true" : decodeGroup(st_.mfmaBatch, "bt_", true);
+      em_.line("const bool bok_ = " + bok + ";");
+      if (columnsCached) {
+        cachedColumns();
+        return;
+      }
+      em_.line("const int npos_ = " + std::to_string(numNTfull * 16) + " + 4 * rp_ + (threadIdx.x & 3);");
+      em_.line("const bool nok_ = bok_ && " + decodeGroup(st_.mfmaN, "npos_", true) + ";");
+      em_.line("(void)nok_;");
+    };
+    auto quarterPass = [&]() {
+      decodeQuarter();
+      em_.line("__tc::floatx4 c_;");
+      em_.open("");
+      em_.line("const int mposa_ = mt_ * 16 + lm_;");
+      em_.line("const bool moka_ = bok_ && " + decodeGroup(st_.mfmaM, "mposa_", true) + ";");
+      em_.line("(void)moka_;");
+      em_.line("float bq_[" + std::to_string(ksteps) + "];");
+      if (!resident) em_.line("float aq_[" + std::to_string(ksteps) + "];");
+      bool masked = openSteps(ksteps);
+      if (!resident) em_.line("aq_[ks_] = " + operandValue(loadA, masked) + ";");
+      em_.line("bq_[ks_] = " + operandValue(loadB, masked) + ";");
+      em_.close();
+      // four independent accumulators: a chain of dependent 4x4x1 instructions issues at a third of
+      // the rate of independent ones
+      em_.line("__tc::floatx4 cq_[4];");
+      em_.line("#pragma unroll");
+      em_.line("for (int q_ = 0; q_ < 4; ++q_) cq_[q_] = __tc::floatx4{0.0f, 0.0f, 0.0f, 0.0f};");
+      em_.line("#pragma unroll");
+      em_.open("for (int ks_ = 0; ks_ < " + std::to_string(ksteps) + "; ++ks_)");
+      em_.line(std::string("cq_[ks_ & 3] = __builtin_amdgcn_mfma_f32_4x4x1f32(") + (resident ? "am_" : "aq_") +
+               "[ks_], bq_[ks_], cq_[ks_ & 3], 0, 0, 0);");
+      em_.close();
+      em_.line("c_ = (cq_[0] + cq_[1]) + (cq_[2] + cq_[3]);");
+      // the four quarters of the reduction meet: lanes l, l ^ 16, l ^ 32, l ^ 48
+      em_.line("#pragma unroll");
+      em_.open("for (int r_ = 0; r_ < 4; ++r_)");
+      em_.line("float v_ = c_[r_];");
+      em_.line("v_ += __shfl_xor(v_, 16, 64);");
+      em_.line("v_ += __shfl_xor(v_, 32, 64);");
+      em_.line("c_[r_] = v_;");
+      em_.close();
+      em_.close();
+      // rows of this lane in the quarter-tile layout; the first 16 lanes store
+      em_.open("");
+      em_.line("const int lj_ = " + quadOfLane + ";");
+      em_.line("const bool nokq_ = nok_ && threadIdx.x < 16;");
+      auto saved = hoistedLoads_;
+      for (size_t h = 0; h < hoistedCount; ++h) hoistedLoads_[hoistedTexts[h]] = "er" + std::to_string(h) + "_[r_]";
+      finish("c_", "nokq_");
+      hoistedLoads_ = saved;
       em_.close();
     };
     // Which tile a wavefront works on, who multiplies and who finishes it.  Without a split
@@ -1847,7 +1977,47 @@ class StageCodegen {
     int opened = 0;
     em_.open("");
     ++opened;
+    // Column indices ahead of the staging.  Decoding a column position into the indices of the
+    // N-side variables divides by the tile extents (pixel -> row, column of a 14 x 14 image); for
+    // an unrolled tile loop behind a staging copy that is done for all tiles of the wavefront
+    // while the copy's loads are in flight, and kept (an empty asm pins each value: the compiler
+    // would otherwise move the arithmetic back behind the barrier, into the multiplications).
+    const int64_t unitsAll = quarterTiles ? fullTiles + remUnits : tiles;
+    const bool cacheColumns = raisePriority && !kTiled && split == 1 && tilesPerWave <= 8 && !st_.mfmaN.empty();
+    if (cacheColumns) {
+      const std::string J = std::to_string(tilesPerWave);
+      em_.line(waveRotation);
+      for (size_t i = 0; i < st_.mfmaN.size(); ++i) em_.line("int dn" + std::to_string(i) + "_[" + J + "];");
+      em_.line("bool dok_[" + J + "];");
+      em_.line("#pragma unroll");
+      em_.open("for (int j_ = 0; j_ < " + J + "; ++j_)");
+      em_.line("const int tl_ = wv_ + j_ * " + std::to_string(st_.waves) + ";");
+      for (size_t i = 0; i < st_.mfmaN.size(); ++i) em_.line("dn" + std::to_string(i) + "_[j_] = 0;");
+      em_.line("dok_[j_] = false;");
+      auto keep = [&]() {
+        for (size_t i = 0; i < st_.mfmaN.size(); ++i) {
+          em_.line("dn" + std::to_string(i) + "_[j_] = " + iv(var(st_.mfmaN[i])) + ";");
+        }
+        em_.line("dok_[j_] = nok_;");
+      };
+      if (!quarterTiles || fullTiles > 0) {
+        em_.open("if (tl_ < " + std::to_string(quarterTiles ? fullTiles : tiles) + ")");
+        decodeTile();
+        keep();
+        em_.close();
+      }
+      if (quarterTiles) {
+        em_.open(std::string(fullTiles > 0 ? "else " : "") + "if (tl_ < " + std::to_string(unitsAll) + ")");
+        decodeQuarter();
+        keep();
+        em_.close();
+      }
+      for (size_t i = 0; i < st_.mfmaN.size(); ++i) em_.line("asm volatile(\"\" : \"+v\"(dn" + std::to_string(i) + "_[j_]));");
+      em_.close();
+    }
     stagePromotions(false);
+    columnsCached = cacheColumns;
+    if (raisePriority) em_.line("__builtin_amdgcn_s_setprio(0);");
     if (resident && residentFromLds) fillResident();
     if (!kTiled && split > 1) {
       em_.line(waveRotation);
@@ -1869,7 +2039,8 @@ class StageCodegen {
       gather("c_");
       finish("c_");
     } else if (!kTiled) {
-      em_.line(waveRotation);
+      if (!cacheColumns) em_.line(waveRotation);
+      const int64_t units = unitsAll;
       if (tilesPerWave <= 8) {
         // few tiles per wavefront: unrolled, so that the operand reads of a tile can be scheduled
         // above the epilogue and the stores of the tile before it
@@ -1877,17 +2048,26 @@ class StageCodegen {
         em_.open("for (int j_ = 0; j_ < " + std::to_string(tilesPerWave) + "; ++j_)");
         ++opened;
         em_.line("const int tl_ = wv_ + j_ * " + std::to_string(st_.waves) + ";");
-        em_.open("if (tl_ < " + std::to_string(tiles) + ")");
-        ++opened;
       } else {
-        em_.open("for (int tl_ = wv_; tl_ < " + std::to_string(tiles) + "; tl_ += " + std::to_string(st_.waves) + ")");
+        em_.open("for (int tl_ = wv_; tl_ < " + std::to_string(units) + "; tl_ += " + std::to_string(st_.waves) + ")");
         ++opened;
       }
-      decodeTile();
-      em_.line("__tc::floatx4 c_ = {0.0f, 0.0f, 0.0f, 0.0f};");
-      if (!s.init) loadExisting("c_");
-      multiply("c_");
-      finish("c_");
+      if (!quarterTiles || fullTiles > 0) {
+        em_.open("if (tl_ < " + std::to_string(quarterTiles ? fullTiles : tiles) + ")");
+        decodeTile();
+        em_.line("__tc::floatx4 c_ = {0.0f, 0.0f, 0.0f, 0.0f};");
+        if (!s.init) loadExisting("c_");
+        multiply("c_");
+        finish("c_");
+        em_.close();
+      }
+      if (quarterTiles) {
+        // (the quarter-tile passes continue the round-robin of the full tiles, so they go to the
+        // wavefronts with the fewest full tiles)
+        em_.open(std::string(fullTiles > 0 ? "else " : "") + "if (tl_ < " + std::to_string(units) + ")");
+        quarterPass();
+        em_.close();
+      }
     } else {
       em_.line(waveRotation);
       em_.line("__tc::floatx4 cacc_[" + std::to_string(tilesPerWave) + "];");

@@ -18,7 +18,7 @@ TMM = "def tmm(float(M, K) A, float(N, K) B) -> (C) { C(m, n) +=! A(m, r_k) * B(
 def run(src, entry, ins_np, options, outs_init=None):
     ins = [torch.from_numpy(a).cuda() for a in ins_np]
     ex = tc.compile(src, entry, ins, options)
-    assert "__builtin_amdgcn_mfma_f32_16x16x4f32" in ex.compiled_source
+    assert "__builtin_amdgcn_mfma_f32_" in ex.compiled_source
     outs = tc.prepare_outputs(src, entry, ins)
     for i, o in enumerate(outs):
         if outs_init is not None:
@@ -44,6 +44,40 @@ def test_matmul_shapes_exact(m, k, n, waves):
     assert np.array_equal(C, A @ B)
     (Ct,) = run(TMM, "tmm", [A, np.ascontiguousarray(B.T)], opts)
     assert np.array_equal(Ct, A @ B)
+
+
+# (m, k, n, tile of n, wavefronts, operands through LDS, quarter-tile passes expected)
+QUARTER_CASES = [
+    (16, 8, 20, 32, 1, 0, True), (40, 36, 17, 32, 1, 0, True), (16, 16, 4, 32, 1, 0, True), (16, 16, 4, 32, 4, 1, True),
+    (48, 10, 196, 0, 1, 0, True), (48, 10, 196, 0, 4, 1, True),
+    # not where the busiest wavefront would get more to do, or where the reduction is divided among wavefronts
+    (16, 8, 20, 32, 4, 1, False), (33, 144, 26, 32, 1, 0, False), (33, 144, 26, 32, 4, 1, False), (20, 7, 52, 28, 4, 1, False),
+    (16, 64, 9, 0, 4, 1, False),
+]
+
+
+@pytest.mark.parametrize("m,k,n,tile_n,waves,lds,quarter", QUARTER_CASES)
+def test_surplus_columns_go_through_quarter_tile_passes(m, k, n, tile_n, waves, lds, quarter):
+    """Up to twelve surplus columns of a block tile are multiplied by v_mfma_f32_4x4x1 passes of
+    four columns each (another lane layout for operand, result and epilogue than the 16x16 tiles):
+    bit-exact on integer-valued data, row-wise epilogue operand included."""
+    print(f"quarter tiles {m}x{k}x{n} tile_n={tile_n} waves={waves} lds={lds}", flush=True)
+    src = """
+def mmb(float(M, K) A, float(K, N) B, float(M) bias) -> (C) {
+    C(m, n) +=! A(m, r_k) * B(r_k, n)
+    C(m, n) = C(m, n) + bias(m)
+}
+"""
+    A, B, bias = ints((m, k), m + k), ints((k, n), n + 7), ints((m,), 11)
+    opts = f"naive;tile=16,{tile_n};mapToThreads=64,{waves};mapToBlocks=64,64;useMfma=1;useSharedMemory={lds}"
+    ins = [torch.from_numpy(a).cuda() for a in (A, B, bias)]
+    ex = tc.compile(src, "mmb", ins, opts)
+    assert ("__builtin_amdgcn_mfma_f32_4x4x1f32" in ex.compiled_source) == quarter
+    outs = tc.prepare_outputs(src, "mmb", ins)
+    outs[0].fill_(float("nan"))
+    tc.run(ex, ins, outs)
+    torch.cuda.synchronize()
+    assert np.array_equal(outs[0].cpu().numpy(), A @ B + bias[:, None])
 
 
 def test_matmul_with_lds_operands_and_untiled_problem():
