@@ -114,6 +114,40 @@ class StageCodegen {
     return ss.str();
   }
 
+  // Column sums.  While the body of an unrolled matrix-core tile loop is generated behind a cache
+  // of column indices, the part of an element offset that depends on the N-side variables alone
+  // (14 * i_h + 100352 * i_n + i_w of a store, 16 * i_h + i_w of an LDS read) is replaced by one
+  // value per unrolled tile, ds<k>_[j_], which the pass ahead of the staging copy computes: the
+  // multiplications leave the code behind the barrier.  Each distinct combination of coefficients
+  // gets one such array.
+  bool columnSums_ = false;
+  std::vector<std::string> columnVars_;
+  std::vector<Affine> columnCombos_;
+  std::string columnSumOf(const Affine& part) {
+    for (size_t k = 0; k < columnCombos_.size(); ++k) {
+      bool same = true;
+      for (const auto& n : columnVars_) same &= columnCombos_[k].coefOf(n) == part.coefOf(n);
+      if (same) return "ds" + std::to_string(k) + "_[j_]";
+    }
+    columnCombos_.push_back(part);
+    return "ds" + std::to_string(columnCombos_.size() - 1) + "_[j_]";
+  }
+  // moves the N-side terms of `a` (each scaled by `scale`) into `part`
+  void takeColumnTerms(Affine& a, int64_t scale, Affine& part) const {
+    for (const auto& n : columnVars_) {
+      auto it = a.coef.find(n);
+      if (it == a.coef.end() || it->second == 0) continue;
+      part.coef[n] += it->second * scale;
+      it->second = 0;
+    }
+  }
+  static bool anyTerm(const Affine& a) {
+    for (const auto& c : a.coef) {
+      if (c.second != 0) return true;
+    }
+    return false;
+  }
+
   // --- expressions --------------------------------------------------------------------------
   std::string castTo(const ExprRef& e, const ScalarType& t, const std::string& accRef) {
     std::string s = expr(e, accRef);
@@ -154,6 +188,12 @@ class StageCodegen {
       } else {
         extra += " + " + std::to_string(strides[j]) + " * (" + kc_.idx + ")(" + expr(subs[j], accRef) + ")";
       }
+    }
+    if (columnSums_ && !kc_.wide) {
+      Affine part;
+      part.valid = true;
+      takeColumnTerms(total, 1, part);
+      if (anyTerm(part)) return columnSumOf(part) + " + " + affineStr(total, false) + extra;
     }
     return affineStr(total, kc_.wide) + extra;
   }
@@ -452,9 +492,29 @@ class StageCodegen {
 
   std::string ldsIndex(const Promotion& p, const std::vector<ExprRef>& subs) {
     std::ostringstream ss;
+    std::vector<Affine> forms;
+    for (size_t j = 0; j < subs.size(); ++j) forms.push_back(ir::toAffine(subs[j]));
+    if (columnSums_) {
+      Affine part;
+      part.valid = true;
+      bool ok = true;
+      std::vector<Affine> rest = forms;
+      for (size_t j = 0; j < subs.size(); ++j) {
+        Affine probe;
+        Affine copy = rest[j];
+        takeColumnTerms(copy, 1, probe);
+        if (!anyTerm(probe)) continue;
+        ok &= p.steps[j] == 1; // (a stepped dimension divides the whole difference)
+        takeColumnTerms(rest[j], p.ldsStrides[j], part);
+      }
+      if (ok && anyTerm(part)) {
+        forms = rest;
+        ss << columnSumOf(part) << " + ";
+      }
+    }
     for (size_t j = 0; j < subs.size(); ++j) {
       if (j) ss << " + ";
-      ss << "((" << affineStr(ir::toAffine(subs[j])) << ") - lo" << stageIdx_ << "_" << p.tensor << "_" << j << ")";
+      ss << "((" << affineStr(forms[j]) << ") - lo" << stageIdx_ << "_" << p.tensor << "_" << j << ")";
       if (p.steps[j] != 1) ss << " / " << p.steps[j]; // exact: every access is a whole number of steps from the origin
       if (p.ldsStrides[j] != 1) ss << " * " << p.ldsStrides[j];
     }
@@ -1491,14 +1551,17 @@ class StageCodegen {
   // Declares i_<v> (and p_<v>) for every variable of `group` from the flattened position `pos`
   // inside the block tile (row-major over the group's tile extents, last variable fastest) and
   // returns the predicate "position exists".
-  std::string decodeGroup(const std::vector<std::string>& group, const std::string& pos, bool clamp = false) {
+  // (inRange: the caller knows the position to lie inside the group's tile box; no test, and no
+  // clamp that would keep the compiler from folding the decoded indices into address immediates)
+  std::string decodeGroup(const std::vector<std::string>& group, const std::string& pos, bool clamp = false,
+                          bool inRange = false) {
     int64_t total = 1;
     for (const auto& n : group) total *= var(n).tile;
-    std::string pred = pos + " < " + std::to_string(total);
+    std::string pred = inRange ? std::string("true") : pos + " < " + std::to_string(total);
     // clamped: positions past the end alias the last valid one, so that addresses computed from
     // the decoded indices are always legal (used for operands whose surplus lanes are discarded)
     std::string src = pos;
-    if (clamp) {
+    if (clamp && !inRange) {
       src = "pc" + std::to_string(clampId_++) + "_";
       em_.line("const int " + src + " = min(" + pos + ", " + std::to_string(total - 1) + ");");
     }
@@ -1621,9 +1684,9 @@ class StageCodegen {
       em_.open("");
       em_.line("const int mt_ = 0, bt_ = 0;");
       em_.line("(void)mt_; (void)bt_;");
-      if (!st_.mfmaBatch.empty()) decodeGroup(st_.mfmaBatch, "bt_", true);
+      if (!st_.mfmaBatch.empty()) decodeGroup(st_.mfmaBatch, "bt_", true, true);
       em_.line("const int mposa_ = lm_;");
-      decodeGroup(st_.mfmaM, "mposa_", true);
+      decodeGroup(st_.mfmaM, "mposa_", true, MT % 16 == 0);
       // consecutive steps of a lane read consecutive elements when the operand's reduction
       // subscripts are jointly contiguous: four steps are then fetched with one 16-byte load
       bool contiguous = !residentFromLds && !forwardOf(loadA->name) && aligned && quarter * 4 == KT && ksteps % 4 == 0;
@@ -1694,8 +1757,8 @@ class StageCodegen {
         em_.open("for (int r_ = 0; r_ < 4; ++r_)");
         em_.line("const int bt_ = 0, mpos_ = 4 * lj_ + r_;");
         em_.line("(void)bt_;");
-        if (!st_.mfmaBatch.empty()) decodeGroup(st_.mfmaBatch, "bt_", true);
-        decodeGroup(st_.mfmaM, "mpos_", true);
+        if (!st_.mfmaBatch.empty()) decodeGroup(st_.mfmaBatch, "bt_", true, true);
+        decodeGroup(st_.mfmaM, "mpos_", true, MT % 16 == 0);
         for (size_t h = 0; h < invariant.size(); ++h) {
           em_.line("eh" + std::to_string(h) + "_[r_] = " + invariant[h].first + ";");
         }
@@ -1751,8 +1814,8 @@ class StageCodegen {
       em_.open("for (int r_ = 0; r_ < 4; ++r_)");
       em_.line("const int bt_ = 0, mpos_ = 4 * " + quadOfLane + " + r_;");
       em_.line("(void)bt_;");
-      if (!st_.mfmaBatch.empty()) decodeGroup(st_.mfmaBatch, "bt_", true);
-      decodeGroup(st_.mfmaM, "mpos_", true);
+      if (!st_.mfmaBatch.empty()) decodeGroup(st_.mfmaBatch, "bt_", true, true);
+      decodeGroup(st_.mfmaM, "mpos_", true, MT % 16 == 0);
       for (size_t h = 0; h < hoistedCount; ++h) em_.line("er" + std::to_string(h) + "_[r_] = " + hoistedTexts[h] + ";");
       em_.close();
     }
@@ -1776,6 +1839,7 @@ class StageCodegen {
     auto cachedColumns = [&]() {
       for (size_t i = 0; i < st_.mfmaN.size(); ++i) {
         em_.line("const int " + iv(var(st_.mfmaN[i])) + " = dn" + std::to_string(i) + "_[j_];");
+        em_.line("(void)" + iv(var(st_.mfmaN[i])) + ";");
       }
       em_.line("const bool nok_ = dok_[j_];");
       em_.line("(void)nok_;");
@@ -1787,14 +1851,14 @@ class StageCodegen {
       // A row of the product depends on one row of the M-side operand only and a column on one
       // column of the N-side operand, so lanes past the end of a partial tile may load any legal
       // element (clamped indices): their results are never stored.
-      std::string bok = st_.mfmaBatch.empty() ? "true" : decodeGroup(st_.mfmaBatch, "bt_", true);
+      std::string bok = st_.mfmaBatch.empty() ? "true" : decodeGroup(st_.mfmaBatch, "bt_", true, true);
       em_.line("const bool bok_ = " + bok + ";");
       if (columnsCached) {
         cachedColumns();
         return;
       }
       em_.line("const int npos_ = nt_ * 16 + lm_;");
-      em_.line("const bool nok_ = bok_ && " + decodeGroup(st_.mfmaN, "npos_", true) + ";");
+      em_.line("const bool nok_ = bok_ && " + decodeGroup(st_.mfmaN, "npos_", true, quarterTiles || NT % 16 == 0) + ";");
       em_.line("(void)nok_;");
     };
     // existing output values when the statement accumulates into them
@@ -1810,7 +1874,7 @@ class StageCodegen {
     auto multiply = [&](const std::string& acc) {
       em_.open("");
       em_.line("const int mposa_ = mt_ * 16 + lm_;");
-      em_.line("const bool moka_ = bok_ && " + decodeGroup(st_.mfmaM, "mposa_", true) + ";");
+      em_.line("const bool moka_ = bok_ && " + decodeGroup(st_.mfmaM, "mposa_", true, MT % 16 == 0) + ";");
       em_.line("(void)moka_;");
       // `count` steps of this wavefront
       auto steps = [&](int64_t count) {
@@ -1860,7 +1924,7 @@ class StageCodegen {
       em_.line("#pragma unroll");
       em_.open("for (int r_ = 0; r_ < 4; ++r_)");
       em_.line("const int mpos_ = mt_ * 16 + 4 * lj_ + r_;");
-      decodeGroup(st_.mfmaM, "mpos_", true);
+      decodeGroup(st_.mfmaM, "mpos_", true, MT % 16 == 0);
       em_.line(accType_.cName() + " acc_[1];");
       em_.line("acc_[0] = " + acc + "[r_];");
       outerPred_ = "";
@@ -1881,7 +1945,7 @@ class StageCodegen {
       em_.line("#pragma unroll");
       em_.open("for (int r_ = 0; r_ < 4; ++r_)");
       em_.line("const int mpos_ = mt_ * 16 + 4 * lj_ + r_;");
-      std::string mok = decodeGroup(st_.mfmaM, "mpos_", true);
+      std::string mok = decodeGroup(st_.mfmaM, "mpos_", true, MT % 16 == 0);
       em_.line(storeStmt(mExact ? "true" : mok, "out_[r_]"));
       em_.close();
       em_.close();
@@ -1893,14 +1957,14 @@ class StageCodegen {
       em_.line("const int rp_ = ru_ % " + Q + ", mt_ = (ru_ / " + Q + ") % " + std::to_string(numMT) + ", bt_ = ru_ / " +
                std::to_string(remPasses * numMT) + ";");
       em_.line("(void)rp_;");
-      std::string bok = st_.mfmaBatch.empty() ? "true" : decodeGroup(st_.mfmaBatch, "bt_", true);
+      std::string bok = st_.mfmaBatch.empty() ? "true" : decodeGroup(st_.mfmaBatch, "bt_", true, true);
       em_.line("const bool bok_ = " + bok + ";");
       if (columnsCached) {
         cachedColumns();
         return;
       }
       em_.line("const int npos_ = " + std::to_string(numNTfull * 16) + " + 4 * rp_ + (threadIdx.x & 3);");
-      em_.line("const bool nok_ = bok_ && " + decodeGroup(st_.mfmaN, "npos_", true) + ";");
+      em_.line("const bool nok_ = bok_ && " + decodeGroup(st_.mfmaN, "npos_", true, remCols % 4 == 0) + ";");
       em_.line("(void)nok_;");
     };
     auto quarterPass = [&]() {
@@ -1908,7 +1972,7 @@ class StageCodegen {
       em_.line("__tc::floatx4 c_;");
       em_.open("");
       em_.line("const int mposa_ = mt_ * 16 + lm_;");
-      em_.line("const bool moka_ = bok_ && " + decodeGroup(st_.mfmaM, "mposa_", true) + ";");
+      em_.line("const bool moka_ = bok_ && " + decodeGroup(st_.mfmaM, "mposa_", true, MT % 16 == 0) + ";");
       em_.line("(void)moka_;");
       em_.line("float bq_[" + std::to_string(ksteps) + "];");
       if (!resident) em_.line("float aq_[" + std::to_string(ksteps) + "];");
@@ -1980,23 +2044,73 @@ class StageCodegen {
     // Column indices ahead of the staging.  Decoding a column position into the indices of the
     // N-side variables divides by the tile extents (pixel -> row, column of a 14 x 14 image); for
     // an unrolled tile loop behind a staging copy that is done for all tiles of the wavefront
-    // while the copy's loads are in flight, and kept (an empty asm pins each value: the compiler
-    // would otherwise move the arithmetic back behind the barrier, into the multiplications).
+    // while the copy's loads are in flight, together with the N-side part of every element offset
+    // (columnSumOf), and kept: an empty asm pins each value, the compiler would otherwise move the
+    // arithmetic back behind the barrier, between the multiplications.  The code behind this point
+    // is generated first, since it tells which sums it needs, and is appended to the pass.
     const int64_t unitsAll = quarterTiles ? fullTiles + remUnits : tiles;
     const bool cacheColumns = raisePriority && !kTiled && split == 1 && tilesPerWave <= 8 && !st_.mfmaN.empty();
+    std::string headText;
+    int headIndent = 0;
     if (cacheColumns) {
-      const std::string J = std::to_string(tilesPerWave);
       em_.line(waveRotation);
+      headText = em_.out.str();
+      em_.out.str("");
+      em_.out.clear();
+      headIndent = em_.indent;
+    }
+    stagePromotions(false);
+    columnsCached = cacheColumns;
+    if (cacheColumns) {
+      columnSums_ = true;
+      columnVars_ = st_.mfmaN;
+      columnCombos_.clear();
+    }
+    if (raisePriority) em_.line("__builtin_amdgcn_s_setprio(0);");
+    auto emitColumnPass = [&]() {
+      const std::string body = em_.out.str();
+      const int tailIndent = em_.indent;
+      em_.out.str("");
+      em_.out.clear();
+      em_.out << headText;
+      em_.indent = headIndent;
+      columnSums_ = false;
+      columnsCached = false;
+      // an index variable the body names outside its own declarations is handed over as well
+      std::vector<bool> indexUsed;
+      for (const auto& n : st_.mfmaN) {
+        const std::string name = iv(var(n));
+        size_t uses = 0, decls = 0;
+        for (size_t at = body.find(name); at != std::string::npos; at = body.find(name, at + 1)) {
+          const bool startsWord = at == 0 || !(std::isalnum(static_cast<unsigned char>(body[at - 1])) || body[at - 1] == '_');
+          const size_t end = at + name.size();
+          const bool endsWord = end >= body.size() || !(std::isalnum(static_cast<unsigned char>(body[end])) || body[end] == '_');
+          if (!startsWord || !endsWord) continue;
+          ++uses;
+          // (its declaration from the cache and the cast that keeps an unused one quiet do not count)
+          if (body.compare(end, 5, " = dn") == 0) ++decls;
+          if (at >= 6 && body.compare(at - 6, 6, "(void)") == 0) ++decls;
+        }
+        indexUsed.push_back(uses > decls);
+      }
+      const std::string J = std::to_string(tilesPerWave);
       for (size_t i = 0; i < st_.mfmaN.size(); ++i) em_.line("int dn" + std::to_string(i) + "_[" + J + "];");
+      for (size_t k = 0; k < columnCombos_.size(); ++k) em_.line("int ds" + std::to_string(k) + "_[" + J + "];");
       em_.line("bool dok_[" + J + "];");
       em_.line("#pragma unroll");
       em_.open("for (int j_ = 0; j_ < " + J + "; ++j_)");
       em_.line("const int tl_ = wv_ + j_ * " + std::to_string(st_.waves) + ";");
       for (size_t i = 0; i < st_.mfmaN.size(); ++i) em_.line("dn" + std::to_string(i) + "_[j_] = 0;");
+      for (size_t k = 0; k < columnCombos_.size(); ++k) em_.line("ds" + std::to_string(k) + "_[j_] = 0;");
       em_.line("dok_[j_] = false;");
       auto keep = [&]() {
         for (size_t i = 0; i < st_.mfmaN.size(); ++i) {
-          em_.line("dn" + std::to_string(i) + "_[j_] = " + iv(var(st_.mfmaN[i])) + ";");
+          if (indexUsed[i]) em_.line("dn" + std::to_string(i) + "_[j_] = " + iv(var(st_.mfmaN[i])) + ";");
+        }
+        for (size_t k = 0; k < columnCombos_.size(); ++k) {
+          Affine a = columnCombos_[k];
+          a.constant = 0;
+          em_.line("ds" + std::to_string(k) + "_[j_] = " + affineStr(a) + ";");
         }
         em_.line("dok_[j_] = nok_;");
       };
@@ -2012,12 +2126,16 @@ class StageCodegen {
         keep();
         em_.close();
       }
-      for (size_t i = 0; i < st_.mfmaN.size(); ++i) em_.line("asm volatile(\"\" : \"+v\"(dn" + std::to_string(i) + "_[j_]));");
+      for (size_t i = 0; i < st_.mfmaN.size(); ++i) {
+        if (indexUsed[i]) em_.line("asm volatile(\"\" : \"+v\"(dn" + std::to_string(i) + "_[j_]));");
+      }
+      for (size_t k = 0; k < columnCombos_.size(); ++k) em_.line("asm volatile(\"\" : \"+v\"(ds" + std::to_string(k) + "_[j_]));");
       em_.close();
-    }
-    stagePromotions(false);
-    columnsCached = cacheColumns;
-    if (raisePriority) em_.line("__builtin_amdgcn_s_setprio(0);");
+      em_.out << body;
+      em_.indent = tailIndent;
+      columnCombos_.clear();
+      columnVars_.clear();
+    };
     if (resident && residentFromLds) fillResident();
     if (!kTiled && split > 1) {
       em_.line(waveRotation);
@@ -2171,6 +2289,7 @@ class StageCodegen {
     closeN(opened);
     // inside loops the partial tiles are written again: not before every owner has read them
     if (split > 1 && (kc_.kernelLoops || stageTileLoops_)) em_.line("__syncthreads();");
+    if (cacheColumns) emitColumnPass();
     hoistedLoads_.clear();
     for (const auto& p : st_.promotions) activePromotions_.erase(p.tensor);
   }
