@@ -50,6 +50,23 @@ def flops(name, shapes):
 
 
 SPIN_MS = 150.0
+# Options cache written by the autotuner (`--tune ... --save-cache`), compcache wire format; the
+# backend adds ".hip" to the name (HipBackend::makeDeviceFilename).
+OPTIONS_CACHE = os.path.join(ROOT, "tensorcomprehensions_amd", "tuned", "benchmark_configs")
+MIN_BURST = 200                # launches per timed burst of the workloads beside the headline one
+
+
+def stored_options(name, ins):
+    """The mapping options a workload is timed under: the best entry the autotuner recorded for
+    this TC and these input sizes in the committed options cache; the tuner's base mapping of
+    tests/workloads.py when the cache has none.  Returns (options text, where they came from)."""
+    import tensorcomprehensions_amd as tc
+    from tests import workloads as W
+    src, entry = W.CONFIGS[name][0], W.CONFIGS[name][1]
+    best = tc.load_from_cache(src, entry, ins, OPTIONS_CACHE, 1)
+    if best:
+        return best[0].to_text(), "autotuner's options cache " + os.path.relpath(OPTIONS_CACHE + ".hip", ROOT)
+    return W.TUNED[name], "tests/workloads.py:TUNED (no entry in the options cache)"
 
 
 def spin(ex, ins, outs, ms):
@@ -94,7 +111,7 @@ def measure(name, steps, warmup, options=None, bursts=1):
 
     src, entry, shapes, _, _ = W.CONFIGS[name]
     ins = [to_device(a) for a in W.make_inputs(name)]
-    opts = options or W.TUNED[name]
+    opts, opts_from = (options, "command line or this run's tuning") if options else stored_options(name, ins)
     ex = tc.compile(src, entry, ins, opts)
     outs = tc.prepare_outputs(src, entry, ins)
     spin(ex, ins, outs, SPIN_MS)
@@ -106,15 +123,17 @@ def measure(name, steps, warmup, options=None, bursts=1):
     device_us = tc.profile_repeated(ex, ins, outs, steps)
     device_sync()
     wall = time.perf_counter() - t0
-    if bursts > 1:
-        # (the workloads beside the headline one: the median of several such bursts, since K launches
-        # of a kernel of a few microseconds are over before the figure has settled)
-        more = [device_us] + [tc.profile_repeated(ex, ins, outs, steps) for _ in range(bursts - 1)]
-        device_us = sorted(more)[len(more) // 2]
     kernel_ms = device_us / 1e3 / steps
+    if bursts > 1:
+        # (the workloads beside the headline one: the median of several bursts of at least MIN_BURST
+        # launches each, since K launches of a kernel of a few microseconds are over before the
+        # figure has settled)
+        n = max(steps, MIN_BURST)
+        more = [tc.profile_repeated(ex, ins, outs, n) / n for _ in range(bursts)]
+        kernel_ms = sorted(more)[len(more) // 2] / 1e3
     nbytes = algorithmic_bytes(src, entry, ins)
     return {
-        "name": name, "options": opts, "wall_s": wall, "kernel_ms": kernel_ms, "bytes": nbytes,
+        "name": name, "options": opts, "options_from": opts_from, "wall_s": wall, "kernel_ms": kernel_ms, "bytes": nbytes,
         "flops": flops(name, shapes), "launch": [ex.launch_bounds(k) for k in range(ex.num_kernels)],
         "ins": ins, "outs": outs,
     }
@@ -136,7 +155,7 @@ def calibrate_copy(steps):
     sys.stderr.write(f"copy calibration: {2 * 4 * COPY_ELEMS / us / 1e3:.1f} GB/s, {us:.1f} us per launch\n")
 
 
-def launch_floor(steps):
+def launch_floor(steps, all_shapes=True):
     """Per-launch time of copy kernels that do next to nothing, issued back to back like the
     workloads (one wavefront; 64 and 500 blocks of 256 threads, 4 KiB each): what a launch costs
     on this device whatever the kernel does.  The 3 us workloads are to be read against it."""
@@ -146,12 +165,14 @@ def launch_floor(steps):
     for label, n, opts in [("copy_1_block_of_64", 64, "naive;mapToThreads=64;mapToBlocks=1;tile=64"),
                            ("copy_64_blocks_of_256", 64 * 1024, "naive;mapToThreads=256;mapToBlocks=64;tile=1024;vectorWidth=4"),
                            ("copy_500_blocks_of_256", 500 * 1024, "naive;mapToThreads=256;mapToBlocks=500;tile=1024;vectorWidth=4")]:
+        if not all_shapes and label != "copy_500_blocks_of_256":
+            continue
         src = to_device(np.ones(n, dtype=np.float32))
         ex = tc.compile(COPY_TC, "copy", [src], opts)
         (dst,) = tc.prepare_outputs(COPY_TC, "copy", [src])
         spin(ex, [src], [dst], SPIN_MS)
-        out[label] = {"us_per_launch": round(tc.profile_repeated(ex, [src], [dst], steps) / steps, 3),
-                      "kernel": ex.kernel_name(), "launch": ex.launch_bounds()}
+        us = sorted(tc.profile_repeated(ex, [src], [dst], steps) / steps for _ in range(5))[2]
+        out[label] = {"us_per_launch": round(us, 3), "kernel": ex.kernel_name(), "launch": ex.launch_bounds()}
     return out
 
 
@@ -210,6 +231,19 @@ def measured_traffic(name, options):
         if line.startswith("traffic_bytes_per_launch:"):
             return int(line.split(":")[1])
     return None
+
+
+def with_floor(roof, kernel_us, floor_us):
+    """A kernel of a few microseconds next to what an empty launch costs on this device:
+    floor_us = a near-empty copy kernel launched the same way, above_floor_us = the kernel's time
+    minus that, frac_above_floor = the kernel's ideal time at the roofline / above_floor_us."""
+    ideal_us = roof["frac"] * kernel_us
+    above = kernel_us - floor_us
+    roof["floor_us"] = round(floor_us, 3)
+    roof["above_floor_us"] = round(above, 3)
+    # (capped: a kernel whose time cannot be told from an empty launch's has hidden its work behind the launch)
+    roof["frac_above_floor"] = round(min(1.0, ideal_us / above), 4) if above > 0 else 1.0
+    return roof
 
 
 def roofline(m):
@@ -364,6 +398,10 @@ def main():
                     help="back-to-back launches for this long before the warm-up steps (device clocks)")
     ap.add_argument("--tune", default=None, metavar="GENERATIONSxPOPULATION",
                     help="autotune the workload from the naive options first (e.g. 5x40) and measure the best")
+    ap.add_argument("--tune-base", default="naive", choices=["naive", "stored"],
+                    help="base mapping of --tune: the naive options, or the base mapping of tests/workloads.py")
+    ap.add_argument("--save-cache", action="store_true",
+                    help="--tune reads and extends the committed options cache (tensorcomprehensions_amd/tuned/)")
     ap.add_argument("--tune-settings", default="", metavar="KEY=VALUE;...",
                     help="further tuner settings for --tune (seed_heuristics=0, refinement_rounds=0, seed=3, ...)")
     ap.add_argument("--suite", action="store_true",
@@ -393,8 +431,11 @@ def main():
         ins = [to_device(x) for x in W.make_inputs(a.config)]
         t0 = time.perf_counter()
         settings = {"generations": gens, "pop_size": pop, "threads": 16, "seed": 1, "top_k": 1}
+        if a.save_cache:
+            os.makedirs(os.path.dirname(OPTIONS_CACHE), exist_ok=True)
+            settings["cache_file"] = OPTIONS_CACHE
         settings.update(kv.split("=", 1) for kv in a.tune_settings.split(";") if kv)
-        best = tc.autotune(src, entry, ins, "naive", **settings)
+        best = tc.autotune(src, entry, ins, "naive" if a.tune_base == "naive" else W.TUNED[a.config], **settings)
         tuned_in = time.perf_counter() - t0
         if not best:
             sys.exit("the autotuner found no runnable candidate")
@@ -412,24 +453,32 @@ def main():
         "roofline": roofline(m),
         "device": tc.device_name(),
     }
+    line["config"]["options_from"] = m["options_from"]
     if tuned_in is not None:
-        line["config"]["options_from"] = (f"autotuned from the naive options, {a.tune} candidates, {tuned_in:.0f} s"
+        line["config"]["options_from"] = (f"autotuned from the {a.tune_base} options, {a.tune} candidates, {tuned_in:.0f} s"
                                           + (f", {a.tune_settings}" if a.tune_settings else ""))
     if not a.no_cpu:
         line["cpu_baseline"] = cpu_baseline(a.config, m["bytes"])
         line["cpu_baseline"]["host_cores"] = os.cpu_count()
         line["cpu_baseline"]["aten"] = aten_cpu_baseline(a.config, m["bytes"])
+    # what a launch costs whatever the kernel does: part of every line, the workloads of a few
+    # microseconds are read against it (--floor adds the one-wavefront and 64-block shapes)
+    floor = launch_floor(max(a.steps, MIN_BURST), all_shapes=a.floor)
+    line["launch_floor"] = floor
+    floor_us = floor["copy_500_blocks_of_256"]["us_per_launch"]
     if not a.only:
         others = {}
         for name in W.CONFIGS:
             if name == a.config:
                 continue
             o = measure(name, a.steps, a.warmup, bursts=7)
-            others[name] = {"kernel_us": round(o["kernel_ms"] * 1e3, 3), "roofline": roofline(o),
-                            "gflops": round(o["flops"] / (o["kernel_ms"] * 1e-3) / 1e9, 1), "launch": o["launch"]}
+            roof = roofline(o)
+            if o["kernel_ms"] * 1e3 < 4 * floor_us:
+                roof = with_floor(roof, o["kernel_ms"] * 1e3, floor_us)
+            others[name] = {"kernel_us": round(o["kernel_ms"] * 1e3, 3), "roofline": roof,
+                            "gflops": round(o["flops"] / (o["kernel_ms"] * 1e-3) / 1e9, 1), "launch": o["launch"],
+                            "options": o["options"], "options_from": o["options_from"]}
         line["others"] = others
-    if a.floor:
-        line["launch_floor"] = launch_floor(a.steps)
     if a.stream:
         line["stream_probes"] = stream_probes(a.steps)
     if a.suite:

@@ -51,7 +51,7 @@ def lib():
     if _lib is None:
         if not os.path.exists(_LIB_PATH):
             raise ImportError(
-                f"{_LIB_PATH} is missing: build it with `make -C {os.path.join(_HERE, 'csrc')}` "
+                f"{_LIB_PATH} is missing: build it with `make -C {os.path.join(_HERE, 'csrc')} libs` "
                 "(or python -c 'import __graft_entry__ as g; g.build()')")
         _lib = ctypes.CDLL(_LIB_PATH, mode=ctypes.RTLD_GLOBAL)
         _declare(_lib)

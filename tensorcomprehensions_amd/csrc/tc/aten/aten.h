@@ -17,8 +17,8 @@ inline DLDataType toDLDataType(const at::Tensor& t) {
   d.lanes = 1;
   d.bits = static_cast<uint8_t>(t.element_size() * 8);
   switch (t.scalar_type()) {
-    case at::kFloat: case at::kDouble: d.code = kDLFloat; break;
-    case at::kByte: case at::kBool: d.code = kDLUInt; break;
+    case at::kFloat: case at::kDouble: case at::kHalf: d.code = kDLFloat; break;
+    case at::kByte: case at::kBool: case at::kUInt16: case at::kUInt32: case at::kUInt64: d.code = kDLUInt; break;
     case at::kChar: case at::kShort: case at::kInt: case at::kLong: d.code = kDLInt; break;
     default: TC_CHECK(false) << "unsupported ATen scalar type";
   }
@@ -26,8 +26,11 @@ inline DLDataType toDLDataType(const at::Tensor& t) {
 }
 
 inline at::ScalarType toScalarType(const DLDataType& d) {
-  if (d.code == kDLFloat) return d.bits == 64 ? at::kDouble : at::kFloat;
-  if (d.code == kDLUInt) return at::kByte;
+  if (d.code == kDLFloat) return d.bits == 64 ? at::kDouble : d.bits == 16 ? at::kHalf : at::kFloat;
+  if (d.code == kDLUInt) {
+    // (a TC `bool` is an 8-bit unsigned value on the device, like uint8)
+    return d.bits == 64 ? at::kUInt64 : d.bits == 32 ? at::kUInt32 : d.bits == 16 ? at::kUInt16 : at::kByte;
+  }
   switch (d.bits) {
     case 8: return at::kChar;
     case 16: return at::kShort;

@@ -14,7 +14,8 @@ namespace aten {
 template <typename Backend, typename Search>
 class ATenAutotuner : public tc::autotune::Autotuner<Backend, Search> {
  public:
-  using MappingOptionsType = typename Backend::MappingOptionsType;
+  using BackendType = Backend;
+  using MappingOptionsType = typename BackendType::MappingOptionsType;
 
   explicit ATenAutotuner(const std::string& tc) : tc_(tc) {}
 
@@ -37,8 +38,10 @@ class ATenAutotuner : public tc::autotune::Autotuner<Backend, Search> {
         tc_, tcEntryPoint, inMap, outMap, baseMappings, topK, fixedParams, settings);
   }
 
- private:
-  std::string tc_;
+ protected:
+  // (kept so that one tuner serves every function of the text; subclasses read it, as in the
+  // reference, tc/aten/aten_autotuner.h:86-90)
+  const std::string tc_;
 };
 
 } // namespace aten

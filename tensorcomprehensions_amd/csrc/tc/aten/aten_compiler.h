@@ -14,10 +14,16 @@
 namespace tc {
 namespace aten {
 
-inline std::vector<TensorInfo> inferOutputTensorInfo(
+// The (contiguous) output shapes as metadata-owning DLTensors without data, as the reference
+// returns them (tc/aten/aten_compiler.h:35-38): infos[0]->shape[0], ->ndim, ->dtype.
+inline std::vector<tc::DLTensorUPtr> inferOutputTensorInfo(
     const std::string& tc, const std::string& entryPoint, const std::vector<at::Tensor>& inputs) {
   auto in = makeDLConstTensors(inputs);
-  return tc::inferOutputTensorInfo(tc, entryPoint, extractRawPtrs(in));
+  std::vector<tc::DLTensorUPtr> out;
+  for (const auto& info : tc::inferOutputTensorInfo(tc, entryPoint, extractRawPtrs(in))) {
+    out.push_back(makeDLTensor<DLTensor>(info));
+  }
+  return out;
 }
 
 // Uninitialised outputs on the device (and with the options) of inputs[0].
@@ -26,7 +32,8 @@ inline std::vector<at::Tensor> prepareOutputs(
   TC_CHECK_GE(inputs.size(), 1u) << "NYI: Need >0 inputs to determine the backend for the outputs";
   std::vector<at::Tensor> outputs;
   for (const auto& info : inferOutputTensorInfo(tc, entryPoint, inputs)) {
-    outputs.push_back(at::empty(info.shape, inputs[0].options().dtype(toScalarType(info.dtype))));
+    std::vector<int64_t> shape(info->shape, info->shape + info->ndim);
+    outputs.push_back(at::empty(shape, inputs[0].options().dtype(toScalarType(info->dtype))));
   }
   return outputs;
 }

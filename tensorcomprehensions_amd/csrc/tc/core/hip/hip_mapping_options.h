@@ -187,11 +187,12 @@ class HipMappingOptions : public GenericOptionsFluent<HipMappingOptions> {
         case 8: useReadOnlyCacheValue = r.value() != 0; break;
         case 9: hasPrivateDepth = true; privateDepthValue = static_cast<uint32_t>(r.value()); break;
         case 10: hasSharedDepth = true; sharedDepthValue = static_cast<uint32_t>(r.value()); break;
-        case 11: vectorWidthValue = static_cast<uint32_t>(r.value()); break;
+        // (through the setters: a foreign or damaged file must not plant a value the text form refuses)
+        case 11: vectorWidth(static_cast<uint32_t>(std::min<uint64_t>(r.value(), 1u << 20))); break;
         case 12: collapseContiguousValue = r.value() != 0; break;
         case 13: useMfmaValue = r.value() != 0; break;
         case 14: prefetchSharedValue = r.value() != 0; break;
-        case 15: reductionBlocksValue = static_cast<uint32_t>(r.value()); break;
+        case 15: reductionBlocks(static_cast<uint32_t>(std::min<uint64_t>(r.value(), 1u << 20))); break;
         default: break;
       }
     }

@@ -35,7 +35,7 @@ HipRTCFunction::~HipRTCFunction() {
 }
 
 void HipRTCFunction::clear() {
-  std::lock_guard<std::mutex> lock(mutex_);
+  std::unique_lock<std::shared_mutex> lock(mutex_);
   if (cleared_) return;
   for (auto& m : modules_) {
     int old = 0;
@@ -95,25 +95,42 @@ Duration HipRTCFunction::Launch(
   int dev = 0;
   TC_HIP_CHECK(tchip_get_device(&dev));
   std::vector<tchip_function_t> fns;
-  {
-    // the per-device module and function handles are filled in lazily: one thread at a time
-    std::lock_guard<std::mutex> lock(mutex_);
-    TC_CHECK(!cleared_) << "launch of a cleared RTC function";
-    if (!modules_.count(dev)) {
-      tchip_module_t m = nullptr;
-      TC_HIP_CHECK(tchip_module_load(code_.data(), &m));
-      modules_[dev] = m;
-    }
+  // every handle of this launch, if all of them are there (call with the lock held)
+  auto lookUp = [&]() {
+    fns.clear();
+    if (!modules_.count(dev)) return false;
     for (const auto& k : kernels) {
-      auto key = std::make_pair(dev, k.name);
-      auto it = functions_.find(key);
-      if (it == functions_.end()) {
-        tchip_function_t fn = nullptr;
-        TC_HIP_CHECK(tchip_module_get_function(modules_[dev], k.name.c_str(), &fn));
-        it = functions_.emplace(key, fn).first;
-      }
+      auto it = functions_.find(std::make_pair(dev, k.name));
+      if (it == functions_.end()) return false;
       fns.push_back(it->second);
     }
+    return true;
+  };
+  std::shared_lock<std::shared_mutex> launching(mutex_);
+  TC_CHECK(!cleared_) << "launch of a cleared RTC function";
+  if (!lookUp()) {
+    // the per-device module and function handles are filled in lazily: one thread at a time
+    launching.unlock();
+    {
+      std::unique_lock<std::shared_mutex> loading(mutex_);
+      TC_CHECK(!cleared_) << "launch of a cleared RTC function";
+      if (!modules_.count(dev)) {
+        tchip_module_t m = nullptr;
+        TC_HIP_CHECK(tchip_module_load(code_.data(), &m));
+        modules_[dev] = m;
+      }
+      for (const auto& k : kernels) {
+        auto key = std::make_pair(dev, k.name);
+        if (!functions_.count(key)) {
+          tchip_function_t fn = nullptr;
+          TC_HIP_CHECK(tchip_module_get_function(modules_[dev], k.name.c_str(), &fn));
+          functions_.emplace(key, fn);
+        }
+      }
+    }
+    launching.lock();
+    // (a clear() may have run in between: then the launch is refused, never made on stale handles)
+    TC_CHECK(!cleared_ && lookUp()) << "launch of a cleared RTC function";
   }
   std::vector<void*> args;
   for (auto& p : params) args.push_back(&p);

@@ -7,6 +7,7 @@
 #include <map>
 #include <memory>
 #include <mutex>
+#include <shared_mutex>
 #include <string>
 #include <vector>
 
@@ -47,7 +48,10 @@ class HipRTCFunction {
   HipRTCFunction() = default;
   std::string name_;
   std::string code_; // code object
-  mutable std::mutex mutex_;                                                   // guards the two maps
+  // guards the two maps: launches hold it shared from the lookup of their handles to the end of
+  // their launch calls, clear() and the lazy loading hold it exclusively, so a module is never
+  // unloaded between a lookup and the launch that uses it
+  mutable std::shared_mutex mutex_;
   mutable std::map<int, tchip_module_t> modules_;                              // per device id
   mutable std::map<std::pair<int, std::string>, tchip_function_t> functions_;  // (device, kernel)
   bool cleared_ = false;

@@ -1262,12 +1262,12 @@ class StageCodegen {
       if (cond.empty()) {
         em_.line(target + "[a_] = " + combine(s.op, target + "[a_]", rhs) + ";");
       } else {
-        // A double-precision math routine whose result is combined under a condition: hipcc (ROCm
-        // 7.0 and 7.2, -O1 and up) does not finish compiling `r = tanh(x); if (c) acc = max(acc, r)`
-        // inside these loops; with the value pinned in a register first it compiles in a second.
-        bool mathCall = false;
-        visit(s.rhs, [&](const ExprRef& e) { mathCall |= e->kind == Expr::Call; });
-        if (mathCall && accType_.isFloat() && accType_.bits == 64) {
+        // A double-precision value combined under a condition: hipcc (ROCm 7.0 and 7.2, -O1 and
+        // up) does not finish compiling `r = tanh(x); if (c) acc = max(acc, r)` inside these loops;
+        // with the value pinned in a register first it compiles in a second.  Every conditional
+        // combine in double precision is pinned, whatever computes the value: the JIT has no
+        // time limit, a second trigger of the defect would block compile() for good.
+        if (accType_.isFloat() && accType_.bits == 64) {
           em_.line(accType_.cName() + " r_ = " + rhs + ";");
           em_.line("asm volatile(\"\" : \"+v\"(r_));");
         } else {

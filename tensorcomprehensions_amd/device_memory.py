@@ -20,7 +20,7 @@ def _tchip():
     if _hip is None:
         path = os.path.join(_HERE, "libtchip.so")
         if not os.path.exists(path):
-            raise ImportError(f"{path} is missing: build it with `make -C {os.path.join(_HERE, 'csrc')}`")
+            raise ImportError(f"{path} is missing: build it with `make -C {os.path.join(_HERE, 'csrc')} libs`")
         _hip = ctypes.CDLL(path, mode=ctypes.RTLD_GLOBAL)
         _hip.tchip_malloc.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_size_t]
         _hip.tchip_free_device.argtypes = [ctypes.c_void_p]

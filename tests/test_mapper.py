@@ -473,6 +473,13 @@ def test_double_math_results_are_pinned_before_a_conditional_combine():
     assert 'double r_ = tanh(' in src and 'asm volatile("" : "+v"(r_));' in src
     single, _ = mapped(text.replace("double", "float"), "f", [(70, 33)], "naive")
     assert 'asm volatile("" : "+v"(r_));' not in single.split('extern "C"', 1)[1]
+    # the JIT step in a child process under a time limit: a recurrence of the defect fails this
+    # test instead of hanging the suite (hipRTC needs no device)
+    import os, subprocess, sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = (f"import sys; sys.path.insert(0, {root!r}); import tensorcomprehensions_amd as tc; "
+            f"tc.compile({text!r}, 'f', [tc.ShapeOnly((70, 33), 'float64')], 'naive'); print('compiled')")
     t0 = time.time()
-    tc.compile(text, "f", [tc.ShapeOnly((70, 33), "float64")], "naive")
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0 and "compiled" in r.stdout, r.stderr[-2000:]
     assert time.time() - t0 < 60

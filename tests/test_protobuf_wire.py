@@ -170,6 +170,25 @@ def test_packed_repeated_fields_are_accepted():
     assert "tile=3,5,7" in from_serialized(bytes(grown)).split(";")
 
 
+@pytest.mark.parametrize("field,value,message", [(15, 0, "reductionBlocks must be between 1 and 1024"),
+                                                  (15, 5000, "reductionBlocks must be between 1 and 1024"),
+                                                  (11, 3, "vector width must be 1, 2 or 4")])
+def test_out_of_range_scalars_in_a_message_are_refused_like_in_the_text_form(field, value, message):
+    """A foreign or damaged cache file must not plant a value the setters and the text form refuse
+    (the options would print and then not parse again)."""
+    raw = serialized("naive")
+    tail = bytes([field << 3])
+    v = value
+    while True:
+        tail += bytes([(v & 0x7F) | (0x80 if v > 0x7F else 0)])
+        v >>= 7
+        if not v:
+            break
+    with pytest.raises(tc.TcError) as e:
+        from_serialized(raw + tail)
+    assert message in str(e.value)
+
+
 @pytest.mark.parametrize("damage", ["truncated", "overlong_varint", "length_past_end", "scalar_for_message"])
 def test_corrupt_messages_are_refused_not_read_out_of_bounds(damage):
     raw = serialized(OPTIONS)
