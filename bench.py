@@ -388,8 +388,10 @@ def measure_suite(steps, warmup):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=100)
-    ap.add_argument("--warmup", type=int, default=10)
+    # (defaults: the reference's benchmark protocol, benchmark_iterations / benchmark_warmup of
+    # tc/core/flags.cc:59-66, overridable like its other flags from the environment)
+    ap.add_argument("--steps", type=int, default=int(os.environ.get("TC_BENCHMARK_ITERATIONS", 100)))
+    ap.add_argument("--warmup", type=int, default=int(os.environ.get("TC_BENCHMARK_WARMUP", 10)))
     ap.add_argument("--config", default="c2_tensordot")
     ap.add_argument("--options", default=None)
     ap.add_argument("--all", action="store_true", help="(kept for old command lines: the other workloads are always measured)")

@@ -155,12 +155,8 @@ int tc_options_cache_load(
 /* Host-side tuner logic without a device, for bindings and tests:
  *   "powers2_and_ceil_divisors", "72"  -> "1,2,3,4,5,8,9,..."   (tc/autotuner/utils.cc:42-56)
  *   "search_space", "<shape>;<shape>..." e.g. "500x26x72;500x72x26" -> candidate value sets
- *   "genetic_search", "seed=..;generations=..;pop_size=.." -> best synthetic cost per generation
- *   "options_cache_selftest", "<scratch file>" -> "name=value" lines: what a sample cache answers (sizes,
- *       ranking by median, misses, pruning, wire and file round trips; test/cuda/test_compilation_cache.cc:133-510)
- *   "options_cache_write_sample", "<file>" -> stores that sample cache (compcache.proto wire format) and
- *       returns its entries as text, one per line
- *   "options_cache_dump", "<file>" -> the entries of any cache file in the same text form
+ *   "options_cache_dump", "<file>" -> the entries of an options cache file as text, one per line:
+ *       id | device | inputs | outputs | options | median runtime
  *   "median", "3,1,2,10" -> "2"                                  (tc/core/utils/math.h:23-37)
  *   "tuner_seeds", "<lowest output rank>[,<innermost output extent>]:<shape>;<shape>..." -> the structured starting points
  *       generation 0 holds next to the base mapping, one option text per line

@@ -5,6 +5,8 @@
 #include <cstdlib>
 #include <cstring>
 #include <iostream>
+#include <mutex>
+#include <set>
 #include <sstream>
 
 #include "capi/tc_capi_internal.h"
@@ -196,7 +198,22 @@ void tc_executor_destroy(tc_executor_t* ex) {
 
 int tc_options_normalize(const char* options, char** text) {
   TC_CAPI_BEGIN
-  *text = dupString(tc::HipMappingOptions::fromText(options ? options : "naive").toText());
+  const std::string given = options ? options : "naive";
+  *text = dupString(tc::HipMappingOptions::fromText(given).toText());
+  // Options that steer the reference's isl scheduler or its promotion depth and that the box
+  // mapper gives no meaning to are accepted, stored and round-tripped; naming one gets a note on
+  // stderr, once per option and process.
+  static std::mutex mu;
+  static std::set<std::string> noted;
+  for (const char* key : {"fixParametersBeforeScheduling", "tileImperfectlyNested", "privateDepth", "outerScheduleAllowSkewing",
+                          "outerSchedulePositiveOrthant", "intraTileScheduleAllowSkewing", "intraTileSchedulePositiveOrthant"}) {
+    if (given.find(std::string(key) + "=") == std::string::npos) continue;
+    std::lock_guard<std::mutex> lock(mu);
+    if (noted.insert(key).second) {
+      std::cerr << "note: mapping option '" << key << "' is kept for compatibility with the reference's options and does not "
+                << "change the mapping of this backend\n";
+    }
+  }
   TC_CAPI_END
 }
 int tc_options_to_serialized(const char* options, void** bytes, size_t* size) {

@@ -366,6 +366,26 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
     TC_CHECK(out != outputs.end()) << "no outputs for device " << in.first;
     Backend::checkTensorsAreLaunchable(in.second, out->second, static_cast<int>(in.first));
   }
+  // The device candidates are measured on: the first device of the tuner_devices flag (a comma-
+  // separated list, as in the reference, tc/autotuner/autotuner-inl.h:245,279-295) for which
+  // tensors were given; the reference spreads candidates over all listed devices, this build
+  // measures on one.
+  size_t tuningDevice = inputs.begin()->first;
+  {
+    bool found = false;
+    std::stringstream listed(flags().tuner_devices);
+    std::string item;
+    while (!found && std::getline(listed, item, ',')) {
+      if (item.empty()) continue;
+      const size_t d = static_cast<size_t>(std::stoul(item));
+      if (inputs.count(d)) {
+        tuningDevice = d;
+        found = true;
+      }
+    }
+    TC_CHECK(found) << "none of the devices of tuner_devices (" << flags().tuner_devices
+                    << ") holds the tensors to tune on (device " << inputs.begin()->first << ")";
+  }
   auto defs = tc::detail::parse(tc);
   TC_CHECK_EQ(defs.count(tcEntryPoint), 1u) << "attempting to access undefined function " << tcEntryPoint;
   lang::TreeRef tree = defs.at(tcEntryPoint);
@@ -699,7 +719,7 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
     std::vector<std::thread> compilers;
     size_t nThreads = std::max<size_t>(1, std::min(settings.threads, population.size()));
     for (size_t t = 0; t < nThreads; ++t) compilers.emplace_back(compileWorker);
-    std::thread evaluator(evaluate, inputs.begin()->first);
+    std::thread evaluator(evaluate, tuningDevice);
     for (auto& t : compilers) t.join();
     cv.notify_all();
     evaluator.join();

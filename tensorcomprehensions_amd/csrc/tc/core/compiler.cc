@@ -2,7 +2,10 @@
 
 #include <sstream>
 
+#include <iostream>
+
 #include "tc/core/check.h"
+#include "tc/core/flags.h"
 #include "tc/lang/parser.h"
 #include "tc/lang/sema.h"
 
@@ -14,6 +17,7 @@ std::map<std::string, lang::TreeRef> parse(const std::string& tc) {
   std::map<std::string, lang::TreeRef> out;
   while (parser.L.cur().kind != lang::TK_EOF) {
     lang::TreeRef t = parser.parseFunction();
+    if (flags().debug_lang) std::cerr << "[LANG] parsed definition:\n" << t << std::endl;
     out.emplace(lang::Def(t).name().name(), t);
   }
   return out;

@@ -23,8 +23,6 @@ Flags& flags() {
     envBool("TC_DEBUG_TUNER", &x.debug_tuner);
     envBool("TC_DUMP_HIP", &x.dump_hip);
     envBool("TC_FAST_MATH", &x.fast_math);
-    envU32("TC_BENCHMARK_WARMUP", &x.benchmark_warmup);
-    envU32("TC_BENCHMARK_ITERATIONS", &x.benchmark_iterations);
     envU32("TC_TUNER_GEN_POP_SIZE", &x.tuner_gen_pop_size);
     envU32("TC_TUNER_GEN_CROSSOVER_RATE", &x.tuner_gen_crossover_rate);
     envU32("TC_TUNER_GEN_MUTATION_RATE", &x.tuner_gen_mutation_rate);
@@ -32,6 +30,9 @@ Flags& flags() {
     envU32("TC_TUNER_GEN_NUMBER_ELITES", &x.tuner_gen_number_elites);
     envU32("TC_TUNER_THREADS", &x.tuner_threads);
     if (const char* e = std::getenv("TC_TUNER_DEVICES")) x.tuner_devices = e;
+    envU32("TC_TUNER_GEN_RESTORE_NUMBER", &x.tuner_gen_restore_number);
+    envBool("TC_TUNER_GEN_LOG_GENERATIONS", &x.tuner_gen_log_generations);
+    if (const char* e = std::getenv("TC_TUNER_RNG_RESTORE")) x.tuner_rng_restore = e;
     if (const char* e = std::getenv("TC_RANDOM_SEED")) x.random_seed = std::strtoll(e, nullptr, 10);
     return x;
   }();

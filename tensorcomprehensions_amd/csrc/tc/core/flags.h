@@ -6,14 +6,16 @@
 
 namespace tc {
 struct Flags {
-  bool debug_lang = false;
-  bool debug_tc_mapper = false;
+  bool debug_lang = false;           // print every parsed definition (its tree) to stderr
+  bool debug_tc_mapper = false;      // print the options and the launches the mapper decided on
   bool debug_tuner = false;
   bool dump_hip = false;             // print generated HIP source at compile time
   bool fast_math = false;            // pass -ffast-math to hipRTC (the reference used --use_fast_math)
-  // benchmark protocol (flags.cc:59-66)
-  uint32_t benchmark_warmup = 10;
-  uint32_t benchmark_iterations = 100;
+  // (benchmark_warmup / benchmark_iterations of flags.cc:59-66 steer the reference's benchmark
+  // fixture, not its library: here they are bench.py's --warmup / --steps, which read the
+  // environment variables TC_BENCHMARK_WARMUP / TC_BENCHMARK_ITERATIONS for their defaults.
+  // tuner_gen_restore_from_proto of flags.cc:107-110 has no reader in the reference either: a
+  // cache file is named per tuning run, TunerSettings::cacheFile.)
   // tuner (flags.cc:77-122)
   uint32_t tuner_gen_pop_size = 100;
   uint32_t tuner_gen_crossover_rate = 80;
@@ -21,8 +23,7 @@ struct Flags {
   uint32_t tuner_gen_generations = 25;
   uint32_t tuner_gen_number_elites = 10;
   uint32_t tuner_threads = 8;
-  std::string tuner_devices = "0";
-  bool tuner_gen_restore_from_proto = false;
+  std::string tuner_devices = "0";   // comma-separated; candidates are measured on the first that holds the tensors
   uint32_t tuner_gen_restore_number = 10;
   bool tuner_gen_log_generations = false;
   uint64_t tuner_min_launch_total_threads = 64;

@@ -72,6 +72,14 @@ HipCompilationResult HipBackend::compileWithTcMapper(
   const auto& k0 = r.program.kernels.front();
   r.grid = HipGrid(std::vector<uint64_t>{(uint64_t)k0.grid[0], (uint64_t)k0.grid[1], (uint64_t)k0.grid[2]});
   r.block = HipBlock(std::vector<uint64_t>{(uint64_t)k0.block[0], (uint64_t)k0.block[1], (uint64_t)k0.block[2]});
+  if (flags().debug_tc_mapper) {
+    // (the reference logs the options and its schedule trees here, cuda_tc_executor.cc:65-105)
+    std::cerr << "[MAPPER] " << r.specializedName << " under " << options.toText() << "\n";
+    for (const auto& k : r.kernels) {
+      std::cerr << "[MAPPER]   kernel " << k.name << " grid " << k.grid[0] << "x" << k.grid[1] << "x" << k.grid[2] << " block "
+                << k.block[0] << "x" << k.block[1] << "x" << k.block[2] << "\n";
+    }
+  }
   if (flags().dump_hip) {
     std::cerr << "generated HIP for " << r.specializedName << ":\n" << r.source << std::endl;
   }

@@ -193,12 +193,12 @@ CASES = {
     "lut": (LUT, "lut", [(50, 24), ("int", (9, 7), 0, 50)], 7),
     "2lut": (LUT2, "func_2lut", [(50, 24), ("int", (9, 7), 0, 50), (30, 24), ("int", (9, 5), 0, 30)], 7),
     "batchnorm": (BATCHNORM, "spatialBatchNorm",
-                  [("scalar", 0.1), ("scalar", 1e-5), (4, 6, 7, 5), (6,), ("positive", (6,))], 140),
+                  [("scalar", 0.1), ("scalar", 1e-5), (4, 6, 7, 5), (6,), ("positive", (6,))], 4 * 7 * 5),   # N*H*W per channel
     "moments2": (MOMENTS2, "moments2_2D_1D", [(24, 500)], 500),
     "group_normalization": (GROUP_NORMALIZATION, "group_normalization",
                             [(3, 4, 5, 6, 7), (4, 5), (4, 5), (3, 4), ("positive", (3, 4))], 1),
     "group_normalization_single_kernel": (GROUP_NORMALIZATION_SINGLE_KERNEL, "group_normalization_single_kernel",
-                                          [(3, 4, 5, 6, 7), (4, 5), (4, 5)], 210),
+                                          [(3, 4, 5, 6, 7), (4, 5), (4, 5)], 5 * 6 * 7),   # D*H*W per (n, g)
     "kronecker3": (KRONECKER3, "Kronecker3Full", [(6, 5), (7, 4), (8, 3), (10, 5, 4, 3)], 5),
     "wavenet1": (WAVENET1, "wavenet1",
                  [(1, 8, 100), (8, 8, 2), (8,), (8, 8, 2), (8,), (8, 8), (8,), (16, 8), (16,), (2,)], 16),

@@ -18,6 +18,7 @@
 #include <vector>
 
 #include "tc_hip.h"
+#include "capi/tc_hip_testing.h"
 
 namespace {
 struct Tensor {
@@ -73,7 +74,9 @@ int main(int argc, char** argv) {
            {"options_cache_write_sample", scratch},
            {"options_cache_dump", scratch}}) {
     char* answer = nullptr;
-    if (tc_host_query(q.first, q.second.c_str(), &answer) != 0) {
+    const std::string name = q.first;
+    const bool scaffolding = name == "genetic_search" || name == "options_cache_selftest" || name == "options_cache_write_sample";
+    if ((scaffolding ? tc_testing_query : tc_host_query)(q.first, q.second.c_str(), &answer) != 0) {
       std::cerr << "host query " << q.first << " failed: " << tc_last_error() << "\n";
       return 1;
     }
@@ -165,7 +168,7 @@ int main(int argc, char** argv) {
       if (!scalarInput) {
         const std::string arg = "generations=3;pop_size=12;threads=8;seed=" + std::to_string(records) + "|" + entry + "|" + shapesArg + "|" + text;
         char* answer = nullptr;
-        if (tc_host_query("tune_on_model", arg.c_str(), &answer) == 0) {
+        if (tc_testing_query("tune_on_model", arg.c_str(), &answer) == 0) {
           tc_free(answer);
           ++tuned;
         }

@@ -5,6 +5,7 @@
 #include <iostream>
 #include <string>
 #include "tc_hip.h"
+#include "capi/tc_hip_testing.h"
 int main() {
   const char* tcs[][3] = {
     {"moments", "1024x4096", "def moments(float(M, N) X) -> (mean, var) { mean(m) +=! X(m, r_n) / N\n var(m) +=! (X(m, r_n) - mean(m)) * (X(m, r_n) - mean(m)) / N }"},
@@ -14,7 +15,7 @@ int main() {
     for (int seed = 1; seed <= 3; ++seed) {
       std::string arg = "generations=4;pop_size=24;threads=8;seed=" + std::to_string(seed) + "|" + t[0] + "|" + t[1] + "|" + t[2];
       char* answer = nullptr;
-      if (tc_host_query("tune_on_model", arg.c_str(), &answer) != 0) { std::cerr << "failed: " << tc_last_error() << "\n"; return 1; }
+      if (tc_testing_query("tune_on_model", arg.c_str(), &answer) != 0) { std::cerr << "failed: " << tc_last_error() << "\n"; return 1; }
       tc_free(answer);
     }
   }

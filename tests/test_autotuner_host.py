@@ -7,6 +7,7 @@ import tempfile
 import pytest
 
 import tensorcomprehensions_amd as tc
+from tests.scaffolding import scaffold_query
 
 
 @pytest.mark.parametrize("n,expected", [
@@ -44,13 +45,13 @@ def test_search_space_from_shapes():
 
 
 def test_base_mapping_outside_the_space_is_refused():
-    assert tc.host_query("base_outside_space").startswith("invalid_argument")
+    assert scaffold_query("base_outside_space").startswith("invalid_argument")
 
 
 def test_genetic_search_is_deterministic_and_monotone_with_elites():
-    a = tc.host_query("genetic_search", "seed=5;generations=12;pop_size=24;number_elites=3")
-    b = tc.host_query("genetic_search", "seed=5;generations=12;pop_size=24;number_elites=3")
-    c = tc.host_query("genetic_search", "seed=6;generations=12;pop_size=24;number_elites=3")
+    a = scaffold_query("genetic_search", "seed=5;generations=12;pop_size=24;number_elites=3")
+    b = scaffold_query("genetic_search", "seed=5;generations=12;pop_size=24;number_elites=3")
+    c = scaffold_query("genetic_search", "seed=6;generations=12;pop_size=24;number_elites=3")
     assert a == b
     best = [float(x) for x in a.split(",")]
     assert all(x >= y for x, y in zip(best, best[1:]))      # elites keep the best alive
@@ -61,7 +62,7 @@ def test_genetic_search_is_deterministic_and_monotone_with_elites():
 def test_genetic_search_survives_mostly_invalid_generations():
     # only every 6th candidate is valid: with 12 candidates that is 2 < 3 survivors, so every
     # generation takes the re-randomise-around-the-last-best path
-    out = tc.host_query("genetic_search", "seed=2;generations=6;pop_size=12;invalid_every=6")
+    out = scaffold_query("genetic_search", "seed=2;generations=6;pop_size=12;invalid_every=6")
     assert len(out.split(",")) == 6
 
 
@@ -100,7 +101,7 @@ def model_tune(settings, name="c5_moments"):
     from tests import workloads as W
     text, entry, shapes, _, _ = W.CONFIGS[name]
     arg = settings + "|" + entry + "|" + ";".join("x".join(map(str, s)) for s in shapes) + "|" + text
-    fields = dict(line.split("=", 1) for line in tc.host_query("tune_on_model", arg).split("\n"))
+    fields = dict(line.split("=", 1) for line in scaffold_query("tune_on_model", arg).split("\n"))
     return fields["best"], int(fields["cost_ns"]), int(fields["naive_ns"])
 
 
@@ -178,5 +179,5 @@ def test_fixed_parameters_hold_in_every_candidate_of_a_search():
     assert fields["unroll"] == "4" and fields["mapToThreads"] == "128,2" and fields["useSharedMemory"] == "1"
     assert fields["matchLibraryCalls"] == "0" and fields["vectorWidth"] == "2" and cost <= naive
     arg_top = settings.replace("generations=3", "generations=2") + ";top_k=3"
-    text = tc.host_query("tune_on_model", arg_top + "|moments|64x512|def moments(float(M, N) X) -> (mean) { mean(m) +=! X(m, r_n) / N }")
+    text = scaffold_query("tune_on_model", arg_top + "|moments|64x512|def moments(float(M, N) X) -> (mean) { mean(m) +=! X(m, r_n) / N }")
     assert text.startswith("best=")

@@ -22,8 +22,12 @@ def chain(*lengths):
     return float(sum(np.sqrt(k) for k in lengths)) ** 2
 
 
-CHAINED = {"2fcrelu": chain(48, 36), "mlp3": chain(24, 18, 10), "kronecker3": chain(5, 4, 3), "batchnorm": 140, "wavenet1": chain(16, 8, 8),
-           "group_normalization_single_kernel": 210}
+# Reduction lengths at the test sizes of tests/benchmark_tcs.py:CASES.  Chains: the lengths of the
+# reductions that feed one another.  The normalisations reduce over everything but the dimension
+# they normalise per: batch norm of a 4x6x7x5 input over N*H*W = 4*7*5 per channel, the one-kernel
+# group norm of a 3x4x5x6x7 input over D*H*W = 5*6*7 per (n, g).
+CHAINED = {"2fcrelu": chain(48, 36), "mlp3": chain(24, 18, 10), "kronecker3": chain(5, 4, 3), "batchnorm": 4 * 7 * 5,
+           "wavenet1": chain(16, 8, 8), "group_normalization_single_kernel": 5 * 6 * 7}
 
 
 @pytest.mark.parametrize("options", sorted(OPTION_SETS))
@@ -44,7 +48,7 @@ def test_parity_with_oracle(name, options):
     for o, r in zip(outs, ref):
         got = o.cpu().numpy()
         assert got.shape == r.shape
-        scale = max(1.0, float(np.abs(r).max()))
+        scale = max(float(np.abs(r).max()), 1e-30)
         assert np.abs(got - r).max() <= 1e-5 * np.sqrt(k) * scale, (name, options, ex.launch_bounds())
 
 
@@ -61,15 +65,17 @@ def test_parity_at_the_reference_sizes_with_the_tuned_options(name):
         o.fill_(float("nan"))
     tc.run(ex, ins, outs)
     torch.cuda.synchronize()
-    # reduction lengths at these sizes (chains: see chain())
+    # reduction lengths at these sizes (chains: see chain()); the group normalisation from given
+    # means and variances reduces nothing (1), the one-kernel form and the moments reduce over
+    # D*H*W = 16*48*48 elements per (n, g), respectively over a row of 36864
     k = {"tmm": 256, "matmul": 1000, "convolution": 36, "group_convolution": 36, "2fcrelu": chain(2000, 128), "mlp1": 2000, "mlp3": chain(128, 64, 32), "lut": 50,
          "c3": 1000, "2lut": 50, "group_normalization": 1,
-         "moments2": 36864, "group_normalization_single_kernel": 36864, "kronecker3": chain(16, 16, 16),
+         "moments2": 36864, "group_normalization_single_kernel": 16 * 48 * 48, "kronecker3": chain(16, 16, 16),
          "wavenet1": chain(64, 32, 32)}[name]
     for o, r in zip(outs, ref):
         got = o.cpu().numpy()
         assert got.shape == r.shape
-        scale = max(1.0, float(np.abs(r).max()))
+        scale = max(float(np.abs(r).max()), 1e-30)
         assert np.abs(got - r).max() <= 1e-5 * np.sqrt(k) * scale, (name, ex.launch_bounds())
 
 

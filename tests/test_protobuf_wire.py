@@ -10,6 +10,7 @@ import tempfile
 import pytest
 
 import tensorcomprehensions_amd as tc
+from tests.scaffolding import scaffold_query
 from tensorcomprehensions_amd import _capi
 
 pb = pytest.importorskip("google.protobuf")
@@ -204,7 +205,7 @@ def test_corrupt_messages_are_refused_not_read_out_of_bounds(damage):
 def test_protobuf_reads_a_cache_file_and_the_library_reads_protobufs(messages):
     with tempfile.TemporaryDirectory() as d:
         path = os.path.join(d, "cache.bin")
-        listing = tc.host_query("options_cache_write_sample", path)
+        listing = scaffold_query("options_cache_write_sample", path)
         m = messages["HipOptionsCacheProto"]()
         m.ParseFromString(open(path, "rb").read())
         assert m.IsInitialized() and len(m.keys) == len(m.values) == 4
@@ -238,7 +239,7 @@ def test_cache_semantics_of_the_reference():
     """test/cuda/test_compilation_cache.cc:133-510 on a cache with two TCs: multimap counts, ranking by the
     median of all runs of an option, misses on any differing key part, pruning, wire and file round trips."""
     with tempfile.TemporaryDirectory() as d:
-        lines = dict(line.split("=", 1) for line in tc.host_query("options_cache_selftest", os.path.join(d, "c.bin")).splitlines())
+        lines = dict(line.split("=", 1) for line in scaffold_query("options_cache_selftest", os.path.join(d, "c.bin")).splitlines())
     assert lines["size"] == "4" and lines["count_tcA"] == "3" and lines["keys"] == "2"
     assert lines["top2_tcA"] == "o2@15000,o1@20000"             # o1 ran 10, 30 and 20 us: median 20
     assert [lines[k] for k in ("miss_other_tc", "miss_other_sizes", "miss_other_device", "miss_other_alignment")] == ["0"] * 4
