@@ -50,6 +50,7 @@ inline void readTunerSettings(const char* text, tc::autotune::TunerSettings& st,
     else if (k == "min_launch_total_threads") st.minLaunchTotalThreads = num();
     else if (k == "max_serial_depth_ratio") st.maxSerialDepthRatio = std::stod(v);
     else if (k == "seed_heuristics") st.seedHeuristics = num() != 0;
+    else if (k == "structured_random") st.structuredRandom = num() != 0;
     else if (k == "refinement_rounds") st.refinementRounds = num();
     else if (k == "fix_inert") st.fixInertParameters = num() != 0;
     else if (k == "resample_duplicates") st.resampleDuplicates = num();

@@ -51,6 +51,10 @@ struct TunerSettings {
   // generation 0 also holds a few structured variants of the first base mapping (streaming,
   // row-reduction and matrix-core shapes); the search then starts from more than one basin
   bool seedHeuristics = true;
+  // Half of the random members of generation 0 are drawn from what the output shape suggests
+  // (structuredRandomMembers) instead of uniformly from the value sets; 0 = the reference's
+  // uniform draw for all of them.
+  bool structuredRandom = true;
   // after the last generation: rounds of one-gene steps around the best candidate (every gene
   // moved to its neighbouring values, one at a time); a round that finds nothing better ends it
   size_t refinementRounds = 2;
@@ -123,6 +127,93 @@ inline std::vector<size_t> mergedDimensionThreadCounts(const std::vector<const D
   std::sort(merged.begin(), merged.end());
   merged.erase(std::unique(merged.begin(), merged.end()), merged.end());
   return merged;
+}
+
+// Random members of generation 0 with informed priors.  A member drawn uniformly from the value
+// sets is, for most comprehensions, a kernel of small scalar blocks that loop over what should be
+// spread: its tiles, thread counts and grid sizes are independent draws from the divisors of all
+// dimensions.  These members are random too, but each draw is coherent with the output's shape:
+// some number of trailing output dimensions, taken whole, is spread over the threads (the thread
+// count covers their merged extent exactly, in lanes of 1, 2 or 4, or is a plain multiple of the
+// wavefront), the dimensions ahead of them get tiles of 1 or a small divisor of their own extent,
+// the grid covers the tiles, the unroll budget is large; the remaining switches are coin tosses.
+// No family of kernels is named: what the shapes allow is drawn from.
+inline std::vector<HipMappingOptions> structuredRandomMembers(
+    const HipMappingOptions& base, const std::vector<int64_t>& outShape, size_t count, uint64_t seed) {
+  std::vector<HipMappingOptions> members;
+  const size_t R = outShape.size();
+  if (R == 0 || count == 0) return members;
+  std::mt19937_64 rng(seed * 6364136223846793005ULL + 1442695040888963407ULL);
+  auto pick = [&](size_t n) { return std::uniform_int_distribution<size_t>(0, n - 1)(rng); };
+  auto coin = [&](double p) { return std::bernoulli_distribution(p)(rng); };
+  // (threads, lanes, trailing dimensions covered)
+  struct Spread {
+    uint64_t threads;
+    uint32_t lanes;
+    size_t dims;
+  };
+  std::vector<Spread> spreads;
+  {
+    int64_t merged = 1;
+    for (size_t j = R; j-- > 0;) {
+      merged *= outShape[j];
+      if (merged > 4096) break;
+      for (uint32_t lanes : {1u, 2u, 4u}) {
+        if (merged % lanes != 0 || outShape[R - 1] % lanes != 0) continue;
+        const int64_t t = merged / lanes;
+        if (t >= 32 && t <= 1024) spreads.push_back({static_cast<uint64_t>(t), lanes, R - j});
+      }
+    }
+    // plain wavefront multiples over the innermost dimension alone
+    for (uint64_t t : {64u, 128u, 256u, 512u}) {
+      for (uint32_t lanes : {1u, 2u, 4u}) {
+        if (outShape[R - 1] % lanes == 0) spreads.push_back({t, lanes, 1});
+      }
+    }
+  }
+  auto smallDivisor = [&](int64_t extent) {
+    std::vector<uint64_t> d;
+    for (int64_t k = 1; k <= std::min<int64_t>(extent, 32); ++k) {
+      if (extent % k == 0) d.push_back(static_cast<uint64_t>(k));
+    }
+    return d[pick(d.size())];
+  };
+  const std::vector<FusionStrategy> fusions{FusionStrategy::Max, FusionStrategy::Preserve3Coincident, FusionStrategy::Min};
+  for (size_t made = 0, tries = 0; made < count && tries < 20 * count; ++tries) {
+    const Spread sp = spreads[pick(spreads.size())];
+    const bool rows = coin(0.25); // every output element a reduction of its own along the threads
+    HipMappingOptions o = base;
+    std::vector<uint64_t> tile, grid;
+    const size_t lead = rows ? R : R - std::min(R, sp.dims);
+    for (size_t i = 0; i < R; ++i) {
+      if (i < lead) {
+        const uint64_t t = rows || coin(0.5) ? 1 : smallDivisor(outShape[i]);
+        tile.push_back(t);
+        if (grid.size() < 3) grid.push_back(static_cast<uint64_t>((outShape[i] + t - 1) / t));
+      } else {
+        tile.push_back(0);
+      }
+    }
+    if (grid.empty()) grid.push_back(256);
+    o.tile(tile);
+    o.mapToBlocks(grid);
+    o.mapToThreads(std::vector<uint64_t>{rows ? std::vector<uint64_t>{256, 512, 1024}[pick(3)] : sp.threads});
+    o.vectorWidth(rows ? std::vector<uint32_t>{1, 4}[pick(2)] : sp.lanes);
+    o.unroll(std::vector<uint64_t>{8, 32, 128, 256}[pick(4)]);
+    o.matchLibraryCalls(rows || coin(0.2));
+    o.useSharedMemory(coin(0.3));
+    o.usePrivateMemory(coin(rows ? 0.7 : 0.3));
+    o.useReadOnlyCache(coin(0.8));
+    o.collapseContiguous(true);
+    o.useMfma(!rows && coin(0.15));
+    o.prefetchShared(coin(0.2));
+    o.outerScheduleFusionStrategy(fusions[pick(3)]);
+    o.intraTileScheduleFusionStrategy(fusions[pick(3)]);
+    if (std::find(members.begin(), members.end(), o) != members.end()) continue;
+    members.push_back(o);
+    ++made;
+  }
+  return members;
 }
 
 // Structured starting points next to the caller's base mapping.  The genetic search from one
@@ -454,6 +545,20 @@ std::vector<typename Backend::MappingOptionsType> Autotuner<Backend, SearchStrat
       try {
         TuningConfiguration c = space;
         c.fromHipMappingOptions(seed);
+        if (c.isValid()) configs.push_back(c);
+      } catch (const std::invalid_argument&) {
+      }
+    }
+  }
+  if (settings.structuredRandom && !outputsInfo.empty() && configs.size() < settings.populationSize / 2) {
+    // (a member the possibly restricted space cannot express is left out; the rest of the
+    // generation is the uniform draw of the search itself)
+    const uint64_t drawSeed = settings.seed >= 0 ? static_cast<uint64_t>(settings.seed) : randomSeed();
+    for (const auto& member : detail::structuredRandomMembers(
+             bases.front(), outputsInfo.front().shape, settings.populationSize / 2 - configs.size(), drawSeed)) {
+      try {
+        TuningConfiguration c = space;
+        c.fromHipMappingOptions(member);
         if (c.isValid()) configs.push_back(c);
       } catch (const std::invalid_argument&) {
       }

@@ -256,7 +256,7 @@ def test_device_buffers_stand_in_for_tensors():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("name", ["c2_tensordot", "c5_moments"])
+@pytest.mark.parametrize("name", ["c2_tensordot", "c3_batch_matmul", "c4_group_convolution", "c5_moments"])
 def test_autotune_from_the_naive_options_reaches_the_stored_options(name):
     """What 'after autotuning' means for the benchmark configurations: a short, seeded search that
     starts from the naive options ends within 15 % of the options the benchmark stores, and its
