@@ -67,6 +67,10 @@ struct Promotion {
   int64_t elems = 0;                 // LDS elements including padding
   int64_t reuse = 1;                 // accesses per staged element
   bool insideReductionTiles = false;
+  // 2: the software pipeline over the reduction tiles alternates between two copies of the
+  // array (the next tile is stored while the current one is still being read: one barrier per
+  // tile instead of two); `elems` is the size of one copy.
+  int buffers = 1;
   // An earlier stage of the kernel staged the very same footprint and nothing has overwritten it:
   // this stage reads that copy (`ldsName` names the earlier stage's array) and copies nothing.
   bool sharedWithEarlierStage = false;

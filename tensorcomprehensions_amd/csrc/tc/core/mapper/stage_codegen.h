@@ -519,8 +519,12 @@ class StageCodegen {
       if (p.ldsStrides[j] != 1) ss << " * " << p.ldsStrides[j];
     }
     if (subs.empty()) ss << "0";
+    if (p.buffers == 2 && !readBuffer_.empty()) ss << " + " << readBuffer_ << " * " << p.elems;
     return ss.str();
   }
+  // Which of the two copies of a double-buffered array is read and which is written (expressions
+  // with value 0 or 1; empty outside the software pipeline over the reduction tiles).
+  std::string readBuffer_, writeBuffer_;
 
   // Decide which read-only operands of statement `s` to stage in LDS.
   // Matrix-core stages whose block tile holds a single 16-row group of the M side: the M-side
@@ -746,6 +750,25 @@ class StageCodegen {
         st_.promotions.push_back(c.p);
       }
     }
+    // Two copies of the arrays staged per reduction tile when the matrix-core software pipeline
+    // will run over them and LDS has the room.
+    if (st_.mfma && kc_.opts.prefetchSharedValue) {
+      int64_t extra = 0, stagingRegs = 0;
+      bool any = false;
+      for (const auto& p : st_.promotions) {
+        if (!p.insideReductionTiles) continue;
+        any = true;
+        extra += p.elems * st_.views.at(p.tensor).type.bytes();
+        stagingRegs += copyRegisters(p);
+      }
+      // (the pipeline's own conditions, emitMfma: staged per reduction tile, at most 64 staging registers)
+      if (any && stagingRegs <= 64 && extra <= ldsBudgetBytes) {
+        ldsBudgetBytes -= extra;
+        for (auto& p : st_.promotions) {
+          if (p.insideReductionTiles) p.buffers = 2;
+        }
+      }
+    }
   }
 
   bool lanesWalkOuterDim(const std::vector<Affine>& subs) const {
@@ -768,7 +791,7 @@ class StageCodegen {
     for (const auto& p : st_.promotions) {
       if (p.sharedWithEarlierStage) continue;
       em_.line("__shared__ __attribute__((aligned(16))) " + st_.views.at(p.tensor).type.cName() + " " + p.ldsName +
-               "[" + std::to_string(p.elems) + "];");
+               "[" + std::to_string(p.elems * p.buffers) + "];");
     }
   }
 
@@ -950,6 +973,7 @@ class StageCodegen {
       std::string addr = cond.empty() ? gidx : "(" + cond + ") ? (" + gidx + ") : 0";
       em_.line(guard + regs + "[" + slot + "] = " + cast + "p" + p.tensor + "[" + addr + "];");
     } else {
+      if (p.buffers == 2 && !writeBuffer_.empty()) lidx += " + " + writeBuffer_ + " * " + std::to_string(p.elems);
       em_.line(guard + lcast + p.ldsName + "[" + lidx + "] = " + regs + "[" + slot + "];");
     }
   }
@@ -2014,8 +2038,39 @@ class StageCodegen {
     // wavefront wv_ takes tiles wv_, wv_ + waves, ...; with one, wavefront wv_ takes slice
     // wv_ / tiles of the reduction of tile wv_ % tiles and slice 0 owns the tile.
     const std::string T = std::to_string(tiles), W = std::to_string(st_.waves), S = std::to_string(split);
-    const std::string tileDecl = split > 1 ? "const int tl_ = wv_ % " + T + ", sl_ = wv_ / " + T + ";"
-                                           : "const int tl_ = wv_ + j_ * " + W + ";";
+    // Register blocking (reduction-tiled stages).  A wavefront that owns a rectangle of RM x RN
+    // output tiles reads RM M-side and RN N-side operand values per reduction step for RM * RN
+    // multiplications, and its accumulators take turns, so no multiplication waits for the one
+    // before it (a chain of dependent 16x16x4 instructions issues every 43 cycles instead of
+    // every 32 when a SIMD holds a single wavefront).  The wavefronts form a WM x WN grid over
+    // the tiles of the block; without such a grid tiles are dealt round-robin and multiplied one
+    // at a time.
+    int64_t blockWM = 0, blockWN = 0;
+    if (kTiled && split == 1 && BT == 1 && tiles % st_.waves == 0 && ceilDiv(tiles, st_.waves) <= 16) {
+      int64_t bestCost = 0;
+      for (int64_t wm = 1; wm <= st_.waves; ++wm) {
+        if (st_.waves % wm != 0) continue;
+        const int64_t wn = st_.waves / wm;
+        if (numMT % wm != 0 || numNT % wn != 0) continue;
+        const int64_t rm = numMT / wm, rn = numNT / wn;
+        // operand registers of one reduction tile: (rm + rn) values per step
+        if ((rm + rn) * stepsPerWave > 128) continue;
+        if (blockWM == 0 || rm + rn < bestCost) {
+          blockWM = wm;
+          blockWN = wn;
+          bestCost = rm + rn;
+        }
+      }
+    }
+    const bool registerBlocked = blockWM > 0;
+    const int64_t RM = registerBlocked ? numMT / blockWM : 0, RN = registerBlocked ? numNT / blockWN : 0;
+    const std::string tileDecl =
+        split > 1 ? "const int tl_ = wv_ % " + T + ", sl_ = wv_ / " + T + ";"
+        : registerBlocked
+            ? "const int tl_ = ((wv_ / " + std::to_string(blockWN) + ") * " + std::to_string(RM) + " + j_ / " + std::to_string(RN) +
+                  ") * " + std::to_string(numNT) + " + (wv_ % " + std::to_string(blockWN) + ") * " + std::to_string(RN) + " + j_ % " +
+                  std::to_string(RN) + ";"
+            : "const int tl_ = wv_ + j_ * " + W + ";";
     const std::string worksOnTile = split > 1 ? "sl_ < " + S : "tl_ < " + T;
     const std::string ownsTile = split > 1 ? "sl_ == 0" : "tl_ < " + T;
     const std::string partialAt = kSplitName() + "[((%s * " + T + " + tl_) * 64 + threadIdx.x) * 4]";
@@ -2213,6 +2268,10 @@ class StageCodegen {
       }
       pipelineK = pipelineK && anyInside && stagingRegs <= 64;
       const std::string tk = tv(k0);
+      // (two copies of every array staged per reduction tile: the next tile is stored into the
+      // other copy right after the multiplications, no barrier between reading and overwriting)
+      bool twoCopies = pipelineK;
+      for (const auto& p : st_.promotions) twoCopies &= !p.insideReductionTiles || p.buffers == 2;
       if (pipelineK) {
         em_.open("");
         ++opened;
@@ -2227,12 +2286,18 @@ class StageCodegen {
           emitCopyLoads(p, "pk_" + p.tensor + "_");
         }
         em_.line("__syncthreads();");
+        if (twoCopies) writeBuffer_ = "0";
         for (const auto& p : st_.promotions) {
           if (p.insideReductionTiles) emitCopyStores(p, "pk_" + p.tensor + "_");
         }
+        writeBuffer_.clear();
         em_.close();
       }
       em_.open("for (int " + tk + " = 0; " + tk + " < " + std::to_string(k0.numTiles) + "; ++" + tk + ")");
+      if (pipelineK && twoCopies) {
+        readBuffer_ = "(" + tk + " & 1)";
+        writeBuffer_ = "((" + tk + " + 1) & 1)";
+      }
       if (pipelineK) {
         em_.line("__syncthreads();");
         em_.line("const bool more_ = " + tk + " + 1 < " + std::to_string(k0.numTiles) + ";");
@@ -2253,22 +2318,74 @@ class StageCodegen {
       } else {
         stagePromotions(true);
       }
-      em_.line("#pragma unroll");
-      em_.open("for (int j_ = 0; j_ < " + std::to_string(tilesPerWave) + "; ++j_)");
-      em_.line(tileDecl);
-      em_.open("if (" + worksOnTile + ")");
-      decodeTile();
-      multiply("cacc_[j_]");
-      em_.close();
-      em_.close();
+      if (registerBlocked) {
+        const std::string steps = std::to_string(stepsPerWave);
+        em_.open("");
+        em_.line("const int bt_ = 0;");
+        em_.line("(void)bt_;");
+        std::string bok = st_.mfmaBatch.empty() ? "true" : decodeGroup(st_.mfmaBatch, "bt_", true, true);
+        em_.line("const bool bok_ = " + bok + ";");
+        em_.line("(void)bok_;");
+        em_.line("float ra_[" + std::to_string(RM) + "][" + steps + "];");
+        em_.line("float rb_[" + std::to_string(RN) + "][" + steps + "];");
+        // the operand values of the whole reduction tile first ...
+        em_.line("#pragma unroll");
+        em_.open("for (int a_ = 0; a_ < " + std::to_string(RM) + "; ++a_)");
+        em_.line("const int mt_ = (wv_ / " + std::to_string(blockWN) + ") * " + std::to_string(RM) + " + a_;");
+        em_.line("const int mposa_ = mt_ * 16 + lm_;");
+        em_.line("const bool moka_ = bok_ && " + decodeGroup(st_.mfmaM, "mposa_", true, MT % 16 == 0) + ";");
+        em_.line("(void)moka_;");
+        {
+          bool masked = openSteps(stepsPerWave);
+          em_.line("ra_[a_][ks_] = " + operandValue(loadA, masked) + ";");
+          em_.close();
+        }
+        em_.close();
+        em_.line("#pragma unroll");
+        em_.open("for (int b_ = 0; b_ < " + std::to_string(RN) + "; ++b_)");
+        em_.line("const int nt_ = (wv_ % " + std::to_string(blockWN) + ") * " + std::to_string(RN) + " + b_;");
+        em_.line("const int npos_ = nt_ * 16 + lm_;");
+        em_.line("const bool nok_ = bok_ && " + decodeGroup(st_.mfmaN, "npos_", true, NT % 16 == 0) + ";");
+        em_.line("(void)nok_;");
+        {
+          bool masked = openSteps(stepsPerWave);
+          em_.line("rb_[b_][ks_] = " + operandValue(loadB, masked) + ";");
+          em_.close();
+        }
+        em_.close();
+        // ... then the multiplications, step by step over all tiles of the rectangle
+        em_.line("#pragma unroll");
+        em_.open("for (int ks_ = 0; ks_ < " + steps + "; ++ks_)");
+        em_.line("#pragma unroll");
+        em_.open("for (int a_ = 0; a_ < " + std::to_string(RM) + "; ++a_)");
+        em_.line("#pragma unroll");
+        em_.open("for (int b_ = 0; b_ < " + std::to_string(RN) + "; ++b_)");
+        em_.line("cacc_[a_ * " + std::to_string(RN) + " + b_] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra_[a_][ks_], rb_[b_][ks_], cacc_[a_ * " +
+                 std::to_string(RN) + " + b_], 0, 0, 0);");
+        em_.close();
+        em_.close();
+        em_.close();
+        em_.close();
+      } else {
+        em_.line("#pragma unroll");
+        em_.open("for (int j_ = 0; j_ < " + std::to_string(tilesPerWave) + "; ++j_)");
+        em_.line(tileDecl);
+        em_.open("if (" + worksOnTile + ")");
+        decodeTile();
+        multiply("cacc_[j_]");
+        em_.close();
+        em_.close();
+      }
       if (pipelineK) {
-        em_.line("__syncthreads();");
+        if (!twoCopies) em_.line("__syncthreads();");
         em_.open("if (more_)");
         for (const auto& p : st_.promotions) {
           if (p.insideReductionTiles) emitCopyStores(p, "pk_" + p.tensor + "_");
         }
         em_.close();
       }
+      readBuffer_.clear();
+      writeBuffer_.clear();
       em_.close();
       if (split > 1) {
         em_.open("");
