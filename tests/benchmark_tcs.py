@@ -265,8 +265,8 @@ TUNED_AT_REFERENCE_SIZES = {
                                          "useSharedMemory=1;usePrivateMemory=1;useReadOnlyCache=1;vectorWidth=4",
     "group_normalization": "naive;tile=4,1,0,0,0;unroll=16;mapToThreads=48,16,1;mapToBlocks=256,256;useSharedMemory=1;"
                            "useReadOnlyCache=1;vectorWidth=4",
-    "kronecker3": "naive;outerScheduleFusionStrategy=Max;intraTileScheduleFusionStrategy=Max;tile=1,32,32;unroll=8;"
-                  "tileImperfectlyNested=1;mapToThreads=64,16;mapToBlocks=256,256;useSharedMemory=1;useReadOnlyCache=1;"
+    "kronecker3": "naive;outerScheduleFusionStrategy=Max;intraTileScheduleFusionStrategy=Max;tile=1,16,0,0,8;unroll=8;"
+                  "tileImperfectlyNested=1;mapToThreads=64,16;mapToBlocks=256,256,256;useSharedMemory=1;useReadOnlyCache=1;"
                   "privateDepth=5;collapseContiguous=0;useMfma=1;prefetchShared=1",
     "wavenet1": "naive;intraTileScheduleFusionStrategy=Max;fixParametersBeforeScheduling=1;tile=2,2000,16,1;mapToThreads=16,64;"
                 "mapToBlocks=2000,256;useSharedMemory=1;usePrivateMemory=1;privateDepth=8;sharedDepth=3;vectorWidth=4;"
