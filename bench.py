@@ -344,7 +344,7 @@ def suite_library_routines():
     }
 
 
-def measure_suite(steps, warmup):
+def measure_suite(steps, warmup, only=()):
     """Kernel time of every comprehension of tests/benchmark_tcs.py:REFERENCE_SIZES under its tuned
     options (sum over its kernels, HIP events around `steps` back-to-back runs), the bytes of all
     its inputs and outputs counted once (look-up tables: the gathered rows), and the library time."""
@@ -353,9 +353,17 @@ def measure_suite(steps, warmup):
     from tests import benchmark_tcs as B
     routines = suite_library_routines()
     out = {}
-    for name, options in B.TUNED_AT_REFERENCE_SIZES.items():
-        src, entry, _, _ = B.CASES[name]
-        ins = [torch.from_numpy(a).cuda() for a in B.make_inputs(name, reference_sizes=True)]
+    cases = [(name, name, options, None) for name, options in B.TUNED_AT_REFERENCE_SIZES.items()]
+    cases += [(name, case, options, k) for name, (case, _, options, k) in B.LARGE_CONTRACTIONS.items()]
+    unknown = set(only) - {c[0] for c in cases}
+    if unknown:
+        sys.exit(f"--suite-cases: unknown comprehension(s) {sorted(unknown)}")
+    for name, case, options, k in cases:
+        if only and name not in only:
+            continue
+        src, entry, _, _ = B.CASES[case]
+        arrays = B.make_large_inputs(name) if k else B.make_inputs(name, reference_sizes=True)
+        ins = [torch.from_numpy(a).cuda() for a in arrays]
         ex = tc.compile(src, entry, ins, options)
         outs = tc.prepare_outputs(src, entry, ins)
         spin(ex, ins, outs, SPIN_MS / 3)
@@ -369,7 +377,12 @@ def measure_suite(steps, warmup):
         entry_out = {"kernel_us": round(us, 2), "kernels": ex.num_kernels, "bytes": nbytes,
                      "gb_per_s": round(nbytes / us / 1e3, 1),
                      "launch": [ex.launch_bounds(k) for k in range(ex.num_kernels)]}
-        fn = routines.get(name)
+        if k:
+            # a contraction's matrix-core roofline: 2 flops per multiply-add over the 157.3 TFLOP/s fp32 peak
+            flops = 2.0 * outs[0].numel() * k
+            entry_out["tflops"] = round(flops / us * 1e-6, 1)
+            entry_out["frac_of_fp32_matrix_peak"] = round(flops / us * 1e-6 / FP32_PEAK_TFLOPS, 3)
+        fn = routines.get(case)
         if fn is not None:
             for _ in range(warmup):
                 fn(*ins)
@@ -408,6 +421,8 @@ def main():
                     help="further tuner settings for --tune (seed_heuristics=0, refinement_rounds=0, seed=3, ...)")
     ap.add_argument("--suite", action="store_true",
                     help="also time the reference's other benchmark comprehensions at their default sizes")
+    ap.add_argument("--suite-cases", default="", metavar="NAME,...",
+                    help="restrict --suite to these comprehensions (profiling runs)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--floor", action="store_true",
                     help="also time near-empty copy kernels of 1, 64 and 500 blocks (the cost of a launch)")
@@ -484,7 +499,7 @@ def main():
     if a.stream:
         line["stream_probes"] = stream_probes(a.steps)
     if a.suite:
-        line["suite"] = measure_suite(a.steps, a.warmup)
+        line["suite"] = measure_suite(a.steps, a.warmup, [n for n in a.suite_cases.split(",") if n])
     print(json.dumps(line))
 
 

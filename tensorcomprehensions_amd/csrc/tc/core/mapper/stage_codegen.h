@@ -1657,14 +1657,14 @@ class StageCodegen {
     const std::string kx = split > 1 ? "kq_" : "ks_"; // counter of a wavefront's own steps
     // Opens the loop over the reduction steps of a lane, decodes the reduction indices of the
     // step and declares kok_ when surplus steps exist; returns whether it did.
-    auto openSteps = [&](int64_t count) {
+    auto openSteps = [&](int64_t count, int64_t first = 0, int64_t last = -1) {
       em_.line(count <= 128 ? "#pragma unroll" : "#pragma unroll 4");
       if (split > 1) {
         // slice sl_ of the steps: ks_ is the step within the whole reduction
         em_.open("for (int kq_ = 0; kq_ < " + std::to_string(count) + "; ++kq_)");
         em_.line("const int ks_ = sl_ * " + std::to_string(stepsPerWave) + " + kq_;");
       } else {
-        em_.open("for (int ks_ = 0; ks_ < " + std::to_string(ksteps) + "; ++ks_)");
+        em_.open("for (int ks_ = " + std::to_string(first) + "; ks_ < " + std::to_string(last < 0 ? ksteps : last) + "; ++ks_)");
       }
       std::string kok;
       if (aligned) {
@@ -2272,63 +2272,30 @@ class StageCodegen {
       // other copy right after the multiplications, no barrier between reading and overwriting)
       bool twoCopies = pipelineK;
       for (const auto& p : st_.promotions) twoCopies &= !p.insideReductionTiles || p.buffers == 2;
-      if (pipelineK) {
-        em_.open("");
-        ++opened;
-        for (const auto& p : st_.promotions) {
-          if (p.insideReductionTiles) em_.line(copyRegisterDecl(p, "pk_" + p.tensor + "_"));
-        }
-        em_.open("");
-        em_.line("const int " + tk + " = 0;");
-        for (const auto& p : st_.promotions) {
-          if (!p.insideReductionTiles) continue;
-          declareLows(p);
-          emitCopyLoads(p, "pk_" + p.tensor + "_");
-        }
-        em_.line("__syncthreads();");
-        if (twoCopies) writeBuffer_ = "0";
-        for (const auto& p : st_.promotions) {
-          if (p.insideReductionTiles) emitCopyStores(p, "pk_" + p.tensor + "_");
-        }
-        writeBuffer_.clear();
-        em_.close();
+      // Rotated pipeline (register-blocked stages with two LDS copies whose operands both come
+      // from LDS).  With one or two wavefronts per SIMD that all pass the same barrier, nothing
+      // multiplies while the block stores a tile, waits and reads its first operand values.  The
+      // steps of a tile are therefore cut in two halves: the operand values of the first half of
+      // tile t+1 are read right behind the barrier that publishes it, while the second half of
+      // tile t (read before the barrier) is still being multiplied, and the stores of tile t+1
+      // sit one step of multiplications ahead of that barrier.
+      bool bothStaged = true;
+      for (const ExprRef* l : {&loadA, &loadB}) {
+        bool staged = false;
+        for (const auto& p : st_.promotions) staged |= p.insideReductionTiles && p.tensor == (*l)->name;
+        bothStaged &= staged;
       }
-      em_.open("for (int " + tk + " = 0; " + tk + " < " + std::to_string(k0.numTiles) + "; ++" + tk + ")");
-      if (pipelineK && twoCopies) {
-        readBuffer_ = "(" + tk + " & 1)";
-        writeBuffer_ = "((" + tk + " + 1) & 1)";
-      }
-      if (pipelineK) {
-        em_.line("__syncthreads();");
-        em_.line("const bool more_ = " + tk + " + 1 < " + std::to_string(k0.numTiles) + ";");
-        em_.open("if (more_)");
-        tileOverride[k0.name] = "(" + tk + " + 1)";
-        for (const auto& p : st_.promotions) {
-          if (!p.insideReductionTiles) continue;
-          declareLows(p);
-          emitCopyLoads(p, "pk_" + p.tensor + "_");
-        }
-        tileOverride.clear();
-        em_.close();
-        for (const auto& p : st_.promotions) {
-          if (!p.insideReductionTiles) continue;
-          declareLows(p);
-          activePromotions_.insert(p.tensor);
-        }
-      } else {
-        stagePromotions(true);
-      }
-      if (registerBlocked) {
-        const std::string steps = std::to_string(stepsPerWave);
+      const bool rotated = registerBlocked && pipelineK && twoCopies && bothStaged && stepsPerWave >= 2 && !forwardOf(loadA->name) &&
+          !forwardOf(loadB->name);
+      const int64_t halfSteps = stepsPerWave / 2;
+      // operand values of steps [first, last) of the wavefront's rectangle into ra_ / rb_
+      auto readOperands = [&](int64_t first, int64_t last) {
         em_.open("");
         em_.line("const int bt_ = 0;");
         em_.line("(void)bt_;");
         std::string bok = st_.mfmaBatch.empty() ? "true" : decodeGroup(st_.mfmaBatch, "bt_", true, true);
         em_.line("const bool bok_ = " + bok + ";");
         em_.line("(void)bok_;");
-        em_.line("float ra_[" + std::to_string(RM) + "][" + steps + "];");
-        em_.line("float rb_[" + std::to_string(RN) + "][" + steps + "];");
-        // the operand values of the whole reduction tile first ...
         em_.line("#pragma unroll");
         em_.open("for (int a_ = 0; a_ < " + std::to_string(RM) + "; ++a_)");
         em_.line("const int mt_ = (wv_ / " + std::to_string(blockWN) + ") * " + std::to_string(RM) + " + a_;");
@@ -2336,7 +2303,7 @@ class StageCodegen {
         em_.line("const bool moka_ = bok_ && " + decodeGroup(st_.mfmaM, "mposa_", true, MT % 16 == 0) + ";");
         em_.line("(void)moka_;");
         {
-          bool masked = openSteps(stepsPerWave);
+          bool masked = openSteps(stepsPerWave, first, last);
           em_.line("ra_[a_][ks_] = " + operandValue(loadA, masked) + ";");
           em_.close();
         }
@@ -2348,14 +2315,18 @@ class StageCodegen {
         em_.line("const bool nok_ = bok_ && " + decodeGroup(st_.mfmaN, "npos_", true, NT % 16 == 0) + ";");
         em_.line("(void)nok_;");
         {
-          bool masked = openSteps(stepsPerWave);
+          bool masked = openSteps(stepsPerWave, first, last);
           em_.line("rb_[b_][ks_] = " + operandValue(loadB, masked) + ";");
           em_.close();
         }
         em_.close();
-        // ... then the multiplications, step by step over all tiles of the rectangle
+        em_.close();
+      };
+      // the multiplications of steps [first, last), step by step over all tiles of the rectangle
+      auto multiplySteps = [&](int64_t first, int64_t last) {
+        if (first >= last) return;
         em_.line("#pragma unroll");
-        em_.open("for (int ks_ = 0; ks_ < " + steps + "; ++ks_)");
+        em_.open("for (int ks_ = " + std::to_string(first) + "; ks_ < " + std::to_string(last) + "; ++ks_)");
         em_.line("#pragma unroll");
         em_.open("for (int a_ = 0; a_ < " + std::to_string(RM) + "; ++a_)");
         em_.line("#pragma unroll");
@@ -2365,28 +2336,173 @@ class StageCodegen {
         em_.close();
         em_.close();
         em_.close();
-        em_.close();
-      } else {
-        em_.line("#pragma unroll");
-        em_.open("for (int j_ = 0; j_ < " + std::to_string(tilesPerWave) + "; ++j_)");
-        em_.line(tileDecl);
-        em_.open("if (" + worksOnTile + ")");
-        decodeTile();
-        multiply("cacc_[j_]");
-        em_.close();
-        em_.close();
-      }
-      if (pipelineK) {
-        if (!twoCopies) em_.line("__syncthreads();");
-        em_.open("if (more_)");
+      };
+      if (rotated) {
+        // Register stages of the staging copies: the loads of a tile are issued `stages` tiles
+        // ahead of the stores that wait for them (a tile of 32 reduction values is multiplied
+        // in about 0.4 us, a load that misses the L2 takes longer), one set of registers per
+        // tile in flight; the tile loop is unrolled by that number so that every set and both
+        // LDS copies are named statically.
+        const int64_t numK = k0.numTiles;
+        int64_t stages = 1;
+        while (stages < 4 && 2 * stages * stagingRegs <= 64 && numK >= 4 * stages && numK % (2 * stages) == 0) stages *= 2;
+        auto regs = [&](const Promotion& p, int64_t st) { return "pk" + std::to_string(st) + "_" + p.tensor + "_"; };
+        em_.open("");
+        ++opened;
+        for (int64_t st = 0; st < stages; ++st) {
+          for (const auto& p : st_.promotions) {
+            if (p.insideReductionTiles) em_.line(copyRegisterDecl(p, regs(p, st)));
+          }
+        }
+        em_.line("float ra_[" + std::to_string(RM) + "][" + std::to_string(stepsPerWave) + "];");
+        em_.line("float rb_[" + std::to_string(RN) + "][" + std::to_string(stepsPerWave) + "];");
+        auto loadTile = [&](const std::string& tile, int64_t st) {
+          em_.open("");
+          tileOverride[k0.name] = tile;
+          for (const auto& p : st_.promotions) {
+            if (!p.insideReductionTiles) continue;
+            declareLows(p);
+            emitCopyLoads(p, regs(p, st));
+          }
+          tileOverride.clear();
+          em_.close();
+        };
+        auto storeTile = [&](const std::string& buffer, int64_t st) {
+          writeBuffer_ = buffer;
+          for (const auto& p : st_.promotions) {
+            if (p.insideReductionTiles) emitCopyStores(p, regs(p, st));
+          }
+          writeBuffer_.clear();
+        };
+        auto readHalf = [&](const std::string& tile, const std::string& buffer, int64_t first, int64_t last) {
+          em_.open("");
+          tileOverride[k0.name] = tile;
+          readBuffer_ = buffer;
+          for (const auto& p : st_.promotions) {
+            if (p.insideReductionTiles) declareLows(p);
+          }
+          readOperands(first, last);
+          tileOverride.clear();
+          readBuffer_.clear();
+          em_.close();
+        };
+        loadTile("0", 0);
+        em_.line("__syncthreads();");
+        storeTile("0", 0);
+        for (int64_t j = 1; j <= stages; ++j) loadTile(std::to_string(std::min(j, numK - 1)), j % stages);
+        em_.line("__syncthreads();");
         for (const auto& p : st_.promotions) {
-          if (p.insideReductionTiles) emitCopyStores(p, "pk_" + p.tensor + "_");
+          if (p.insideReductionTiles) activePromotions_.insert(p.tensor);
+        }
+        readHalf("0", "0", 0, halfSteps);
+        const std::string t0 = tk + "0_", NK = std::to_string(numK), ST = std::to_string(stages);
+        em_.open("for (int " + t0 + " = 0; " + t0 + " < " + NK + "; " + t0 + " += " + ST + ")");
+        for (int64_t d = 0; d < stages; ++d) {
+          em_.open("");
+          em_.line("const int " + tk + " = " + t0 + " + " + std::to_string(d) + ";");
+          const bool staticCopy = stages % 2 == 0;
+          const std::string cur = staticCopy ? std::to_string(d & 1) : "(" + tk + " & 1)";
+          const std::string nxt = staticCopy ? std::to_string((d + 1) & 1) : "((" + tk + " + 1) & 1)";
+          const int64_t nextStage = (d + 1) % stages;
+          // second half of this tile's operand values, while the first half is multiplied
+          readHalf(tk, cur, halfSteps, stepsPerWave);
+          multiplySteps(0, halfSteps - 1);
+          em_.line("__builtin_amdgcn_sched_barrier(0);");
+          // (no branches in the loop body: with them the compiler waits for every load in flight
+          // ahead of a store instead of the oldest ones.  Past the last tile the loads fetch the
+          // last tile again and the stores and reads move values nobody multiplies.)
+          storeTile(nxt, nextStage);
+          loadTile("min(" + tk + " + " + std::to_string(1 + stages) + ", " + std::to_string(numK - 1) + ")", nextStage);
+          em_.line("__builtin_amdgcn_sched_barrier(0);");
+          // (one step of multiplications between the stores and the barrier that waits for them)
+          multiplySteps(halfSteps - 1, halfSteps);
+          em_.line("__syncthreads();");
+          readHalf("min(" + tk + " + 1, " + std::to_string(numK - 1) + ")", nxt, 0, halfSteps);
+          em_.line("__builtin_amdgcn_sched_barrier(0);"); // (the reads stay ahead of the multiplications that cover them)
+          multiplySteps(halfSteps, stepsPerWave);
+          em_.close();
         }
         em_.close();
+      } else {
+        if (pipelineK) {
+          em_.open("");
+          ++opened;
+          for (const auto& p : st_.promotions) {
+            if (p.insideReductionTiles) em_.line(copyRegisterDecl(p, "pk_" + p.tensor + "_"));
+          }
+          em_.open("");
+          em_.line("const int " + tk + " = 0;");
+          for (const auto& p : st_.promotions) {
+            if (!p.insideReductionTiles) continue;
+            declareLows(p);
+            emitCopyLoads(p, "pk_" + p.tensor + "_");
+          }
+          em_.line("__syncthreads();");
+          if (twoCopies) writeBuffer_ = "0";
+          for (const auto& p : st_.promotions) {
+            if (p.insideReductionTiles) emitCopyStores(p, "pk_" + p.tensor + "_");
+          }
+          writeBuffer_.clear();
+          em_.close();
+        }
+        em_.open("for (int " + tk + " = 0; " + tk + " < " + std::to_string(k0.numTiles) + "; ++" + tk + ")");
+        if (pipelineK && twoCopies) {
+          readBuffer_ = "(" + tk + " & 1)";
+          writeBuffer_ = "((" + tk + " + 1) & 1)";
+        }
+        if (pipelineK) {
+          em_.line("__syncthreads();");
+          em_.line("const bool more_ = " + tk + " + 1 < " + std::to_string(k0.numTiles) + ";");
+          em_.open("if (more_)");
+          tileOverride[k0.name] = "(" + tk + " + 1)";
+          for (const auto& p : st_.promotions) {
+            if (!p.insideReductionTiles) continue;
+            declareLows(p);
+            emitCopyLoads(p, "pk_" + p.tensor + "_");
+          }
+          tileOverride.clear();
+          em_.close();
+          // (the loads of the next tile are issued here, a whole tile of multiplications ahead of
+          // the stores that wait for them: the instruction scheduler would otherwise sink them next
+          // to those stores and every wavefront would sit out the memory latency once per tile)
+          em_.line("__builtin_amdgcn_sched_barrier(0);");
+          for (const auto& p : st_.promotions) {
+            if (!p.insideReductionTiles) continue;
+            declareLows(p);
+            activePromotions_.insert(p.tensor);
+          }
+        } else {
+          stagePromotions(true);
+        }
+        if (registerBlocked) {
+          em_.line("float ra_[" + std::to_string(RM) + "][" + std::to_string(stepsPerWave) + "];");
+          em_.line("float rb_[" + std::to_string(RN) + "][" + std::to_string(stepsPerWave) + "];");
+          // the operand values of the whole reduction tile first, then the multiplications
+          readOperands(0, stepsPerWave);
+          multiplySteps(0, stepsPerWave);
+        } else {
+          em_.line("#pragma unroll");
+          em_.open("for (int j_ = 0; j_ < " + std::to_string(tilesPerWave) + "; ++j_)");
+          em_.line(tileDecl);
+          em_.open("if (" + worksOnTile + ")");
+          decodeTile();
+          multiply("cacc_[j_]");
+          em_.close();
+          em_.close();
+        }
+        if (pipelineK) {
+          if (!twoCopies) em_.line("__syncthreads();");
+          else em_.line("__builtin_amdgcn_sched_barrier(0);"); // (nor may the stores rise among the multiplications)
+          em_.open("if (more_)");
+          for (const auto& p : st_.promotions) {
+            if (p.insideReductionTiles) emitCopyStores(p, "pk_" + p.tensor + "_");
+          }
+          em_.close();
+        }
+        readBuffer_.clear();
+        writeBuffer_.clear();
+        em_.close();
       }
-      readBuffer_.clear();
-      writeBuffer_.clear();
-      em_.close();
       if (split > 1) {
         em_.open("");
         em_.line(tileDecl);

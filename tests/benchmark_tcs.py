@@ -274,6 +274,28 @@ TUNED_AT_REFERENCE_SIZES = {
 }
 
 
+# Contractions large enough to fill the device: the transposed product at the size of the reference's
+# regression fixture TMM_128_1024_1024 (test/cuda/test_tc_mapper_bugs.cc:555-656) and square matrix
+# products.  name -> (key of CASES, input shapes, mapping options, reduction length)
+LARGE_CONTRACTIONS = {
+    "tmm_128_1024_1024": ("tmm", [(128, 1024), (1024, 1024)],
+                          "naive;tile=16,32,64;mapToThreads=64,8;mapToBlocks=256,256;useMfma=1;useSharedMemory=1;"
+                          "prefetchShared=1", 1024),
+    "matmul_1024": ("matmul", [(1024, 1024), (1024, 1024)],
+                    "naive;tile=64,64,32;mapToThreads=64,8;mapToBlocks=256,256;useMfma=1;useSharedMemory=1;"
+                    "prefetchShared=1", 1024),
+    "matmul_2048": ("matmul", [(2048, 2048), (2048, 2048)],
+                    "naive;tile=128,128,16;mapToThreads=64,8;mapToBlocks=256,256;useMfma=1;useSharedMemory=1;"
+                    "prefetchShared=1", 2048),
+}
+
+
+def make_large_inputs(name, seed=2024):
+    import numpy as np
+    rng = np.random.Generator(np.random.Philox(seed))
+    return [rng.standard_normal(shape, dtype=np.float32) for shape in LARGE_CONTRACTIONS[name][1]]
+
+
 def make_inputs(name, seed=2024, reference_sizes=False):
     import numpy as np
     rng = np.random.Generator(np.random.Philox(seed))

@@ -79,6 +79,25 @@ def test_parity_at_the_reference_sizes_with_the_tuned_options(name):
         assert np.abs(got - r).max() <= 1e-5 * np.sqrt(k) * scale, (name, ex.launch_bounds())
 
 
+@pytest.mark.parametrize("name", sorted(B.LARGE_CONTRACTIONS))
+def test_parity_of_the_large_contractions(name):
+    case, _, options, k = B.LARGE_CONTRACTIONS[name]
+    src, entry, _, _ = B.CASES[case]
+    print(f"case {name}", flush=True)
+    ins_np = B.make_large_inputs(name)
+    ref = tc_oracle.run(src, entry, ins_np)
+    ins = [torch.from_numpy(a).cuda() for a in ins_np]
+    ex = tc.compile(src, entry, ins, options)
+    outs = tc.prepare_outputs(src, entry, ins)
+    outs[0].fill_(float("nan"))
+    tc.run(ex, ins, outs)
+    torch.cuda.synchronize()
+    got = outs[0].cpu().numpy()
+    assert got.shape == ref[0].shape
+    scale = max(float(np.abs(ref[0]).max()), 1e-30)
+    assert np.abs(got - ref[0]).max() <= 1e-5 * np.sqrt(k) * scale, (name, ex.launch_bounds())
+
+
 def test_lookup_indices_are_exact():
     """Indirect indexing with integer-valued tables: sums are exact, any wrong row shows."""
     rng = np.random.Generator(np.random.Philox(5))
