@@ -279,7 +279,7 @@ TUNED_AT_REFERENCE_SIZES = {
 # products.  name -> (key of CASES, input shapes, mapping options, reduction length)
 LARGE_CONTRACTIONS = {
     "tmm_128_1024_1024": ("tmm", [(128, 1024), (1024, 1024)],
-                          "naive;tile=16,32,64;mapToThreads=64,8;mapToBlocks=256,256;useMfma=1;useSharedMemory=1;"
+                          "naive;tile=16,32,128;mapToThreads=64,8;mapToBlocks=256,256;useMfma=1;useSharedMemory=1;"
                           "prefetchShared=1", 1024),
     "matmul_1024": ("matmul", [(1024, 1024), (1024, 1024)],
                     "naive;tile=64,64,32;mapToThreads=64,8;mapToBlocks=256,256;useMfma=1;useSharedMemory=1;"
