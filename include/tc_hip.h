@@ -63,7 +63,11 @@ int tc_infer_output_info(
     tc_tensor_info* outputs, int capacity, int* count);
 
 /* tc::compile<HipBackend> (tc/core/compiler.h:71-78; tc::aten::compile, aten_compiler.h:56-62).
- * `options` is option text; see tc_options_* below. */
+ * `options` is option text; see tc_options_* below.  With the option reductionBlocks above 1 the
+ * kernels add floating-point partial sums with the hardware atomic (hipRTC gets
+ * -munsafe-fp-atomics for such sources only): the outputs must then lie in ordinary
+ * coarse-grained device memory (hipMalloc, a torch tensor), not in fine-grained or host-mapped
+ * allocations. */
 int tc_compile(
     const char* tc, const char* entry_point,
     const tc_dl_tensor* const* inputs, int num_inputs,

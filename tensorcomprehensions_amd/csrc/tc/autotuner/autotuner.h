@@ -341,12 +341,14 @@ inline std::vector<HipMappingOptions> heuristicSeeds(
     seeds.push_back(o);
   }
   if (matrix) {
-    // many output tiles: 64x64 per block, the reduction in tiles of 32 staged through LDS while
-    // the previous tile multiplies
-    {
+    // many output tiles: 64x64 per block (128x128 for outputs that fill the device with those),
+    // the reduction in tiles of 32 (16) staged through LDS while earlier tiles multiply; four
+    // wavefronts, or eight that own rectangles of output tiles
+    for (int variant = 0; variant < 3; ++variant) {
       HipMappingOptions o = base;
-      o.generic.tile(std::vector<uint64_t>{64, 64, 32});
-      o.mapToThreads(64, 4).mapToBlocks(largest, largest).useSharedMemory(true).useReadOnlyCache(true);
+      const uint64_t side = variant == 2 ? 128 : 64;
+      o.generic.tile(std::vector<uint64_t>{side, side, variant == 2 ? 16u : 32u});
+      o.mapToThreads(64, variant == 0 ? 4 : 8).mapToBlocks(largest, largest).useSharedMemory(true).useReadOnlyCache(true);
       o.useMfmaValue = true;
       o.prefetchSharedValue = true;
       seeds.push_back(o);

@@ -209,6 +209,44 @@ FC = """def fc(float(B, K) I, float(N, K) W1, float(N) B1) -> (O1) {
     O1(b, n) = fmax(O1(b, n), 0) }"""
 
 
+ROTATED_CASES = [
+    # (M, N, K, tile, wavefronts, register stages the tile loop is unrolled by)
+    (128, 128, 64, "64,64,32", 8, 1),     # two reduction tiles
+    (128, 128, 96, "64,64,32", 8, 1),     # three: an odd number of tiles keeps one stage
+    (128, 128, 128, "64,64,32", 4, 2),
+    (128, 128, 256, "64,64,32", 8, 4),
+    (100, 72, 160, "32,32,32", 4, 1),     # partial row and column tiles, five reduction tiles
+    (200, 136, 1000, "64,32,40", 4, 1),   # 25 reduction tiles of 10 steps
+    (64, 192, 384, "64,64,16", 8, 4),     # 24 tiles of 4 steps
+    (256, 256, 512, "128,128,16", 8, 4),
+]
+
+
+@pytest.mark.parametrize("transposed", [False, True])
+@pytest.mark.parametrize("m,n,k,tile,waves,stages", ROTATED_CASES)
+def test_rotated_pipeline_with_register_stages_is_exact(m, n, k, tile, waves, stages, transposed):
+    """Register-blocked, reduction-tiled products with two LDS copies: the operand values of the
+    next tile's first half are read behind the barrier while this tile's second half multiplies,
+    and the loads of up to four tiles are in flight (past the last tile they fetch it again)."""
+    src = ("def mm(float(M, K) A, float(N, K) B) -> (C) { C(m, n) +=! A(m, r_k) * B(n, r_k) }" if transposed else
+           "def mm(float(M, K) A, float(K, N) B) -> (C) { C(m, n) +=! A(m, r_k) * B(r_k, n) }")
+    rng = np.random.Generator(np.random.Philox(43))
+    A = rng.integers(-3, 4, size=(m, k)).astype(np.float32)
+    B = rng.integers(-3, 4, size=((n, k) if transposed else (k, n))).astype(np.float32)
+    ins = [torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()]
+    opts = f"naive;tile={tile};mapToThreads=64,{waves};mapToBlocks=256,256;useMfma=1;useSharedMemory=1;prefetchShared=1"
+    print(f"case {m}x{n}x{k} tile {tile} waves {waves} transposed {transposed}", flush=True)
+    ex = tc.compile(src, "mm", ins, opts)
+    source = ex.compiled_source
+    assert "pk0_A_" in source and "ra_[" in source, "not the rotated, register-blocked form"
+    assert (f"pk{stages - 1}_A_" in source) and (f"pk{stages}_A_" not in source), "number of register stages"
+    (C,) = tc.prepare_outputs(src, "mm", ins)
+    C.fill_(float("nan"))
+    tc.run(ex, ins, [C])
+    torch.cuda.synchronize()
+    assert np.array_equal(C.cpu().numpy(), A @ (B.T if transposed else B))     # small integers: exact in fp32
+
+
 @pytest.mark.parametrize("k,opts,split", [
     # one tile, 16 wavefronts, 128 steps: 16 slices of 8
     (512, "naive;tile=16,16;mapToThreads=512,2;mapToBlocks=64,64;useMfma=1", 16),
