@@ -1657,15 +1657,9 @@ class StageCodegen {
     const std::string kx = split > 1 ? "kq_" : "ks_"; // counter of a wavefront's own steps
     // Opens the loop over the reduction steps of a lane, decodes the reduction indices of the
     // step and declares kok_ when surplus steps exist; returns whether it did.
-    auto openSteps = [&](int64_t count, int64_t first = 0, int64_t last = -1) {
-      em_.line(count <= 128 ? "#pragma unroll" : "#pragma unroll 4");
-      if (split > 1) {
-        // slice sl_ of the steps: ks_ is the step within the whole reduction
-        em_.open("for (int kq_ = 0; kq_ < " + std::to_string(count) + "; ++kq_)");
-        em_.line("const int ks_ = sl_ * " + std::to_string(stepsPerWave) + " + kq_;");
-      } else {
-        em_.open("for (int ks_ = " + std::to_string(first) + "; ks_ < " + std::to_string(last < 0 ? ksteps : last) + "; ++ks_)");
-      }
+    // Decodes the reduction indices of step ks_ and declares kok_ when surplus steps exist;
+    // returns whether it did.
+    auto declareStepIndices = [&]() {
       std::string kok;
       if (aligned) {
         int64_t div = innerProd;
@@ -1693,6 +1687,33 @@ class StageCodegen {
       }
       if (!kok.empty()) em_.line("const bool kok_ = " + kok + ";");
       return !kok.empty();
+    };
+    auto openSteps = [&](int64_t count, int64_t first = 0, int64_t last = -1) {
+      em_.line(count <= 128 ? "#pragma unroll" : "#pragma unroll 4");
+      if (split > 1) {
+        // slice sl_ of the steps: ks_ is the step within the whole reduction
+        em_.open("for (int kq_ = " + std::to_string(first) + "; kq_ < " + std::to_string(last < 0 ? count : last) + "; ++kq_)");
+        em_.line("const int ks_ = sl_ * " + std::to_string(stepsPerWave) + " + kq_;");
+      } else {
+        em_.open("for (int ks_ = " + std::to_string(first) + "; ks_ < " + std::to_string(last < 0 ? ksteps : last) + "; ++ks_)");
+      }
+      return declareStepIndices();
+    };
+    // An operand read straight from global memory whose elements of consecutive steps of a lane
+    // are consecutive in memory (the reduction subscripts are jointly contiguous): four steps
+    // can then be fetched with one 16-byte load.
+    auto contiguousAlongSteps = [&](const ExprRef& load) {
+      if (!aligned || quarter * 4 != KT || activePromotions_.count(load->name) || forwardOf(load->name)) return false;
+      if (st_.views.at(load->name).type.bits != 32) return false;
+      Affine fa = flatAffine(load->name, load->args);
+      if (!fa.valid) return false;
+      int64_t expect = 1;
+      for (size_t i = st_.mfmaK.size(); i-- > 0;) {
+        const LoopVar& v = var(st_.mfmaK[i]);
+        if (fa.coefOf(v.name) != expect) return false;
+        expect *= v.tile;
+      }
+      return true;
     };
     // surplus reduction steps must contribute exact zeros
     auto operandValue = [&](const ExprRef& load, bool masked) {
@@ -1908,10 +1929,41 @@ class StageCodegen {
           // but their own operands (10.5 -> 10.0 us on the 16-channel 3x3 group convolution).
           em_.line("float bq_[" + std::to_string(count) + "];");
           if (!resident) em_.line("float aq_[" + std::to_string(count) + "];");
-          bool masked = openSteps(count);
-          if (!resident) em_.line("aq_[" + kx + "] = " + operandValue(loadA, masked) + ";");
-          em_.line("bq_[" + kx + "] = " + operandValue(loadB, masked) + ";");
-          em_.close();
+          // operands whose steps are consecutive in memory: 16-byte loads for groups of four
+          // steps, single loads for the rest (a lane of the 128x1000x1024 matmul fetches its 63
+          // values of the first operand with 15 + 3 loads instead of 63, each of which touched
+          // 64 cache lines per wavefront)
+          auto vectorLoads = [&](const ExprRef& load, const std::string& regs) {
+            const int64_t groups = count / 4;
+            em_.line("#pragma unroll");
+            em_.open("for (int kv_ = 0; kv_ < " + std::to_string(groups) + "; ++kv_)");
+            if (split > 1) {
+              em_.line("const int kq_ = 4 * kv_;");
+              em_.line("const int ks_ = sl_ * " + std::to_string(stepsPerWave) + " + kq_;");
+            } else {
+              em_.line("const int ks_ = 4 * kv_;");
+            }
+            declareStepIndices();
+            em_.line("const __tc::floatx4 v_ = *(const __tc::floatx4u*)&p" + load->name + "[" + flatIndex(load->name, load->args, "") + "];");
+            em_.line(regs + "[" + kx + "] = v_[0]; " + regs + "[" + kx + " + 1] = v_[1]; " + regs + "[" + kx + " + 2] = v_[2]; " + regs +
+                     "[" + kx + " + 3] = v_[3];");
+            em_.close();
+            if (groups * 4 < count) {
+              openSteps(count, groups * 4, count);
+              em_.line(regs + "[" + kx + "] = " + operandValue(load, false) + ";");
+              em_.close();
+            }
+          };
+          const bool vectorA = !resident && count >= 4 && contiguousAlongSteps(loadA);
+          const bool vectorB = count >= 4 && contiguousAlongSteps(loadB);
+          if (vectorA) vectorLoads(loadA, "aq_");
+          if (vectorB) vectorLoads(loadB, "bq_");
+          if ((!resident && !vectorA) || !vectorB) {
+            bool masked = openSteps(count);
+            if (!resident && !vectorA) em_.line("aq_[" + kx + "] = " + operandValue(loadA, masked) + ";");
+            if (!vectorB) em_.line("bq_[" + kx + "] = " + operandValue(loadB, masked) + ";");
+            em_.close();
+          }
           em_.line("#pragma unroll");
           em_.open("for (int " + kx + " = 0; " + kx + " < " + std::to_string(count) + "; ++" + kx + ")");
           em_.line(acc + " = __builtin_amdgcn_mfma_f32_16x16x4f32(" + (resident ? "am_" : "aq_") + "[" + kx + "], bq_[" + kx + "], " +
