@@ -325,6 +325,7 @@ inline std::vector<HipMappingOptions> heuristicSeeds(
       HipMappingOptions o = base;
       o.generic.tile(std::vector<uint64_t>{1, wide ? 32u : 16u, band, 0, wide ? 8u : 16u});
       o.mapToThreads(64, wide ? 8 : 4).mapToBlocks(largest, 256, 256).useSharedMemory(true).useReadOnlyCache(true);
+      o.sharedDepth(7);
       o.useMfmaValue = true;
       o.prefetchSharedValue = wide;
       seeds.push_back(o);
@@ -349,6 +350,7 @@ inline std::vector<HipMappingOptions> heuristicSeeds(
       const uint64_t side = variant == 2 ? 128 : 64;
       o.generic.tile(std::vector<uint64_t>{side, side, variant == 2 ? 16u : 32u});
       o.mapToThreads(64, variant == 0 ? 4 : 8).mapToBlocks(largest, largest).useSharedMemory(true).useReadOnlyCache(true);
+      o.sharedDepth(7); // (a depth beyond the parallel dimensions: the copies stay inside the reduction tile loop)
       o.useMfmaValue = true;
       o.prefetchSharedValue = true;
       seeds.push_back(o);

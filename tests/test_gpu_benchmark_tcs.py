@@ -98,6 +98,35 @@ def test_parity_of_the_large_contractions(name):
     assert np.abs(got - ref[0]).max() <= 1e-5 * np.sqrt(k) * scale, (name, ex.launch_bounds())
 
 
+def test_autotuning_the_1024_matmul_from_the_naive_options_reaches_the_stored_options():
+    """A short, seeded search from the naive options ends within 15 % of the stored options of the
+    1024 x 1024 x 1024 product (reduction tiles staged through two LDS copies, loads of several
+    tiles in flight), and its winner computes the oracle's values."""
+    case, _, stored, k = B.LARGE_CONTRACTIONS["matmul_1024"]
+    src, entry, _, _ = B.CASES[case]
+    ins_np = B.make_large_inputs("matmul_1024")
+    ins = [torch.from_numpy(a).cuda() for a in ins_np]
+    outs = tc.prepare_outputs(src, entry, ins)
+
+    def kernel_us(options):
+        ex = tc.compile(src, entry, ins, options)
+        for _ in range(20):
+            tc.profile_repeated(ex, ins, outs, 100)
+        return min(tc.profile_repeated(ex, ins, outs, 50) / 50 for _ in range(5))
+
+    best = tc.autotune(src, entry, ins, "naive", outputs=outs, generations=3, pop_size=30, threads=16, seed=1)
+    t_stored, t_tuned = kernel_us(stored), kernel_us(best[0])
+    print(f"matmul_1024: stored {t_stored:.1f} us, tuned from naive {t_tuned:.1f} us with {best[0]}", flush=True)
+    assert t_tuned <= 1.15 * t_stored
+    ex = tc.compile(src, entry, ins, best[0])
+    outs[0].fill_(float("nan"))
+    tc.run(ex, ins, outs)
+    torch.cuda.synchronize()
+    ref = tc_oracle.run(src, entry, ins_np)[0]
+    scale = max(float(np.abs(ref).max()), 1e-30)
+    assert np.abs(outs[0].cpu().numpy() - ref).max() <= 1e-5 * np.sqrt(k) * scale
+
+
 def test_lookup_indices_are_exact():
     """Indirect indexing with integer-valued tables: sums are exact, any wrong row shows."""
     rng = np.random.Generator(np.random.Philox(5))
