@@ -71,6 +71,25 @@ template <typename Op, typename T> __device__ __forceinline__ void atomicCombine
     }
   }
 }
+// Value of lane ^ MASK for MASK = 16 or 32, through v_permlane16_swap_b32 / v_permlane32_swap_b32
+// (gfx950: rows, respectively halves, of two registers change places in the vector ALU; a
+// ds_bpermute would go through the LDS crossbar and its wait counter).  With both operands equal
+// to u the instruction leaves {even rows | low half} of u everywhere in the first result and
+// {odd rows | high half} in the second: a lane takes the one its partner lives in.
+template <int MASK> __device__ __forceinline__ unsigned laneXor32(unsigned u) {
+  static_assert(MASK == 16 || MASK == 32, "partner across 16-lane rows or across the halves of a wavefront");
+  const unsigned lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+  if constexpr (MASK == 16) {
+    const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    return (lane & 16u) ? r[0] : r[1];
+  } else {
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return (lane & 32u) ? r[0] : r[1];
+  }
+}
+template <int MASK> __device__ __forceinline__ float laneXor32(float v) {
+  return __builtin_bit_cast(float, laneXor32<MASK>(__builtin_bit_cast(unsigned, v)));
+}
 template <typename T> __device__ __forceinline__ T tmin(T a, T b) { return a < b ? a : b; }
 template <typename T> __device__ __forceinline__ T tmax(T a, T b) { return a > b ? a : b; }
 __device__ __forceinline__ float tmin(float a, float b) { return fminf(a, b); }
@@ -120,16 +139,19 @@ template <int CTRL, typename T> __device__ __forceinline__ T dppMov(T v) {
     return (T)dppMov32<CTRL>((int)v);
   }
 }
-// exchange with lane ^ MASK across the 16-lane rows of a wavefront
+// exchange with lane ^ MASK (16 or 32) across the 16-lane rows of a wavefront
 template <int MASK, typename T> __device__ __forceinline__ T laneXor(T v) {
   if constexpr (sizeof(T) == 8) {
-    return __builtin_bit_cast(T, __shfl_xor(__builtin_bit_cast(unsigned long long, v), MASK, 64));
+    const unsigned long long b = __builtin_bit_cast(unsigned long long, v);
+    const unsigned lo = laneXor32<MASK>((unsigned)(b & 0xffffffffULL));
+    const unsigned hi = laneXor32<MASK>((unsigned)(b >> 32));
+    return __builtin_bit_cast(T, ((unsigned long long)hi << 32) | lo);
   } else if constexpr (sizeof(T) == 4) {
-    return __builtin_bit_cast(T, __shfl_xor(__builtin_bit_cast(int, v), MASK, 64));
+    return __builtin_bit_cast(T, laneXor32<MASK>(__builtin_bit_cast(unsigned, v)));
   } else if constexpr (sizeof(T) == 2) {
-    return __builtin_bit_cast(T, (unsigned short)__shfl_xor((int)__builtin_bit_cast(unsigned short, v), MASK, 64));
+    return __builtin_bit_cast(T, (unsigned short)laneXor32<MASK>((unsigned)__builtin_bit_cast(unsigned short, v)));
   } else {
-    return (T)__shfl_xor((int)v, MASK, 64);
+    return (T)(int)laneXor32<MASK>((unsigned)(int)v);
   }
 }
 

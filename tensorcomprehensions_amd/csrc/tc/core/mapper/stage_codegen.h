@@ -2071,8 +2071,8 @@ class StageCodegen {
       em_.line("#pragma unroll");
       em_.open("for (int r_ = 0; r_ < 4; ++r_)");
       em_.line("float v_ = c_[r_];");
-      em_.line("v_ += __shfl_xor(v_, 16, 64);");
-      em_.line("v_ += __shfl_xor(v_, 32, 64);");
+      em_.line("v_ += __tc::laneXor32<16>(v_);");
+      em_.line("v_ += __tc::laneXor32<32>(v_);");
       em_.line("c_[r_] = v_;");
       em_.close();
       em_.close();
