@@ -331,6 +331,17 @@ inline std::vector<HipMappingOptions> heuristicSeeds(
       seeds.push_back(o);
     }
   }
+  // small batched contractions on the matrix cores: one element of the leading (batch-like)
+  // dimensions per block, its whole output tile over four wavefronts, operands through LDS
+  if (firstOutputShape.size() >= 3) {
+    HipMappingOptions o = base;
+    std::vector<uint64_t> tile(firstOutputShape.size(), 0);
+    for (size_t i = 0; i < std::max<size_t>(1, firstOutputShape.size() - 3); ++i) tile[i] = 1;
+    o.generic.tile(tile);
+    o.mapToThreads(64, 4).mapToBlocks(largest, largest).useSharedMemory(true).useReadOnlyCache(true);
+    o.useMfmaValue = true;
+    seeds.push_back(o);
+  }
   // dense contractions on the matrix cores: a 32x32 output tile per block (of one batch element,
   // when the output has more than two dimensions), operands from memory or through LDS
   const bool matrix = firstOutputShape.size() == 2;
