@@ -132,7 +132,11 @@ int tc_map(
     char** source, int* num_kernels, unsigned* grids /* [8][3] */, unsigned* blocks /* [8][3] */);
 
 /* Front-end dumps in the format of the reference's golden files (tc/lang/test_expected/).
- * what: "lexer", "exp", "stmt", "function", "sema", "sema_env", "canonical" */
+ * what: "lexer", "exp", "stmt", "function", "sema", "sema_env", "canonical"; and "ranges":
+ * size-parametric range inference of one definition (tc/core/tc2halide.cc:270-498) — the bounds
+ * of every tensor as expressions of the size parameters in the layout of the reference's
+ * inference tests (test/test_inference.cc:28-67: "mins:" / "extents:" blocks, '//' for floor
+ * division), followed by "statements:" with the range of every index variable. */
 int tc_lang_dump(const char* text, const char* what, char** out);
 
 /* ATenAutotuner<HipBackend, GeneticSearch>::tune (tc/aten/aten_autotuner.h:79-84,

@@ -275,3 +275,4 @@ def load_from_cache(tc, entry_point, inputs, cache_file, count=1):
 from .highlevel import (TC, TunerConfig, assert_almost_equal, autotune_and_compile, define,  # noqa: E402
                         make_autograd, make_autotuned_options_factory, make_load_from_cache_options_factory,
                         make_naive_options_factory)
+from .symbolic import SymbolicRanges, infer_ranges  # noqa: E402

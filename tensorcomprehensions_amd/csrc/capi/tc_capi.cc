@@ -1,5 +1,6 @@
 // C ABI over the C++ library (declared in include/tc_hip.h).  Exceptions stop here: each entry
 // point catches, stores the message per thread and returns a non-zero status.
+#include "tc/core/symbolic_ranges.h"
 #include "tc_hip.h"
 
 #include <cstdlib>
@@ -288,6 +289,16 @@ int tc_lang_dump(const char* text, const char* what, char** out) {
     tc::CompilerOptions quiet;
     quiet.emitWarnings = false;
     ss << lang::canonicalize(lang::Sema(quiet).checkFunction(lang::Parser(text).parseFunction()));
+  } else if (w == "ranges") {
+    // size-parametric range inference: tensor bounds in the layout of the reference's inference
+    // tests (test/test_inference.cc:28-67), then the ranges of every statement's variables
+    tc::symbolic::FunctionRanges r = tc::symbolic::inferRanges(lang::Parser(text).parseFunction(), compilerOptions);
+    ss << r.dump() << "statements:\n";
+    for (const auto& st : r.statements) {
+      ss << st.tensor << ":";
+      for (const auto& v : st.vars) ss << " " << v.first << " in [" << r.text(v.second.min) << ", " << r.text(v.second.max) << "];";
+      ss << "\n";
+    }
   } else {
     TC_CHECK(false) << "unknown dump kind " << w;
   }

@@ -122,7 +122,7 @@ int main(int argc, char** argv) {
     for (auto& x : tensors) ptrs.push_back(&x.t);
     ++records;
     // front end alone
-    for (const char* what : {"function", "sema", "canonical"}) {
+    for (const char* what : {"function", "sema", "canonical", "ranges"}) {
       char* dump = nullptr;
       if (tc_lang_dump(text.c_str(), what, &dump) == 0) tc_free(dump);
     }
@@ -144,6 +144,7 @@ int main(int argc, char** argv) {
       }
       char* dump = nullptr;
       if (tc_lang_dump(m.c_str(), "sema", &dump) == 0) tc_free(dump);
+      if (tc_lang_dump(m.c_str(), "ranges", &dump) == 0) tc_free(dump);
       tc_infer_output_info(m.c_str(), entry.c_str(), ptrs.data(), static_cast<int>(ptrs.size()), infos, 16, &count);
       char* source = nullptr;
       int kernels = 0;
