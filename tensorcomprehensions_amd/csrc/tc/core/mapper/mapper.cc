@@ -100,10 +100,6 @@ bool sameExpr(const ExprRef& a, const ExprRef& b) {
   return true;
 }
 
-bool affineEqual(const Affine& a, const Affine& b) {
-  return a.valid && b.valid && a.coef == b.coef && a.constant == b.constant;
-}
-
 ScalarType matchType(const ScalarType& a, const ScalarType& b) {
   if (a == b) return a;
   if (!a.isFloat() && b.isFloat()) return b;

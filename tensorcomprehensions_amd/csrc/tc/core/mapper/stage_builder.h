@@ -47,19 +47,6 @@ bool sameBox(const ir::Statement& a, const ir::Statement& b) {
   return true;
 }
 
-std::set<std::string> tensorsRead(const ir::Statement& s) {
-  std::set<std::string> r;
-  visit(s.rhs, [&](const ExprRef& e) {
-    if (e->kind == Expr::Load) {
-      r.insert(e->name);
-    }
-  });
-  if (s.op != ReduceOp::None && !s.init) {
-    r.insert(s.tensor);
-  }
-  return r;
-}
-
 // Largest d such that the dependence between stages A (earlier) and B is point-wise in the
 // first d left-hand-side positions of both, or -1 when they cannot share a kernel.
 int sharedPrefix(const RawStage& A, const RawStage& B) {
