@@ -2438,10 +2438,12 @@ class StageCodegen {
           readBuffer_.clear();
           em_.close();
         };
-        loadTile("0", 0);
+        // (the loads of the first tiles all leave before the first of them is waited for: one
+        // memory latency ahead of the loop instead of two)
+        for (int64_t j = 0; j < stages; ++j) loadTile(std::to_string(std::min(j, numK - 1)), j);
         em_.line("__syncthreads();");
         storeTile("0", 0);
-        for (int64_t j = 1; j <= stages; ++j) loadTile(std::to_string(std::min(j, numK - 1)), j % stages);
+        loadTile(std::to_string(std::min(stages, numK - 1)), 0);
         em_.line("__syncthreads();");
         for (const auto& p : st_.promotions) {
           if (p.insideReductionTiles) activePromotions_.insert(p.tensor);
@@ -2468,6 +2470,9 @@ class StageCodegen {
           em_.line("__builtin_amdgcn_sched_barrier(0);");
           // (one step of multiplications between the stores and the barrier that waits for them)
           multiplySteps(halfSteps - 1, halfSteps);
+          // (and they stay there: the scheduler would lift the barrier, which is no memory
+          // operation to the multiplications, above all but one of them)
+          em_.line("__builtin_amdgcn_sched_barrier(0);");
           em_.line("__syncthreads();");
           readHalf("min(" + tk + " + 1, " + std::to_string(numK - 1) + ")", nxt, 0, halfSteps);
           em_.line("__builtin_amdgcn_sched_barrier(0);"); // (the reads stay ahead of the multiplications that cover them)
