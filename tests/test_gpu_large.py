@@ -43,6 +43,39 @@ def test_offsets_beyond_32_bits(options):
     assert np.array_equal(got, ref_Y)
 
 
+@pytest.mark.parametrize("options", [
+    # reduction tiles staged through two LDS copies, loads of four tiles in flight
+    "naive;tile=64,64,32;mapToThreads=64,8;mapToBlocks=1024,1;useMfma=1;useSharedMemory=1;prefetchShared=1",
+    # operands straight from memory, the reduction of a tile split over four wavefronts
+    "naive;tile=16,32;unroll=256;mapToThreads=256,2;mapToBlocks=4096,2;useSharedMemory=1;useReadOnlyCache=1;useMfma=1",
+])
+def test_matrix_core_product_with_an_operand_of_2_to_the_31_elements(options):
+    """A(65536 x 32768) . B(32768 x 64) in fp32: 8 GiB for the first operand, built on the device.
+    A(m, k) = ((m + k) mod 3) - 1 and B(k, n) = 1 + (n mod 2) are small integers, so every sum is
+    exact in fp32 and has a closed form: the residues of (m + k) mod 3 over k = 0 .. K-1 occur
+    c0, c1, c2 times and C(m, n) = (c2 - c0) * (1 + n mod 2)."""
+    mm = "def mm(float(M, K) A, float(K, N) B) -> (C) { C(m, n) +=! A(m, r_k) * B(r_k, n) }"
+    m_, k_, n_ = 65536, 32768, 64
+    rows = torch.arange(m_, device="cuda", dtype=torch.int32).unsqueeze(1)
+    cols = torch.arange(k_, device="cuda", dtype=torch.int32).unsqueeze(0)
+    A = (((rows + cols) % 3) - 1).to(torch.float32)
+    del rows, cols
+    B = (1 + (torch.arange(n_, device="cuda") % 2)).to(torch.float32).repeat(k_, 1).contiguous()
+    print(f"case {options}", flush=True)
+    ex = tc.compile(mm, "mm", [A, B], options)
+    assert "(int64)" in ex.compiled_source
+    (C,) = tc.prepare_outputs(mm, "mm", [A, B])
+    C.fill_(float("nan"))
+    tc.run(ex, [A, B], [C])
+    torch.cuda.synchronize()
+    got = C.cpu().numpy()
+    # residue r of (m + k) mod 3 occurs for k = (r - m) mod 3, +3, ...: count = ceil((K - first) / 3)
+    mrow = np.arange(m_, dtype=np.int64)
+    count = lambda r: (k_ - ((r - mrow) % 3) + 2) // 3
+    expected = np.outer(count(2) - count(0), 1 + (np.arange(n_) % 2)).astype(np.float32)
+    assert np.array_equal(got, expected)
+
+
 def test_a_single_dimension_of_2_to_the_31_is_refused():
     with pytest.raises(tc.TcError) as e:
         tc.compile("def f(int8(N) A) -> (B) { B(i) = A(i) }", "f", [tc.ShapeOnly((2 ** 31 + 8,), "int8")], "naive")
