@@ -338,6 +338,14 @@ def suite_library_routines():
             g[None, :, :, None, None] * (i - mean[:, :, None, None, None]) * torch.rsqrt(var[:, :, None, None, None] + 1e-5)
             + b[None, :, :, None, None]),
         "moments2": lambda x: (x.mean(1), x.var(1, unbiased=False)),
+        "sum": lambda x: x.sum(1),
+        "mean": lambda x: x.mean(1),
+        "sum_squares": lambda x: (x * x).sum(1),
+        "var": lambda x, mean: (x * x).mean(1) - mean * mean,
+        "sum_and_squares": lambda x: (x.sum(1), (x * x).sum(1)),
+        "kronecker3_1": lambda w2, x: torch.einsum("mabc,kc->mabk", x, w2),
+        "kronecker3_2": lambda w1, x: torch.einsum("mabk,jb->majk", x, w1),
+        "kronecker3_3": lambda w0, x: torch.einsum("majk,ia->mijk", x, w0),
         "group_normalization_single_kernel": lambda i, g, b: F.group_norm(
             i.reshape(i.shape[0], -1, i.shape[3], i.shape[4]), i.shape[1], g.reshape(-1), b.reshape(-1), 1e-5),
         "kronecker3": lambda w0, w1, w2, x: torch.einsum("mabc,ia,jb,kc->mijk", x, w0, w1, w2),

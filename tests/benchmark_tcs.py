@@ -106,6 +106,54 @@ def moments2_2D_1D(float(N, K) I) -> (mean, var) {
 }
 """
 
+# The single statistics of tc/benchmarks/moments.h:29-51 (the program times each of them beside the
+# combined moments2_2D_1D above, moments.cc:162-303).
+SUM = """
+def sum_2D_1D(float(N, K) I) -> (sum) {
+    sum(n) +=! I(n, r_k)
+}
+"""
+MEAN = """
+def mean_2D_1D(float(N, K) I) -> (mean) {
+    mean(n) +=! I(n, r_k)
+    mean(n) = mean(n) / (K)
+}
+"""
+SUM_SQUARES = """
+def sum_squares_2D_1D(float(N, K) I) -> (sum_squares) {
+    sum_squares(n) +=! I(n, r_k) * I(n, r_k)
+}
+"""
+VAR = """
+def var_2D_1D(float(N, K) I, float(N) mean) -> (var) {
+    var(n) +=! I(n, r_k) * I(n, r_k)
+    var(n) = var(n) / (K) - mean(n) * mean(n)
+}
+"""
+SUM_AND_SQUARES = """
+def sum_and_squares_2D_1D(float(N, K) I) -> (sum, sum_squares) {
+    sum(n) +=! I(n, r_k)
+    sum_squares(n) +=! I(n, r_k) * I(n, r_k)
+}
+"""
+
+# The three steps of the Kronecker product as comprehensions of their own (tc/benchmarks/kronecker.h:124-140).
+KRONECKER3_1 = """
+def Kronecker3_1(float(D2, N2) W2, float(M, N0, N1, N2) X) -> (XW2) {
+    XW2(m, n0, n1, d2) +=! X(m, n0, n1, r_n2) * W2(d2, r_n2)
+}
+"""
+KRONECKER3_2 = """
+def Kronecker3_2(float(D1, N1) W1, float(M, N0, N1, D2) XW2) -> (XW2W1) {
+    XW2W1(m, n0, d1, d2) +=! XW2(m, n0, r_n1, d2) * W1(d1, r_n1)
+}
+"""
+KRONECKER3_3 = """
+def Kronecker3_3(float(D0, N0) W0, float(M, N0, D1, D2) XW2W1) -> (Y) {
+    Y(m, d0, d1, d2) +=! XW2W1(m, r_n0, d1, d2) * W0(d0, r_n0)
+}
+"""
+
 GROUP_NORMALIZATION = """
 def group_normalization(float(N, G, D, H, W) I, float(G, D) gamma, float(G, D) beta,
                         float(N, G) mean, float(N, G) var) -> (O) {
@@ -195,6 +243,14 @@ CASES = {
     "batchnorm": (BATCHNORM, "spatialBatchNorm",
                   [("scalar", 0.1), ("scalar", 1e-5), (4, 6, 7, 5), (6,), ("positive", (6,))], 4 * 7 * 5),   # N*H*W per channel
     "moments2": (MOMENTS2, "moments2_2D_1D", [(24, 500)], 500),
+    "sum": (SUM, "sum_2D_1D", [(24, 500)], 500),
+    "mean": (MEAN, "mean_2D_1D", [(24, 500)], 500),
+    "sum_squares": (SUM_SQUARES, "sum_squares_2D_1D", [(24, 500)], 500),
+    "var": (VAR, "var_2D_1D", [(24, 500), (24,)], 500),
+    "sum_and_squares": (SUM_AND_SQUARES, "sum_and_squares_2D_1D", [(24, 500)], 500),
+    "kronecker3_1": (KRONECKER3_1, "Kronecker3_1", [(8, 3), (10, 5, 4, 3)], 3),
+    "kronecker3_2": (KRONECKER3_2, "Kronecker3_2", [(7, 4), (10, 5, 4, 8)], 4),
+    "kronecker3_3": (KRONECKER3_3, "Kronecker3_3", [(6, 5), (10, 5, 7, 8)], 5),
     "group_normalization": (GROUP_NORMALIZATION, "group_normalization",
                             [(3, 4, 5, 6, 7), (4, 5), (4, 5), (3, 4), ("positive", (3, 4))], 1),
     "group_normalization_single_kernel": (GROUP_NORMALIZATION_SINGLE_KERNEL, "group_normalization_single_kernel",
@@ -222,6 +278,14 @@ REFERENCE_SIZES = {
     "lut": [(100000, 64), ("int", (128, 50), 0, 100000)],
     "2lut": [(100000, 64), ("int", (128, 50), 0, 100000), (100000, 64), ("int", (128, 50), 0, 100000)],
     "moments2": [(1024, 36864)],
+    "sum": [(1024, 36864)],
+    "mean": [(1024, 36864)],
+    "sum_squares": [(1024, 36864)],
+    "var": [(1024, 36864), (1024,)],
+    "sum_and_squares": [(1024, 36864)],
+    "kronecker3_1": [(32, 16), (256, 16, 16, 16)],
+    "kronecker3_2": [(32, 16), (256, 16, 16, 32)],
+    "kronecker3_3": [(32, 16), (256, 16, 32, 32)],
     "group_normalization": [(32, 32, 16, 48, 48), (32, 16), (32, 16), (32, 32), ("positive", (32, 32))],
     "group_normalization_single_kernel": [(32, 32, 16, 48, 48), (32, 16), (32, 16)],
     "kronecker3": [(32, 16), (32, 16), (32, 16), (256, 16, 16, 16)],
@@ -268,6 +332,23 @@ TUNED_AT_REFERENCE_SIZES = {
     "kronecker3": "naive;outerScheduleFusionStrategy=Max;intraTileScheduleFusionStrategy=Max;tile=1,16,0,0,8;unroll=8;"
                   "tileImperfectlyNested=1;mapToThreads=64,16;mapToBlocks=256,256,256;useSharedMemory=1;useReadOnlyCache=1;"
                   "privateDepth=5;collapseContiguous=0;useMfma=1;prefetchShared=1",
+    # one statistic per pass: a wavefront (or a few) per row in lanes of four reaches 7.2-7.4 TB/s
+    "sum": "naive;outerScheduleFusionStrategy=Min;tile=1,0;unroll=256;matchLibraryCalls=1;mapToThreads=64;mapToBlocks=1024,1;"
+           "usePrivateMemory=1;useReadOnlyCache=1;sharedDepth=3;vectorWidth=4;prefetchShared=1",
+    "mean": "naive;outerScheduleFusionStrategy=Max;tile=1,0;unroll=16;matchLibraryCalls=1;mapToThreads=128;mapToBlocks=36864,256;"
+            "usePrivateMemory=1;useReadOnlyCache=1;vectorWidth=4",
+    "sum_squares": "naive;outerScheduleFusionStrategy=Max;intraTileScheduleFusionStrategy=Min;tile=1,0;unroll=256;matchLibraryCalls=1;"
+                   "mapToThreads=64;mapToBlocks=36864,1;usePrivateMemory=1;useReadOnlyCache=1;vectorWidth=4;prefetchShared=1",
+    "var": "naive;outerScheduleFusionStrategy=Max;intraTileScheduleFusionStrategy=Max;tile=2;unroll=16;matchLibraryCalls=1;"
+           "mapToThreads=256,1;mapToBlocks=1024,1;useSharedMemory=1;useReadOnlyCache=1;vectorWidth=4;prefetchShared=1",
+    "sum_and_squares": "naive;outerScheduleFusionStrategy=Max;tile=1,0;unroll=8;matchLibraryCalls=1;mapToThreads=256;"
+                       "mapToBlocks=36864,256;usePrivateMemory=1;useReadOnlyCache=1;vectorWidth=4",
+    "kronecker3_1": "naive;tile=256,0,0,2;unroll=64;mapToThreads=128,4;mapToBlocks=256,256;usePrivateMemory=1;useReadOnlyCache=1;"
+                    "useMfma=1;prefetchShared=1",
+    "kronecker3_2": "naive;intraTileScheduleFusionStrategy=Max;tile=1,1,256,0,64;unroll=32;mapToThreads=128;mapToBlocks=128,256,1;"
+                    "useSharedMemory=1;useReadOnlyCache=1;vectorWidth=2;collapseContiguous=0;useMfma=1;prefetchShared=1",
+    "kronecker3_3": "naive;tile=1,32,0,0;unroll=1;mapToThreads=128,4;mapToBlocks=256,8;useSharedMemory=1;unrollCopyShared=1;"
+                    "useReadOnlyCache=1;vectorWidth=2;useMfma=1",
     "wavenet1": "naive;intraTileScheduleFusionStrategy=Max;fixParametersBeforeScheduling=1;tile=2,2000,16,1;mapToThreads=16,64;"
                 "mapToBlocks=2000,256;useSharedMemory=1;usePrivateMemory=1;privateDepth=8;sharedDepth=3;vectorWidth=4;"
                 "collapseContiguous=0;prefetchShared=1",

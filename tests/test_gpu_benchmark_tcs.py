@@ -70,7 +70,9 @@ def test_parity_at_the_reference_sizes_with_the_tuned_options(name):
     # D*H*W = 16*48*48 elements per (n, g), respectively over a row of 36864
     k = {"tmm": 256, "matmul": 1000, "convolution": 36, "group_convolution": 36, "2fcrelu": chain(2000, 128), "mlp1": 2000, "mlp3": chain(128, 64, 32), "lut": 50,
          "c3": 1000, "2lut": 50, "group_normalization": 1,
-         "moments2": 36864, "group_normalization_single_kernel": 16 * 48 * 48, "kronecker3": chain(16, 16, 16),
+         "moments2": 36864, "sum": 36864, "mean": 36864, "sum_squares": 36864, "var": 36864, "sum_and_squares": 36864,
+         "kronecker3_1": 16, "kronecker3_2": 16, "kronecker3_3": 16,
+         "group_normalization_single_kernel": 16 * 48 * 48, "kronecker3": chain(16, 16, 16),
          "wavenet1": chain(64, 32, 32)}[name]
     for o, r in zip(outs, ref):
         got = o.cpu().numpy()
