@@ -446,9 +446,10 @@ void emitKernel(KernelCtx& kc, const DeviceLimits& limits, Emitter& em) {
       const StagePlan& prod = k.stages[i];
       const std::string& t = prod.tensor;
       if (!prod.threadReduction || prod.atomic || prod.mfma || prod.accCount != 1) continue;
-      bool sole = true;
-      for (size_t j = 0; j < k.stages.size(); ++j) sole &= j == i || k.stages[j].tensor != t;
-      if (!sole || tensorsRead(prod).count(t)) continue;
+      // the first stage that writes the tensor; later ones may update the value in place (below)
+      bool first = true;
+      for (size_t j = 0; j < i; ++j) first &= k.stages[j].tensor != t;
+      if (!first || tensorsRead(prod).count(t)) continue;
       // the producer's side: one point per thread, rows along threadIdx.y/z only
       std::vector<const LoopVar*> pvars;
       std::vector<int> ppos;
@@ -469,32 +470,51 @@ void emitKernel(KernelCtx& kc, const DeviceLimits& limits, Emitter& em) {
       }
       // a row of threads that works on no element of the tensor reduces nothing but identities
       for (int a = 1; a < 3 && ok; ++a) ok = k.block[a] == 1 || axisUsed[a];
+      // A later stage addresses the element this thread holds: the same variable of the same
+      // tiling in every subscript.  Where the producer's variable is on no thread axis, every
+      // thread holds the value of the block's one point along it, and the reader's variable may
+      // sit on a thread axis: its threads beyond the point compute on the clamped index.
+      auto sameElement = [&](const StagePlan& cons, const std::vector<ExprRef>& subs) {
+        bool same = subs.size() == pvars.size();
+        for (size_t d = 0; same && d < pvars.size(); ++d) {
+          int pos = -1;
+          int64_t c = 0;
+          const LoopVar* v = plainVar(cons, subs[d], &pos, &c);
+          const LoopVar* w = pvars[d];
+          same = v && c == pconst[d] && !v->reduction && !v->vectorLane && v->perThread == 1 && v->min == w->min &&
+              v->extent == w->extent && v->tile == w->tile && v->numTiles == w->numTiles &&
+              v->blockAxis == w->blockAxis && v->gridExtent == w->gridExtent &&
+              (v->threadAxis == w->threadAxis || (w->threadAxis < 0 && v->tile == 1)) &&
+              (v->numTiles == 1 || (pos == ppos[d] && pos < k.sharedDepth));
+        }
+        return same;
+      };
       bool anyReader = false;
+      int lastWriter = static_cast<int>(i);
       for (size_t j = i + 1; j < gens.size() && ok; ++j) {
         const StagePlan& cons = k.stages[j];
-        if (!tensorsRead(cons).count(t)) continue;
+        const bool writes = cons.tensor == t;
+        if (!writes && !tensorsRead(cons).count(t)) continue;
         anyReader = true;
         ok = cons.views.at(t).extents == prod.views.at(t).extents;
+        if (writes) {
+          // an update in place of the value the threads hold: pointwise, one element per thread
+          bool pointwise = !cons.atomic && !cons.mfma && !cons.threadReduction && cons.accCount == 1;
+          for (const auto& stmt : cons.stmts) pointwise &= stmt.redVars.empty();
+          ok = ok && pointwise && sameElement(cons, cons.lhsSubs);
+          lastWriter = static_cast<int>(j);
+        }
         for (const auto& stmt : cons.stmts) {
           visit(stmt.rhs, [&](const ExprRef& e) {
             if (!ok || e->kind != Expr::Load || e->name != t) return;
-            ok = e->args.size() == pvars.size();
-            for (size_t d = 0; ok && d < pvars.size(); ++d) {
-              int pos = -1;
-              int64_t c = 0;
-              const LoopVar* v = plainVar(cons, e->args[d], &pos, &c);
-              const LoopVar* w = pvars[d];
-              ok = v && c == pconst[d] && !v->reduction && !v->vectorLane && v->perThread == 1 && v->min == w->min &&
-                  v->extent == w->extent && v->tile == w->tile && v->numTiles == w->numTiles &&
-                  v->blockAxis == w->blockAxis && v->gridExtent == w->gridExtent && v->threadAxis == w->threadAxis &&
-                  (v->numTiles == 1 || (pos == ppos[d] && pos < k.sharedDepth));
-            }
+            ok = sameElement(cons, e->args);
           });
         }
       }
       if (!anyReader || !ok) continue;
       KernelCtx::RegisterForward f;
       f.producer = static_cast<int>(i);
+      f.lastWriter = lastWriter;
       f.name = "rfwd" + std::to_string(i) + "_" + t;
       forwardDecls.push_back(prod.views.at(t).type.cName() + " " + f.name + ";");
       kc.registerForwards[t] = f;
@@ -741,8 +761,11 @@ void emitKernel(KernelCtx& kc, const DeviceLimits& limits, Emitter& em) {
         const StagePlan& a = k.stages[i];
         const StagePlan& b = k.stages[j];
         // (a result the later stage takes from a register is no dependence through memory)
-        bool conflict = a.tensor == b.tensor || tensorsRead(a).count(b.tensor) ||
-            (tensorsRead(b).count(a.tensor) && !kc.registerForwards.count(a.tensor));
+        // (of its writers the last one alone stores it)
+        auto inRegister = [&](const std::string& t) { return kc.registerForwards.count(t) > 0; };
+        bool conflict = (a.tensor == b.tensor && !inRegister(a.tensor)) ||
+            (tensorsRead(a).count(b.tensor) && !inRegister(b.tensor)) ||
+            (tensorsRead(b).count(a.tensor) && !inRegister(a.tensor));
         if (conflict && !gens[j].readsPrivatelyFrom(a)) need[i][j - i] = level;
       }
     }

@@ -54,10 +54,13 @@ struct KernelCtx {
   std::map<std::string, Forward> forwards;
   // The result of a block-wide reduction that later stages of the kernel read at the element the
   // block has just produced: after the reduction every thread holds the value, so the readers take
-  // it from a register instead of from memory (thread 0 still stores it for later kernels).
+  // it from a register instead of from memory (thread 0 still stores it for later kernels).  Later
+  // stages that update the same element in place (mean(n) = mean(n) / K after the sum) work on the
+  // register too, and only the last of the writers stores.
   struct RegisterForward {
     std::string name;
     int producer = 0;
+    int lastWriter = 0;
   };
   std::map<std::string, RegisterForward> registerForwards;
   int64_t NT() const { return k.block[0] * k.block[1] * k.block[2]; }
@@ -349,7 +352,8 @@ class StageCodegen {
         : "p" + st_.tensor + "[" + index + "] = " + value + ";";
     {
       auto rf = kc_.registerForwards.find(st_.tensor);
-      if (rf != kc_.registerForwards.end() && rf->second.producer == stageIdx_) {
+      if (rf != kc_.registerForwards.end() && rf->second.producer <= stageIdx_) {
+        if (stageIdx_ < rf->second.lastWriter) return rf->second.name + " = " + value + ";";
         return rf->second.name + " = " + value + "; if (" + cond + ") " + store;
       }
     }
@@ -1166,7 +1170,12 @@ class StageCodegen {
 
   void preloadAcc() {
     int n = openUnrolled();
-    em_.line("acc_[a_] = p" + st_.tensor + "[" + flatIndex(st_.tensor, st_.lhsSubs, "") + "];");
+    auto rf = kc_.registerForwards.find(st_.tensor);
+    if (rf != kc_.registerForwards.end() && rf->second.producer < stageIdx_) {
+      em_.line("acc_[a_] = " + rf->second.name + ";");
+    } else {
+      em_.line("acc_[a_] = p" + st_.tensor + "[" + flatIndex(st_.tensor, st_.lhsSubs, "") + "];");
+    }
     closeN(n);
     accValid_ = true;
   }

@@ -318,9 +318,8 @@ TUNED_AT_REFERENCE_SIZES = {
     "lut": "naive;outerScheduleFusionStrategy=Min;tile=4,32,32;unroll=64;usePrivateMemory=1;unrollCopyShared=1;"
            "collapseContiguous=0",
     "2lut": "naive;tile=2,32,32;unroll=256;mapToThreads=64,4,1;mapToBlocks=100000,256;vectorWidth=4;useMfma=1",
-    "moments2": "naive;outerScheduleFusionStrategy=Max;fixParametersBeforeScheduling=1;tile=1;unroll=128;"
-                "tileImperfectlyNested=1;matchLibraryCalls=1;mapToThreads=256;mapToBlocks=1152;usePrivateMemory=1;"
-                "unrollCopyShared=1;vectorWidth=2;collapseContiguous=0;useMfma=1",
+    "moments2": "naive;outerScheduleFusionStrategy=Max;tile=1,0;unroll=32;matchLibraryCalls=1;mapToThreads=512;mapToBlocks=1024,1;"
+                "usePrivateMemory=1;useReadOnlyCache=1;vectorWidth=4",
     # 576 threads x float4 = one 48x48 plane per pass: the normalising stage then finds every
     # element in the register cache the two reductions filled (one read of the input); two groups
     # per block

@@ -427,6 +427,36 @@ def test_block_wide_reduction_result_is_forwarded_in_a_register():
     assert launches[0][1][1] == 4 and "rfwd0_s" not in src
 
 
+def test_in_place_updates_of_a_forwarded_reduction_stay_in_the_register():
+    """`mean(n) = mean(n) / K` after the sum (tc/benchmarks/moments.h:52-59) works on the register
+    every thread holds; the last writer alone stores, and no barrier or reload separates the four
+    statements."""
+    moments2 = """def moments2(float(N, K) I) -> (mean, var) {
+        mean(n) +=! I(n, r_k)
+        var(n) +=! I(n, r_k) * I(n, r_k)
+        mean(n) = mean(n) / (K)
+        var(n) = var(n) / (K) - mean(n) * mean(n) }"""
+    opts = "naive;tile=1,0;mapToThreads=128;mapToBlocks=64;matchLibraryCalls=1;outerScheduleFusionStrategy=Max"
+    src, launches = mapped(moments2, "moments2", [(37, 1000)], opts + ";usePrivateMemory=1")
+    assert launches == [((37, 1, 1), (128, 1, 1))]
+    kernel = src[src.index('extern "C"'):]
+    assert "__syncthreads();" not in kernel
+    stage0, stage1, stage2, stage3 = kernel.split("// stage ")[1:]
+    assert "rfwd0_mean = acc_[a_];" in stage0 and "pmean[" not in stage0
+    assert "rfwd1_var = acc_[a_];" in stage1 and "pvar[" not in stage1
+    assert "acc_[a_] = rfwd0_mean;" in stage2 and "rfwd0_mean = acc_[a_]; if (ok_) pmean[i_n] = acc_[a_];" in stage2
+    assert "acc_[a_] = rfwd1_var;" in stage3 and "(rfwd0_mean * rfwd0_mean)" in stage3
+    assert "if (ok_) pvar[i_n] = acc_[a_];" in stage3 and "pmean[" not in stage3
+    plain, _ = mapped(moments2, "moments2", [(37, 1000)], opts + ";usePrivateMemory=0")
+    assert "rfwd" not in plain and "acc_[a_] = pmean[" in plain and "__syncthreads();" in plain[plain.index('extern "C"'):]
+    # an update that is itself a reduction, or that runs over more points than the block holds,
+    # is not an update of the held element
+    again = """def again(float(N, K) I) -> (s) {
+        s(n) +=! I(n, r_k)
+        s(n) += I(n, r_k) * I(n, r_k) }"""
+    assert "rfwd" not in mapped(again, "again", [(37, 1000)], opts + ";usePrivateMemory=1")[0]
+
+
 def test_reduction_blocks_divides_a_sum_among_blocks():
     """reductionBlocks: `O +=! f` becomes a zeroing kernel and a kernel whose outermost parallel
     variable numbers slices of the outermost reduction index; partial sums meet in atomics."""
