@@ -449,7 +449,17 @@ void emitKernel(KernelCtx& kc, const DeviceLimits& limits, Emitter& em) {
       // the first stage that writes the tensor; later ones may update the value in place (below)
       bool first = true;
       for (size_t j = 0; j < i; ++j) first &= k.stages[j].tensor != t;
-      if (!first || tensorsRead(prod).count(t)) continue;
+      // (an epilogue of the producer may re-read the element it is finishing: its running value)
+      bool readsOtherElements = false;
+      for (const auto& stmt : prod.stmts) {
+        visit(stmt.rhs, [&](const ExprRef& e) {
+          if (e->kind != Expr::Load || e->name != t) return;
+          bool same = e->args.size() == prod.lhsSubs.size();
+          for (size_t d = 0; same && d < e->args.size(); ++d) same = sameExpr(e->args[d], prod.lhsSubs[d]);
+          readsOtherElements |= !same;
+        });
+      }
+      if (!first || readsOtherElements) continue;
       // the producer's side: one point per thread, rows along threadIdx.y/z only
       std::vector<const LoopVar*> pvars;
       std::vector<int> ppos;

@@ -176,6 +176,54 @@ def test_reduction_results_forwarded_in_registers(shape, options):
     np.testing.assert_allclose(got[2].sum(1), 1.0, rtol=1e-5 * np.sqrt(shape[1]))
 
 
+LOG_SUM_EXP = """def lse(float(N, K) I) -> (m, e, O) {
+    m(n) max=! I(n, r_k)
+    m(n) = m(n) * 0.5
+    e(n) +=! exp(I(n, r_k) - m(n))
+    e(n) = log(e(n)) + m(n)
+    O(n, k) = I(n, k) - e(n) }"""
+
+GROUP_MOMENTS = """def gm(float(N, G, K) I) -> (s, q) {
+    s(n, g) +=! I(n, g, r_k)
+    q(n, g) +=! I(n, g, r_k) * I(n, g, r_k)
+    s(n, g) = s(n, g) / K
+    q(n, g) = q(n, g) / K - s(n, g) * s(n, g) }"""
+
+
+@pytest.mark.parametrize("src,entry,shape,options,registers", [
+    # updates in the epilogue of the reductions, then a reader over the whole row
+    (LOG_SUM_EXP, "lse", (13, 700),
+     "naive;tile=1;mapToThreads=128;mapToBlocks=64;matchLibraryCalls=1;usePrivateMemory=1;outerScheduleFusionStrategy=Max", ("rfwd0_m", "rfwd1_e")),
+    (LOG_SUM_EXP, "lse", (13, 700),
+     "naive;tile=2,0;mapToThreads=64,2;mapToBlocks=3;matchLibraryCalls=1;usePrivateMemory=1;vectorWidth=4;outerScheduleFusionStrategy=Max", ("rfwd0_m", "rfwd1_e")),
+    # updates as stages of their own behind both reductions (tc/benchmarks/moments.h:52-59 over two indices)
+    (GROUP_MOMENTS, "gm", (6, 5, 333),
+     "naive;tile=1,1,0;mapToThreads=100;mapToBlocks=256,256;matchLibraryCalls=1;usePrivateMemory=1;outerScheduleFusionStrategy=Max", ("rfwd0_s", "rfwd1_q")),
+    (GROUP_MOMENTS, "gm", (3, 2, 4096),
+     "naive;tile=1,1,0;mapToThreads=256;mapToBlocks=2,2;matchLibraryCalls=1;usePrivateMemory=1;vectorWidth=4;unroll=16;useReadOnlyCache=1;outerScheduleFusionStrategy=Max",
+     ("rfwd0_s", "rfwd1_q")),
+])
+def test_in_place_updates_of_forwarded_reductions(src, entry, shape, options, registers):
+    """A reduction's result that later statements update in place stays in the register of the
+    threads that hold it; the stored values are those of the last update."""
+    X = np.random.Generator(np.random.Philox(49)).standard_normal(shape).astype(np.float32) * 2
+    got, ex = run(src, entry, [X], options)
+    assert all(r in ex.compiled_source for r in registers) and ex.num_kernels == 1
+    ref = tc_oracle.run(src, entry, [X])
+    k = shape[-1]
+    for g, r in zip(got, ref):
+        np.testing.assert_allclose(g, r, rtol=1e-5 * np.sqrt(k), atol=1e-5 * np.sqrt(k))
+    if entry == "gm":
+        np.testing.assert_allclose(got[0], X.mean(2), rtol=1e-5, atol=1e-5)
+        np.testing.assert_allclose(got[1], X.var(2), rtol=1e-4, atol=1e-5)
+    else:
+        half_max = X.max(1) * 0.5
+        assert np.array_equal(got[0], half_max.astype(np.float32))
+        lse = np.log(np.exp(X.astype(np.float64)).sum(1))
+        np.testing.assert_allclose(got[1], lse, rtol=1e-5)
+        np.testing.assert_allclose(got[2], X - got[1][:, None], rtol=1e-6, atol=1e-6)   # the reader saw the stored value
+
+
 def test_reader_of_other_blocks_rows_stays_in_a_kernel_of_its_own():
     """Rows another block produces are read through memory, after the producing kernel: such a
     reader is not fused with its producer, and nothing is forwarded."""
