@@ -258,6 +258,12 @@ CASES = {
     "kronecker3": (KRONECKER3, "Kronecker3Full", [(6, 5), (7, 4), (8, 3), (10, 5, 4, 3)], 5),
     "wavenet1": (WAVENET1, "wavenet1",
                  [(1, 8, 100), (8, 8, 2), (8,), (8, 8, 2), (8,), (8, 8), (8,), (16, 8), (16,), (2,)], 16),
+    # the sizes of the program's tuned runs (wavenet.cc:139-168): eight times the skip channels,
+    # dilation 1 and 32; here two batches, more skip than residual channels, dilations 1 and 5
+    "wavenet1_skip256": (WAVENET1, "wavenet1",
+                         [(2, 4, 50), (6, 4, 2), (6,), (6, 4, 2), (6,), (4, 6), (4,), (24, 6), (24,), (1,)], 8),
+    "wavenet1_skip256_dilation32": (WAVENET1, "wavenet1",
+                                    [(2, 4, 50), (6, 4, 2), (6,), (6, 4, 2), (6,), (4, 6), (4,), (24, 6), (24,), (5,)], 8),
 }
 
 
@@ -290,6 +296,8 @@ REFERENCE_SIZES = {
     "group_normalization_single_kernel": [(32, 32, 16, 48, 48), (32, 16), (32, 16)],
     "kronecker3": [(32, 16), (32, 16), (32, 16), (256, 16, 16, 16)],
     "wavenet1": [(1, 32, 4000), (32, 32, 2), (32,), (32, 32, 2), (32,), (32, 32), (32,), (32, 32), (32,), (1,)],
+    "wavenet1_skip256": [(1, 32, 4000), (32, 32, 2), (32,), (32, 32, 2), (32,), (32, 32), (32,), (256, 32), (256,), (1,)],
+    "wavenet1_skip256_dilation32": [(1, 32, 4000), (32, 32, 2), (32,), (32, 32, 2), (32,), (32, 32), (32,), (256, 32), (256,), (32,)],
 }
 TUNED_AT_REFERENCE_SIZES = {
     # one (n, g) image per block and half its rows per block in z, the 4x56x56 input window in LDS,
@@ -351,6 +359,12 @@ TUNED_AT_REFERENCE_SIZES = {
     "wavenet1": "naive;intraTileScheduleFusionStrategy=Max;fixParametersBeforeScheduling=1;tile=2,2000,16,1;mapToThreads=16,64;"
                 "mapToBlocks=2000,256;useSharedMemory=1;usePrivateMemory=1;privateDepth=8;sharedDepth=3;vectorWidth=4;"
                 "collapseContiguous=0;prefetchShared=1",
+    "wavenet1_skip256": "naive;intraTileScheduleFusionStrategy=Max;fixParametersBeforeScheduling=1;tile=2,2000,16;unroll=128;"
+                        "mapToThreads=16,64;mapToBlocks=2000,256;useSharedMemory=1;usePrivateMemory=1;useReadOnlyCache=1;"
+                        "privateDepth=8;sharedDepth=3;collapseContiguous=0;prefetchShared=1",
+    "wavenet1_skip256_dilation32": "naive;intraTileScheduleFusionStrategy=Max;fixParametersBeforeScheduling=1;tile=2,2000,16;unroll=1;"
+                                   "mapToThreads=16,64;mapToBlocks=4000,256;useSharedMemory=1;usePrivateMemory=1;useReadOnlyCache=1;"
+                                   "privateDepth=8;sharedDepth=3;vectorWidth=4;collapseContiguous=0;useMfma=1;prefetchShared=1",
 }
 
 

@@ -27,7 +27,8 @@ def chain(*lengths):
 # they normalise per: batch norm of a 4x6x7x5 input over N*H*W = 4*7*5 per channel, the one-kernel
 # group norm of a 3x4x5x6x7 input over D*H*W = 5*6*7 per (n, g).
 CHAINED = {"2fcrelu": chain(48, 36), "mlp3": chain(24, 18, 10), "kronecker3": chain(5, 4, 3), "batchnorm": 4 * 7 * 5,
-           "wavenet1": chain(16, 8, 8), "group_normalization_single_kernel": 5 * 6 * 7}
+           "wavenet1": chain(16, 8, 8), "wavenet1_skip256": chain(8, 6, 6), "wavenet1_skip256_dilation32": chain(8, 6, 6),
+           "group_normalization_single_kernel": 5 * 6 * 7}
 
 
 @pytest.mark.parametrize("options", sorted(OPTION_SETS))
@@ -73,7 +74,7 @@ def test_parity_at_the_reference_sizes_with_the_tuned_options(name):
          "moments2": 36864, "sum": 36864, "mean": 36864, "sum_squares": 36864, "var": 36864, "sum_and_squares": 36864,
          "kronecker3_1": 16, "kronecker3_2": 16, "kronecker3_3": 16,
          "group_normalization_single_kernel": 16 * 48 * 48, "kronecker3": chain(16, 16, 16),
-         "wavenet1": chain(64, 32, 32)}[name]
+         "wavenet1": chain(64, 32, 32), "wavenet1_skip256": chain(64, 32, 32), "wavenet1_skip256_dilation32": chain(64, 32, 32)}[name]
     for o, r in zip(outs, ref):
         got = o.cpu().numpy()
         assert got.shape == r.shape
