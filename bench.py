@@ -363,6 +363,7 @@ def measure_suite(steps, warmup, only=()):
     out = {}
     cases = [(name, name, options, None) for name, options in B.TUNED_AT_REFERENCE_SIZES.items()]
     cases += [(name, case, options, k) for name, (case, _, options, k) in B.LARGE_CONTRACTIONS.items()]
+    cases += [(name, case, options, 0) for name, (case, _, options, _k) in B.OTHER_REFERENCE_SIZES.items()]
     unknown = set(only) - {c[0] for c in cases}
     if unknown:
         sys.exit(f"--suite-cases: unknown comprehension(s) {sorted(unknown)}")
@@ -370,7 +371,7 @@ def measure_suite(steps, warmup, only=()):
         if only and name not in only:
             continue
         src, entry, _, _ = B.CASES[case]
-        arrays = B.make_large_inputs(name) if k else B.make_inputs(name, reference_sizes=True)
+        arrays = B.make_inputs(name, reference_sizes=True) if name in B.REFERENCE_SIZES else B.make_large_inputs(name)
         ins = [torch.from_numpy(a).cuda() for a in arrays]
         ex = tc.compile(src, entry, ins, options)
         outs = tc.prepare_outputs(src, entry, ins)

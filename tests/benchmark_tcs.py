@@ -381,30 +381,57 @@ LARGE_CONTRACTIONS = {
     "matmul_2048": ("matmul", [(2048, 2048), (2048, 2048)],
                     "naive;tile=128,128,16;mapToThreads=64,8;mapToBlocks=256,256;useMfma=1;useSharedMemory=1;"
                     "prefetchShared=1", 2048),
+    # the largest size of the transposed product's tuned runs (tc/benchmarks/tmm.cc:138-140)
+    "tmm_128_16384_4096": ("tmm", [(128, 4096), (16384, 4096)],
+                           "naive;tile=64,128,32;mapToThreads=64,8;mapToBlocks=256,256;useMfma=1;useSharedMemory=1;"
+                           "prefetchShared=1", 4096),
 }
+
+# The other sizes the reference's benchmark programs run their tuned options at
+# (group_convolution.cc:104-160, moments.cc:162-303, group_normalization.cc:120-180), same layout.
+OTHER_REFERENCE_SIZES = {
+    "group_convolution_8_8_28": ("group_convolution", [(32, 32, 8, 28, 28), (32, 8, 8, 3, 3), (32, 8)],
+                                 "naive;tile=1,1,8,26,26;mapToThreads=64,8;mapToBlocks=32,32;useSharedMemory=1;useReadOnlyCache=1;"
+                                 "useMfma=1", 72),
+    "group_convolution_32_32_7": ("group_convolution", [(32, 32, 32, 7, 7), (32, 32, 32, 3, 3), (32, 32)],
+                                  "naive;tile=4,1,0,0,8;mapToThreads=256,4;mapToBlocks=32,256;useSharedMemory=1;useReadOnlyCache=1;"
+                                  "useMfma=1", 288),
+    "moments2_128_2304": ("moments2", [(128, 2304)],
+                          "naive;outerScheduleFusionStrategy=Max;tile=1,4096;unroll=32;matchLibraryCalls=1;mapToThreads=256;"
+                          "mapToBlocks=2304,256;usePrivateMemory=1;sharedDepth=6;vectorWidth=2", 2304),
+    "group_normalization_4_512_12": ("group_normalization",
+                                     [(4, 32, 16, 12, 12), (32, 16), (32, 16), (4, 32), ("positive", (4, 32))],
+                                     "naive;tile=1,1,0,0,0;unroll=16;mapToThreads=12,16;mapToBlocks=256,256;useSharedMemory=1;"
+                                     "useReadOnlyCache=1;collapseContiguous=0", 1),
+    "group_normalization_single_kernel_4_512_12": ("group_normalization_single_kernel", [(4, 32, 16, 12, 12), (32, 16), (32, 16)],
+                                                   "naive;outerScheduleFusionStrategy=Max;tile=1,1,0;unroll=64;matchLibraryCalls=1;"
+                                                   "mapToThreads=128,2,1;mapToBlocks=256,256;usePrivateMemory=1;vectorWidth=4",
+                                                   16 * 12 * 12),
+}
+
+
+def _draw(rng, spec):
+    import numpy as np
+    if isinstance(spec[0], str):
+        kind = spec[0]
+        if kind == "int":
+            return rng.integers(spec[2], spec[3], size=spec[1]).astype(np.int32)
+        if kind == "scalar":
+            return np.array(spec[1], dtype=np.float32)
+        if kind == "positive":
+            return (rng.random(spec[1], dtype=np.float32) + 0.5).astype(np.float32)
+        raise ValueError(kind)
+    return rng.standard_normal(spec, dtype=np.float32)
 
 
 def make_large_inputs(name, seed=2024):
     import numpy as np
     rng = np.random.Generator(np.random.Philox(seed))
-    return [rng.standard_normal(shape, dtype=np.float32) for shape in LARGE_CONTRACTIONS[name][1]]
+    table = LARGE_CONTRACTIONS if name in LARGE_CONTRACTIONS else OTHER_REFERENCE_SIZES
+    return [_draw(rng, spec) for spec in table[name][1]]
 
 
 def make_inputs(name, seed=2024, reference_sizes=False):
     import numpy as np
     rng = np.random.Generator(np.random.Philox(seed))
-    out = []
-    for spec in (REFERENCE_SIZES if reference_sizes else {name: CASES[name][2]})[name]:
-        if isinstance(spec[0], str):
-            kind = spec[0]
-            if kind == "int":
-                out.append(rng.integers(spec[2], spec[3], size=spec[1]).astype(np.int32))
-            elif kind == "scalar":
-                out.append(np.array(spec[1], dtype=np.float32))
-            elif kind == "positive":
-                out.append((rng.random(spec[1], dtype=np.float32) + 0.5).astype(np.float32))
-            else:
-                raise ValueError(kind)
-        else:
-            out.append(rng.standard_normal(spec, dtype=np.float32))
-    return out
+    return [_draw(rng, spec) for spec in (REFERENCE_SIZES if reference_sizes else {name: CASES[name][2]})[name]]

@@ -82,9 +82,9 @@ def test_parity_at_the_reference_sizes_with_the_tuned_options(name):
         assert np.abs(got - r).max() <= 1e-5 * np.sqrt(k) * scale, (name, ex.launch_bounds())
 
 
-@pytest.mark.parametrize("name", sorted(B.LARGE_CONTRACTIONS))
-def test_parity_of_the_large_contractions(name):
-    case, _, options, k = B.LARGE_CONTRACTIONS[name]
+@pytest.mark.parametrize("name", sorted(B.LARGE_CONTRACTIONS) + sorted(B.OTHER_REFERENCE_SIZES))
+def test_parity_of_the_large_contractions_and_the_other_reference_sizes(name):
+    case, _, options, k = (B.LARGE_CONTRACTIONS if name in B.LARGE_CONTRACTIONS else B.OTHER_REFERENCE_SIZES)[name]
     src, entry, _, _ = B.CASES[case]
     print(f"case {name}", flush=True)
     ins_np = B.make_large_inputs(name)
@@ -92,13 +92,15 @@ def test_parity_of_the_large_contractions(name):
     ins = [torch.from_numpy(a).cuda() for a in ins_np]
     ex = tc.compile(src, entry, ins, options)
     outs = tc.prepare_outputs(src, entry, ins)
-    outs[0].fill_(float("nan"))
+    for o in outs:
+        o.fill_(float("nan"))
     tc.run(ex, ins, outs)
     torch.cuda.synchronize()
-    got = outs[0].cpu().numpy()
-    assert got.shape == ref[0].shape
-    scale = max(float(np.abs(ref[0]).max()), 1e-30)
-    assert np.abs(got - ref[0]).max() <= 1e-5 * np.sqrt(k) * scale, (name, ex.launch_bounds())
+    for o, r in zip(outs, ref):
+        got = o.cpu().numpy()
+        assert got.shape == r.shape
+        scale = max(float(np.abs(r).max()), 1e-30)
+        assert np.abs(got - r).max() <= 1e-5 * np.sqrt(k) * scale, (name, ex.launch_bounds())
 
 
 def test_autotuning_the_1024_matmul_from_the_naive_options_reaches_the_stored_options():
