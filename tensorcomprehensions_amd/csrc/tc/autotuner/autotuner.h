@@ -356,10 +356,11 @@ inline std::vector<HipMappingOptions> heuristicSeeds(
     // many output tiles: 64x64 per block (128x128 for outputs that fill the device with those),
     // the reduction in tiles of 32 (16) staged through LDS while earlier tiles multiply; four
     // wavefronts, or eight that own rectangles of output tiles
-    for (int variant = 0; variant < 3; ++variant) {
+    // (the fourth: 64x128 for outputs with one short side, whose 128x128 tiles are too few)
+    for (int variant = 0; variant < 4; ++variant) {
       HipMappingOptions o = base;
       const uint64_t side = variant == 2 ? 128 : 64;
-      o.generic.tile(std::vector<uint64_t>{side, side, variant == 2 ? 16u : 32u});
+      o.generic.tile(std::vector<uint64_t>{side, variant == 3 ? 128u : side, variant == 2 ? 16u : 32u});
       o.mapToThreads(64, variant == 0 ? 4 : 8).mapToBlocks(largest, largest).useSharedMemory(true).useReadOnlyCache(true);
       o.sharedDepth(7); // (a depth beyond the parallel dimensions: the copies stay inside the reduction tile loop)
       o.useMfmaValue = true;
