@@ -267,14 +267,15 @@ def test_autotune_from_the_naive_options_reaches_the_stored_options(name):
     ins = [torch.from_numpy(a).cuda() for a in ins_np]
     outs = tc.prepare_outputs(src, entry, ins)
 
-    def kernel_us(options):
+    def kernel_us(options, warm=200, launches=50, bursts=5):
         ex = tc.compile(src, entry, ins, options)
-        tc.profile_repeated(ex, ins, outs, 200)
-        return min(tc.profile_repeated(ex, ins, outs, 50) / 50 for _ in range(5))
+        tc.profile_repeated(ex, ins, outs, warm)
+        return min(tc.profile_repeated(ex, ins, outs, launches) / launches for _ in range(bursts))
 
-    best = tc.autotune(src, entry, ins, "naive", outputs=outs, generations=3, pop_size=30, threads=16, seed=1)
+    best = tc.autotune(src, entry, ins, "naive", outputs=outs, generations=4, pop_size=30, threads=16, seed=1)
     assert len(best) == 1
-    t_stored, t_tuned, t_naive = kernel_us(W.TUNED[name]), kernel_us(best[0]), kernel_us("naive")
+    # (a launch under the naive options takes up to 0.2 s: the group convolution on 32 x 8 threads)
+    t_stored, t_tuned, t_naive = kernel_us(W.TUNED[name]), kernel_us(best[0]), kernel_us("naive", 1, 2, 1)
     print(f"{name}: naive {t_naive:.1f} us, stored {t_stored:.1f} us, tuned from naive {t_tuned:.1f} us with {best[0]}", flush=True)
     assert t_tuned <= 1.15 * t_stored
     ex = tc.compile(src, entry, ins, best[0])
