@@ -321,8 +321,9 @@ TUNED_AT_REFERENCE_SIZES = {
     "mlp3": "naive;outerScheduleFusionStrategy=Max;intraTileScheduleFusionStrategy=Max;tile=16,256;unroll=16;mapToThreads=256;"
             "mapToBlocks=256,128;useSharedMemory=1;unrollCopyShared=1;sharedDepth=4;useMfma=1;prefetchShared=1",
     # two 16x16 tiles per block, the 250 reduction steps of a tile split over two wavefronts each
-    "c3": "naive;tile=16,32;unroll=256;mapToThreads=256;mapToBlocks=1024,1024;useSharedMemory=1;unrollCopyShared=1;"
-          "useReadOnlyCache=1;vectorWidth=2;useMfma=1",
+    # reduction tiles of 200 (five of them) staged through two LDS copies: 7.6 -> 6.4 us
+    "c3": "naive;tile=16,32,200;mapToThreads=64,8;mapToBlocks=256,256;useMfma=1;useSharedMemory=1;prefetchShared=1;"
+          "useReadOnlyCache=1",
     "lut": "naive;outerScheduleFusionStrategy=Min;tile=4,32,32;unroll=64;usePrivateMemory=1;unrollCopyShared=1;"
            "collapseContiguous=0",
     "2lut": "naive;tile=2,32,32;unroll=256;mapToThreads=64,4,1;mapToBlocks=100000,256;vectorWidth=4;useMfma=1",
