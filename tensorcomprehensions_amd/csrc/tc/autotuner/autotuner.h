@@ -12,7 +12,9 @@
 #include <chrono>
 #include <condition_variable>
 #include <cstdlib>
+#include <cmath>
 #include <csignal>
+#include <map>
 #include <deque>
 #include <iostream>
 #include <mutex>
@@ -105,6 +107,16 @@ inline std::vector<size_t> inputDivisorsAndPowers2(
   sizes.erase(std::unique(sizes.begin(), sizes.end()), sizes.end());
   std::vector<size_t> out;
   for (auto s : sizes) out = mergeVectors(std::move(out), powers2andCeilDivisors(s));
+  // Deviation: exact divisors that cut an extent into at most 16 parts of whole matrix-core steps
+  // (multiples of 4, up to 512).  A reduction tile has to divide its extent, and the ceiling
+  // divisors of an extent like 1000 (500, 250, 125, 63, ...) hold no tile between 125 and 500.
+  std::vector<size_t> exact;
+  for (auto s : sizes) {
+    for (size_t d = 4; d <= 512 && d <= s; d += 4) {
+      if (s % d == 0 && s / d <= 16) exact.push_back(d);
+    }
+  }
+  out = mergeVectors(std::move(out), exact);
   return mergeVectors(std::move(out), powers2andCeilDivisors(256));
 }
 
@@ -353,6 +365,40 @@ inline std::vector<HipMappingOptions> heuristicSeeds(
     seeds.push_back(o);
   }
   if (matrix) {
+    // The reduction extent of a product: an extent two input dimensions have, preferably one the
+    // output does not.  Reduction tiles must divide it: the divisor (a multiple of 4, the depth
+    // of a matrix-core step) nearest to the wanted tile on a logarithmic scale.
+    uint64_t reduction = 0;
+    {
+      std::map<uint64_t, int> seen;
+      for (auto t : inputs) {
+        for (int i = 0; i < t->ndim; ++i) ++seen[static_cast<uint64_t>(t->shape[i])];
+      }
+      bool outside = false;
+      for (const auto& e : seen) {
+        if (e.second < 2) continue;
+        const bool inOutput = static_cast<int64_t>(e.first) == firstOutputShape[0] || static_cast<int64_t>(e.first) == firstOutputShape[1];
+        if (!inOutput && !outside) {
+          outside = true;
+          reduction = 0;
+        }
+        if (inOutput == !outside) reduction = std::max(reduction, e.first);
+      }
+    }
+    auto reductionTile = [&](uint64_t wanted) -> uint64_t {
+      if (reduction == 0 || reduction % wanted == 0) return wanted;
+      uint64_t best = 0;
+      double bestDistance = 0;
+      for (uint64_t d = 4; d <= reduction && d <= 8 * wanted; d += 4) {
+        if (reduction % d != 0) continue;
+        const double distance = std::fabs(std::log(static_cast<double>(d) / static_cast<double>(wanted)));
+        if (best == 0 || distance < bestDistance) {
+          best = d;
+          bestDistance = distance;
+        }
+      }
+      return best == 0 ? wanted : best;
+    };
     // many output tiles: 64x64 per block (128x128 for outputs that fill the device with those),
     // the reduction in tiles of 32 (16) staged through LDS while earlier tiles multiply; four
     // wavefronts, or eight that own rectangles of output tiles
@@ -360,9 +406,20 @@ inline std::vector<HipMappingOptions> heuristicSeeds(
     for (int variant = 0; variant < 4; ++variant) {
       HipMappingOptions o = base;
       const uint64_t side = variant == 2 ? 128 : 64;
-      o.generic.tile(std::vector<uint64_t>{side, variant == 3 ? 128u : side, variant == 2 ? 16u : 32u});
+      o.generic.tile(std::vector<uint64_t>{side, variant == 3 ? 128u : side, reductionTile(variant == 2 ? 16 : 32)});
       o.mapToThreads(64, variant == 0 ? 4 : 8).mapToBlocks(largest, largest).useSharedMemory(true).useReadOnlyCache(true);
       o.sharedDepth(7); // (a depth beyond the parallel dimensions: the copies stay inside the reduction tile loop)
+      o.useMfmaValue = true;
+      o.prefetchSharedValue = true;
+      seeds.push_back(o);
+    }
+    // few output tiles, long reductions: two 16x16 tiles per block of 8 wavefronts, the reduction
+    // in tiles of about 256 through two LDS copies
+    {
+      HipMappingOptions o = base;
+      o.generic.tile(std::vector<uint64_t>{16, 32, reductionTile(256)});
+      o.mapToThreads(64, 8).mapToBlocks(largest, largest).useSharedMemory(true).useReadOnlyCache(true);
+      o.sharedDepth(7);
       o.useMfmaValue = true;
       o.prefetchSharedValue = true;
       seeds.push_back(o);
