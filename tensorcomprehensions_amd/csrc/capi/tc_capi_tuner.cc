@@ -131,11 +131,18 @@ extern "C" int tc_host_query(const char* what, const char* arg, char** out) {
       // would hold them next to the naive options
       std::vector<std::vector<int64_t>> shapes;
       size_t colon = a.find(':');
-      TC_CHECK(colon != std::string::npos) << "expected <smallest output rank>:<shapes>";
+      TC_CHECK(colon != std::string::npos) << "expected <smallest output rank>[,<innermost output extent>[,<first output shape>]]:<shapes>";
       std::string head = a.substr(0, colon);
       size_t comma = head.find(',');
       size_t smallestOutputRank = std::stoul(head.substr(0, comma));
       size_t innermostOutputExtent = comma == std::string::npos ? 0 : std::stoul(head.substr(comma + 1));
+      std::vector<int64_t> firstOutputShape;
+      size_t second = comma == std::string::npos ? std::string::npos : head.find(',', comma + 1);
+      if (second != std::string::npos) {
+        std::stringstream os(head.substr(second + 1));
+        std::string d;
+        while (std::getline(os, d, 'x')) firstOutputShape.push_back(std::stoll(d));
+      }
       std::stringstream ss(a.substr(colon + 1));
       std::string sh;
       while (std::getline(ss, sh, ';')) {
@@ -155,7 +162,7 @@ extern "C" int tc_host_query(const char* what, const char* arg, char** out) {
       std::vector<size_t> outputSizes;
       if (innermostOutputExtent > 0) outputSizes.push_back(innermostOutputExtent);
       TuningConfiguration space = tc::autotune::detail::setupTuningParameters(ptrs, {naive}, 256, outputSizes);
-      for (const auto& seed : tc::autotune::detail::heuristicSeeds(naive, ptrs, smallestOutputRank, innermostOutputExtent)) {
+      for (const auto& seed : tc::autotune::detail::heuristicSeeds(naive, ptrs, smallestOutputRank, innermostOutputExtent, false, firstOutputShape)) {
         try {
           TuningConfiguration c = space;
           c.fromHipMappingOptions(seed);

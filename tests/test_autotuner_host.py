@@ -44,6 +44,24 @@ def test_search_space_from_shapes():
     assert sorted(set(block) - set(grid)) == [468, 936] and set(grid) <= set(block)
 
 
+def test_reduction_tiles_of_the_matrix_members_divide_the_reduction_extent():
+    """128 x 1000 times the transpose of 1024 x 1000: the ceiling divisors of 1000 (500, 250, 125, 63, ...)
+    hold no usable reduction tile, so the exact divisors that leave at most 16 tiles of whole matrix-core
+    steps are candidates too, and the matrix members of generation 0 take the divisor nearest to
+    the depth they want (40 for 32, 200 for 256); a power of two stays as it is."""
+    fields = dict(kv.split("=") for kv in tc.host_query("search_space", "128x1000;1024x1000").split(";"))
+    tile = [int(x) for x in fields["tile"].split(",")]
+    assert {100, 200, 500, 250, 125, 63} <= set(tile) and 40 not in tile and 20 not in tile
+    seeds = tc.host_query("tuner_seeds", "2,1024,128x1024:128x1000;1024x1000").split("\n")
+    staged = [s for s in seeds if "prefetchShared=1" in s and "useMfma=1" in s]
+    assert any("tile=16,32,200;" in s and "mapToThreads=64,8" in s for s in staged)
+    assert not any("tile=64,64,32;" in s for s in staged)       # 32 does not divide 1000; 40 is no candidate value
+    seeds = tc.host_query("tuner_seeds", "2,1024,128x1024:128x1024;1024x1024").split("\n")
+    staged = [s for s in seeds if "prefetchShared=1" in s and "useMfma=1" in s]
+    for t in ("tile=64,64,32;", "tile=128,128,16;", "tile=64,128,32;", "tile=16,32,256;"):
+        assert any(t in s for s in staged), t
+
+
 def test_base_mapping_outside_the_space_is_refused():
     assert scaffold_query("base_outside_space").startswith("invalid_argument")
 
