@@ -18,6 +18,8 @@ namespace __tc {
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 // same vector read through a pointer that is only element-aligned
 typedef float floatx4u __attribute__((ext_vector_type(4), aligned(4)));
+typedef _Float16 halfx4 __attribute__((ext_vector_type(4)));
+typedef _Float16 halfx4u __attribute__((ext_vector_type(4), aligned(2)));
 }
 )HIP";
 

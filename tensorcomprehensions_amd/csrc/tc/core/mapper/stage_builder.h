@@ -330,6 +330,18 @@ struct StageBuilder {
   }
 };
 
+// An operand of a product the matrix cores take: a load of a float tensor, or a load of a float16
+// tensor converted to float (`float(A(m, r_k))`: every half is a float, and products of two
+// halves are exact in float).  Null for anything else.
+inline ExprRef contractionOperand(const ExprRef& e) {
+  const ScalarType f32{ScalarType::Float, 32}, f16{ScalarType::Float, 16};
+  if (e->kind == Expr::Load && e->type == f32) return e;
+  if (e->kind == Expr::Cast && e->type == f32 && e->args.size() == 1 && e->args[0]->kind == Expr::Load && e->args[0]->type == f16) {
+    return e->args[0];
+  }
+  return nullptr;
+}
+
 // Decides whether a stage is a dense fp32 contraction the matrix cores can take and assigns the
 // variable roles.  Needs: first statement `out +=(!) A(...) * B(...)` with affine subscripts,
 // float operands, at least one parallel variable private to each operand; later statements are
@@ -344,11 +356,12 @@ bool classifyContraction(StagePlan& st) {
   ScalarType f32{ScalarType::Float, 32};
   if (st.views.at(st.tensor).type != f32) return false;
   const ExprRef& e = s.rhs;
-  if (e->kind != Expr::Binary || e->name != "*" || e->args[0]->kind != Expr::Load || e->args[1]->kind != Expr::Load) {
+  if (e->kind != Expr::Binary || e->name != "*" || !contractionOperand(e->args[0]) || !contractionOperand(e->args[1])) {
     return false;
   }
-  for (const auto& l : e->args) {
-    if (l->type != f32 || l->name == st.tensor) return false;
+  for (const auto& operand : e->args) {
+    const ExprRef l = contractionOperand(operand);
+    if (l->name == st.tensor) return false;
     for (const auto& a : l->args) {
       if (!ir::toAffine(a).valid) return false;
     }

@@ -691,7 +691,7 @@ class StageCodegen {
       // lanes that walk a slower dimension: an odd row length spreads them over the banks
       if (nd >= 2 && c.p.extents.back() > 1 && c.p.extents.back() % 2 == 0 && lanesWalkOuterDim(ref)) pad[nd - 2] += 1;
       if (st_.mfma && nd >= 2 && kMfmaPad > 0) {
-        const bool isA = acc.first == s.rhs->args[st_.mfmaSwapOperands ? 1 : 0]->name;
+        const bool isA = acc.first == contractionOperand(s.rhs->args[st_.mfmaSwapOperands ? 1 : 0])->name;
         // The 16 lanes of a group walk the M- (or N-) side variable.  When that variable is not in
         // the last subscript, consecutive lanes are a whole pitch apart and a pitch that is a
         // multiple of 8 elements piles them onto few LDS banks: four elements of padding spread 16
@@ -900,14 +900,15 @@ class StageCodegen {
     }
     plan.elemType = view.type.cName();
     plan.regType = plan.elemType;
-    if (view.type.isFloat() && view.type.bits == 32 && !dims.empty()) {
+    // (groups of four elements: 16 bytes of floats, 8 bytes of halves)
+    if (view.type.isFloat() && (view.type.bits == 32 || view.type.bits == 16) && !dims.empty()) {
       const CopyDim& in = dims.back();
       bool ok = in.gStride == 1 && in.lStride == 1 && in.step == 1 && in.extent % 4 == 0 && in.tensorExtent % 4 == 0 &&
           in.loGcd % 4 == 0;
       for (size_t j = 0; j + 1 < dims.size(); ++j) ok &= dims[j].gStride % 4 == 0 && dims[j].lStride % 4 == 0;
       if (ok) {
         plan.vec = 4;
-        plan.regType = "__tc::floatx4";
+        plan.regType = view.type.bits == 32 ? "__tc::floatx4" : "__tc::halfx4";
       }
     }
     plan.iters = ceilDiv(plan.count / plan.vec, kc_.NT());
@@ -968,8 +969,8 @@ class StageCodegen {
       lidx += (j ? " + " : "") + l + (dims[j].lStride != 1 ? " * " + std::to_string(dims[j].lStride) : "");
     }
     if (dims.empty()) gidx = lidx = "0";
-    std::string cast = plan.vec > 1 ? "*(const __tc::floatx4u*)&" : "";
-    std::string lcast = plan.vec > 1 ? "*(__tc::floatx4*)&" : "";
+    std::string cast = plan.vec > 1 ? "*(const " + plan.regType + "u*)&" : "";
+    std::string lcast = plan.vec > 1 ? "*(" + plan.regType + "*)&" : "";
     std::string guard = live.empty() ? "" : "if (" + live + ") ";
     if (loads) {
       // inside the footprint but outside the tensor (halo of a partial tile): a clamped address,
@@ -1636,8 +1637,9 @@ class StageCodegen {
       for (const auto& n : g) exact &= !var(n).partial();
       return exact;
     };
-    const ExprRef& loadA = s.rhs->args[st_.mfmaSwapOperands ? 1 : 0]; // holds the M-side variables
-    const ExprRef& loadB = s.rhs->args[st_.mfmaSwapOperands ? 0 : 1]; // holds the N-side variables
+    // (a float16 operand is read as it is and converted where its value enters a float register)
+    const ExprRef loadA = contractionOperand(s.rhs->args[st_.mfmaSwapOperands ? 1 : 0]); // holds the M-side variables
+    const ExprRef loadB = contractionOperand(s.rhs->args[st_.mfmaSwapOperands ? 0 : 1]); // holds the N-side variables
     em_.line("// matrix cores: " + std::to_string(tiles) + " tiles of 16x16 per block, " + std::to_string(ksteps) +
              " steps of v_mfma_f32_16x16x4_f32 each, " + std::to_string(st_.waves) + " wavefront(s)");
     // (the register-resident operand is requested first: its latency overlaps the LDS staging)
@@ -1743,7 +1745,8 @@ class StageCodegen {
       decodeGroup(st_.mfmaM, "mposa_", true, MT % 16 == 0);
       // consecutive steps of a lane read consecutive elements when the operand's reduction
       // subscripts are jointly contiguous: four steps are then fetched with one 16-byte load
-      bool contiguous = !residentFromLds && !forwardOf(loadA->name) && aligned && quarter * 4 == KT && ksteps % 4 == 0;
+      bool contiguous = !residentFromLds && !forwardOf(loadA->name) && aligned && quarter * 4 == KT && ksteps % 4 == 0 &&
+          st_.views.at(loadA->name).type.bits == 32;
       {
         Affine fa = flatAffine(loadA->name, loadA->args);
         contiguous &= fa.valid;
@@ -2349,6 +2352,15 @@ class StageCodegen {
       const bool rotated = registerBlocked && pipelineK && twoCopies && bothStaged && stepsPerWave >= 2 && !forwardOf(loadA->name) &&
           !forwardOf(loadB->name);
       const int64_t halfSteps = stepsPerWave / 2;
+      // Both operands float16: four consecutive steps of a lane (four values of its quarter of the
+      // reduction tile per operand) are one v_mfma_f32_16x16x16_f16 - its lane group g supplies
+      // k = 4g .. 4g+3, the group's four values, so the instruction adds exactly what four
+      // 16x16x4 float steps add (products of halves are exact in float, the sums are float) at a
+      // sixteenth of their issue time.  The operand registers then hold halves.
+      const bool halfSteps16 = registerBlocked && st_.views.at(loadA->name).type.bits == 16 &&
+          st_.views.at(loadB->name).type.bits == 16 && stepsPerWave % 4 == 0 && (!rotated || halfSteps % 4 == 0);
+      const int64_t lead = halfSteps16 ? 4 : 1; // the multiplications kept between the stores and the barrier
+      const std::string operandType = halfSteps16 ? "_Float16" : "float";
       // operand values of steps [first, last) of the wavefront's rectangle into ra_ / rb_
       auto readOperands = [&](int64_t first, int64_t last) {
         em_.open("");
@@ -2386,6 +2398,22 @@ class StageCodegen {
       // the multiplications of steps [first, last), step by step over all tiles of the rectangle
       auto multiplySteps = [&](int64_t first, int64_t last) {
         if (first >= last) return;
+        if (halfSteps16) {
+          em_.line("#pragma unroll");
+          em_.open("for (int ks_ = " + std::to_string(first) + "; ks_ < " + std::to_string(last) + "; ks_ += 4)");
+          em_.line("#pragma unroll");
+          em_.open("for (int a_ = 0; a_ < " + std::to_string(RM) + "; ++a_)");
+          em_.line("const __tc::halfx4 av_ = {ra_[a_][ks_], ra_[a_][ks_ + 1], ra_[a_][ks_ + 2], ra_[a_][ks_ + 3]};");
+          em_.line("#pragma unroll");
+          em_.open("for (int b_ = 0; b_ < " + std::to_string(RN) + "; ++b_)");
+          em_.line("const __tc::halfx4 bv_ = {rb_[b_][ks_], rb_[b_][ks_ + 1], rb_[b_][ks_ + 2], rb_[b_][ks_ + 3]};");
+          em_.line("cacc_[a_ * " + std::to_string(RN) + " + b_] = __builtin_amdgcn_mfma_f32_16x16x16f16(av_, bv_, cacc_[a_ * " +
+                   std::to_string(RN) + " + b_], 0, 0, 0);");
+          em_.close();
+          em_.close();
+          em_.close();
+          return;
+        }
         em_.line("#pragma unroll");
         em_.open("for (int ks_ = " + std::to_string(first) + "; ks_ < " + std::to_string(last) + "; ++ks_)");
         em_.line("#pragma unroll");
@@ -2415,8 +2443,8 @@ class StageCodegen {
             if (p.insideReductionTiles) em_.line(copyRegisterDecl(p, regs(p, st)));
           }
         }
-        em_.line("float ra_[" + std::to_string(RM) + "][" + std::to_string(stepsPerWave) + "];");
-        em_.line("float rb_[" + std::to_string(RN) + "][" + std::to_string(stepsPerWave) + "];");
+        em_.line(operandType + " ra_[" + std::to_string(RM) + "][" + std::to_string(stepsPerWave) + "];");
+        em_.line(operandType + " rb_[" + std::to_string(RN) + "][" + std::to_string(stepsPerWave) + "];");
         auto loadTile = [&](const std::string& tile, int64_t st) {
           em_.open("");
           tileOverride[k0.name] = tile;
@@ -2469,7 +2497,7 @@ class StageCodegen {
           const int64_t nextStage = (d + 1) % stages;
           // second half of this tile's operand values, while the first half is multiplied
           readHalf(tk, cur, halfSteps, stepsPerWave);
-          multiplySteps(0, halfSteps - 1);
+          multiplySteps(0, halfSteps - lead);
           em_.line("__builtin_amdgcn_sched_barrier(0);");
           // (no branches in the loop body: with them the compiler waits for every load in flight
           // ahead of a store instead of the oldest ones.  Past the last tile the loads fetch the
@@ -2478,7 +2506,7 @@ class StageCodegen {
           loadTile("min(" + tk + " + " + std::to_string(1 + stages) + ", " + std::to_string(numK - 1) + ")", nextStage);
           em_.line("__builtin_amdgcn_sched_barrier(0);");
           // (one step of multiplications between the stores and the barrier that waits for them)
-          multiplySteps(halfSteps - 1, halfSteps);
+          multiplySteps(halfSteps - lead, halfSteps);
           // (and they stay there: the scheduler would lift the barrier, which is no memory
           // operation to the multiplications, above all but one of them)
           em_.line("__builtin_amdgcn_sched_barrier(0);");
@@ -2541,8 +2569,8 @@ class StageCodegen {
           stagePromotions(true);
         }
         if (registerBlocked) {
-          em_.line("float ra_[" + std::to_string(RM) + "][" + std::to_string(stepsPerWave) + "];");
-          em_.line("float rb_[" + std::to_string(RN) + "][" + std::to_string(stepsPerWave) + "];");
+          em_.line(operandType + " ra_[" + std::to_string(RM) + "][" + std::to_string(stepsPerWave) + "];");
+          em_.line(operandType + " rb_[" + std::to_string(RN) + "][" + std::to_string(stepsPerWave) + "];");
           // the operand values of the whole reduction tile first, then the multiplications
           readOperands(0, stepsPerWave);
           multiplySteps(0, stepsPerWave);

@@ -282,3 +282,75 @@ def test_split_reduction_accumulates_into_existing_output_and_runs_the_epilogue(
     assert np.array_equal(O, np.maximum(I @ W1.T + B1, 0))
     (ref,) = tc_oracle.run(FC, "fc", [I, W1, B1])
     assert np.array_equal(O, ref)
+
+
+HALF_MM = "def hmm(float16(M, K) A, float16(K, N) B) -> (C) { C(m, n) +=! float(A(m, r_k)) * float(B(r_k, n)) }"
+HALF_TMM = "def htmm(float16(M, K) A, float16(N, K) B) -> (C) { C(m, n) +=! float(A(m, r_k)) * float(B(n, r_k)) }"
+HALF_BMM = """def hbmm(float16(B, N, M) X, float16(B, M, K) Y, float(K) bias) -> (Z) {
+    Z(b, n, k) +=! float(X(b, n, r_m)) * float(Y(b, r_m, k))
+    Z(b, n, k) = Z(b, n, k) + bias(k) }"""
+
+HALF_CASES = [
+    # (text, entry, shapes of the half operands, options, half-precision matrix instruction expected)
+    # rotated pipeline, eight steps a tile: two v_mfma_f32_16x16x16_f16 per tile and pair of output tiles
+    (HALF_MM, "hmm", [(256, 256), (256, 256)],
+     "naive;tile=64,64,32;mapToThreads=64,8;mapToBlocks=256,256;useMfma=1;useSharedMemory=1;prefetchShared=1", True),
+    (HALF_TMM, "htmm", [(128, 512), (256, 512)],
+     "naive;tile=64,128,32;mapToThreads=64,8;mapToBlocks=256,256;useMfma=1;useSharedMemory=1;prefetchShared=1", True),
+    # reduction tiles of 64 and of 16 steps of four: the halves of a tile hold whole groups, or they do not
+    (HALF_MM, "hmm", [(128, 384), (384, 128)],
+     "naive;tile=64,64,64;mapToThreads=64,8;mapToBlocks=256,256;useMfma=1;useSharedMemory=1;prefetchShared=1", True),
+    (HALF_MM, "hmm", [(128, 192), (192, 160)],
+     "naive;tile=32,32,16;mapToThreads=64,4;mapToBlocks=256,256;useMfma=1;useSharedMemory=1;prefetchShared=1", False),
+    # partial tiles on every side, operands through LDS without reduction tiles, and straight from memory
+    (HALF_MM, "hmm", [(100, 90), (90, 70)],
+     "naive;tile=32,32;mapToThreads=64,4;mapToBlocks=256,256;useMfma=1;useSharedMemory=1", False),
+    (HALF_MM, "hmm", [(100, 90), (90, 70)], "naive;tile=16,32;mapToThreads=64,2;mapToBlocks=256,256;useMfma=1", False),
+    (HALF_TMM, "htmm", [(37, 1000), (45, 1000)],
+     "naive;tile=16,32;unroll=256;mapToThreads=256,2;mapToBlocks=256,256;useMfma=1;useSharedMemory=1;vectorWidth=2", False),
+    # a batch index and an epilogue in float
+    (HALF_BMM, "hbmm", [(7, 26, 72), (7, 72, 26)],
+     "naive;tile=1,26,26;mapToThreads=64,4;mapToBlocks=500;useMfma=1;useSharedMemory=1", False),
+]
+
+
+@pytest.mark.parametrize("src,entry,shapes,options,half_instruction", HALF_CASES)
+def test_float16_operands_on_the_matrix_cores(src, entry, shapes, options, half_instruction):
+    """`float(A) * float(B)` of float16 tensors is a contraction the matrix cores take: operands
+    are staged and read as halves, products and sums are float.  Small integers make every sum
+    exact, so the result equals numpy's in every bit; normal deviates stay within the tolerance of
+    a float sum against the oracle (which multiplies the converted values in float)."""
+    rng = np.random.Generator(np.random.Philox(71))
+    ins = [rng.integers(-4, 5, size=s).astype(np.float16) for s in shapes]
+    extra = [rng.integers(-3, 4, size=(shapes[1][-1],)).astype(np.float32)] if entry == "hbmm" else []
+    ex_source = {}
+
+    def go(arrays):
+        ins_t = [torch.from_numpy(a).cuda() for a in arrays]
+        ex = tc.compile(src, entry, ins_t, options)
+        ex_source["text"] = ex.compiled_source
+        outs = tc.prepare_outputs(src, entry, ins_t)
+        outs[0].fill_(float("nan"))
+        tc.run(ex, ins_t, outs)
+        torch.cuda.synchronize()
+        return outs[0].cpu().numpy()
+
+    got = go(ins + extra)
+    text = ex_source["text"]
+    assert ("__builtin_amdgcn_mfma_f32_16x16x16f16" in text) == half_instruction
+    assert half_instruction or "__builtin_amdgcn_mfma_f32_16x16x4f32" in text
+    a, b = ins[0].astype(np.float64), ins[1].astype(np.float64)
+    if entry == "hmm":
+        exact = a @ b
+    elif entry == "htmm":
+        exact = a @ b.T
+    else:
+        exact = np.einsum("bnm,bmk->bnk", a, b) + extra[0]
+    assert got.dtype == np.float32 and np.array_equal(got, exact.astype(np.float32))
+    (ref,) = tc_oracle.run(src, entry, ins + extra)
+    assert np.array_equal(ref, got)
+    normal = [rng.standard_normal(s).astype(np.float16) for s in shapes]
+    got = go(normal + extra)
+    (ref,) = tc_oracle.run(src, entry, normal + extra)
+    k = shapes[0][-1]
+    assert np.abs(got - ref).max() <= 1e-5 * np.sqrt(k) * max(float(np.abs(ref).max()), 1.0)
