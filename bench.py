@@ -30,6 +30,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 FP32_PEAK_TFLOPS = 157.3       # MI355X fp32 matrix/vector, published
+FP16_PEAK_TFLOPS = 2500.0      # MI355X dense fp16 matrix, published
 
 
 def flops(name, shapes):
@@ -324,6 +325,8 @@ def suite_library_routines():
     import torch.nn.functional as F
     return {
         "tmm": lambda a, b: a @ b.t(),
+        "half_tmm": lambda a, b: a @ b.t(),
+        "half_matmul": lambda a, b: a @ b,
         "matmul": lambda a, b: a @ b,
         "convolution": lambda i, w, b: F.conv2d(i, w, b),
         "group_convolution": lambda i, w, b: F.conv2d(
@@ -390,7 +393,10 @@ def measure_suite(steps, warmup, only=()):
             # a contraction's matrix-core roofline: 2 flops per multiply-add over the 157.3 TFLOP/s fp32 peak
             flops = 2.0 * outs[0].numel() * k
             entry_out["tflops"] = round(flops / us * 1e-6, 1)
-            entry_out["frac_of_fp32_matrix_peak"] = round(flops / us * 1e-6 / FP32_PEAK_TFLOPS, 3)
+            if name.startswith("half_"):
+                entry_out["frac_of_fp16_matrix_peak"] = round(flops / us * 1e-6 / FP16_PEAK_TFLOPS, 3)
+            else:
+                entry_out["frac_of_fp32_matrix_peak"] = round(flops / us * 1e-6 / FP32_PEAK_TFLOPS, 3)
         fn = routines.get(case)
         if fn is not None:
             for _ in range(warmup):

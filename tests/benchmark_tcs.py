@@ -20,6 +20,19 @@ def matmul(float(M, K) A, float(K, N) B) -> (O) {
 }
 """
 
+# The same two products over float16 operands converted to float (no counterpart in the reference,
+# whose front end has no half type): products of halves are exact in float, sums are float.
+HALF_TMM = """
+def half_tmm(float16(M, K) A, float16(N, K) B) -> (C) {
+    C(m, n) +=! float(A(m, r_k)) * float(B(n, r_k))
+}
+"""
+HALF_MATMUL = """
+def half_matmul(float16(M, K) A, float16(K, N) B) -> (O) {
+    O(m, n) +=! float(A(m, r_k)) * float(B(r_k, n))
+}
+"""
+
 CONVOLUTION = """
 def convolution(float(N, C, H, W) I, float(M, C, KH, KW) W1, float(M) B) -> (O) {
     O(n, m, h, w) +=! I(n, r_c, h + r_kh, w + r_kw) * W1(m, r_c, r_kh, r_kw)
@@ -231,6 +244,8 @@ def group_convolution(float(N, G, C, H, W) I, float(G, F, C, KH, KW) W1, float(G
 CASES = {
     "group_convolution": (GROUP_CONVOLUTION, "group_convolution", [(2, 3, 4, 10, 9), (3, 5, 4, 3, 3), (3, 5)], 36),
     "tmm": (TMM, "tmm", [(32, 256), (128, 256)], 256),
+    "half_tmm": (HALF_TMM, "half_tmm", [("half", (32, 256)), ("half", (128, 256))], 256),
+    "half_matmul": (HALF_MATMUL, "half_matmul", [("half", (40, 96)), ("half", (96, 72))], 96),
     "tmm_odd": (TMM, "tmm", [(37, 70), (51, 70)], 70),
     "matmul": (MATMUL, "matmul", [(72, 60), (60, 50)], 60),
     "convolution": (CONVOLUTION, "convolution", [(3, 4, 12, 11), (8, 4, 3, 3), (8,)], 36),
@@ -388,6 +403,16 @@ LARGE_CONTRACTIONS = {
                            "prefetchShared=1", 4096),
 }
 
+LARGE_CONTRACTIONS.update({
+    # float16 operands on v_mfma_f32_16x16x16_f16 (the roofline of these two is the 2.5 PFLOP/s half peak)
+    "half_tmm_4096": ("half_tmm", [("half", (4096, 4096)), ("half", (4096, 4096))],
+                      "naive;tile=128,256,32;mapToThreads=64,8;mapToBlocks=256,256;useMfma=1;useSharedMemory=1;"
+                      "prefetchShared=1", 4096),
+    "half_matmul_2048": ("half_matmul", [("half", (2048, 2048)), ("half", (2048, 2048))],
+                         "naive;tile=128,128,64;mapToThreads=64,8;mapToBlocks=256,256;useMfma=1;useSharedMemory=1;"
+                         "prefetchShared=1", 2048),
+})
+
 # The other sizes the reference's benchmark programs run their tuned options at
 # (group_convolution.cc:104-160, moments.cc:162-303, group_normalization.cc:120-180), same layout.
 OTHER_REFERENCE_SIZES = {
@@ -419,6 +444,8 @@ def _draw(rng, spec):
             return rng.integers(spec[2], spec[3], size=spec[1]).astype(np.int32)
         if kind == "scalar":
             return np.array(spec[1], dtype=np.float32)
+        if kind == "half":
+            return rng.standard_normal(spec[1], dtype=np.float32).astype(np.float16)
         if kind == "positive":
             return (rng.random(spec[1], dtype=np.float32) + 0.5).astype(np.float32)
         raise ValueError(kind)

@@ -133,3 +133,23 @@ def test_tuned_options_compile_at_the_reference_sizes(name):
     for k in range(ex.num_kernels):
         grid, block = ex.launch_bounds(k)
         assert 1 <= block[0] * block[1] * block[2] <= 1024 and min(grid) >= 1
+
+
+def test_oracle_products_of_converted_halves_are_float_products():
+    """`float(A) * float(B)` over float16 operands: the oracle's result is the float matrix product
+    of the converted matrices - exactly on small integers, within a float sum on deviates (the
+    closed form the GPU test uses at sizes where the oracle's element-wise evaluation takes minutes)."""
+    rng = np.random.Generator(np.random.Philox(5))
+    for name, transposed in (("half_matmul", False), ("half_tmm", True)):
+        src, entry, _, k = B.CASES[name]
+        shapes = [spec[1] for spec in B.CASES[name][2]]
+        ints = [rng.integers(-4, 5, size=s).astype(np.float16) for s in shapes]
+        (got,) = tc_oracle.run(src, entry, ints)
+        a, b = (x.astype(np.float32) for x in ints)
+        assert got.dtype == np.float32 and np.array_equal(got, a @ (b.T if transposed else b))
+        deviates = B.make_inputs(name)
+        assert all(x.dtype == np.float16 for x in deviates)
+        (got,) = tc_oracle.run(src, entry, deviates)
+        a, b = (x.astype(np.float64) for x in deviates)
+        exact = a @ (b.T if transposed else b)
+        assert np.abs(got - exact).max() <= 1e-6 * np.sqrt(k) * np.abs(exact).max()

@@ -88,7 +88,14 @@ def test_parity_of_the_large_contractions_and_the_other_reference_sizes(name):
     src, entry, _, _ = B.CASES[case]
     print(f"case {name}", flush=True)
     ins_np = B.make_large_inputs(name)
-    ref = tc_oracle.run(src, entry, ins_np)
+    if name.startswith("half_"):
+        # (the oracle evaluates a converted operand element by element: minutes at these sizes.  The
+        # small cases of these two comprehensions pin it to this closed form, the float product of
+        # the converted matrices.)
+        a, b = (x.astype(np.float32) for x in ins_np)
+        ref = [a @ (b.T if case == "half_tmm" else b)]
+    else:
+        ref = tc_oracle.run(src, entry, ins_np)
     ins = [torch.from_numpy(a).cuda() for a in ins_np]
     ex = tc.compile(src, entry, ins, options)
     outs = tc.prepare_outputs(src, entry, ins)
